@@ -1,0 +1,146 @@
+/*
+ * splat_hip.h -- C ABI of libsplat_hip.so: SPLAT's ACSR sparse-attention forward path as
+ * hand-written gfx950 (MI355X) HIP kernels.
+ *
+ * The reference (spikerheado1234/triton-fun, directory SPLAT/) has no FFI: its operator API is a
+ * set of Python functions that launch Triton kernels.  Each entry point below replaces the device
+ * work behind one of them and is what a ctypes / cffi stub in those Python functions binds:
+ *
+ *   splat_acsr_build      <- acsr_helpers.py:99-160   instantiate_metadata + create_acsr
+ *   splat_mask_generate   <- acsr_helpers.py:18-55    create_*_mask (device-side equivalent)
+ *   splat_sddmm           <- r_sddmm.py:15-115,171-184   rsddmm_kernel / rsddmm_launcher
+ *   splat_softmax         <- r_softmax.py:16-59,126-150  r_softmax_1d_kernel / rsoftmax_launcher
+ *   splat_spmm            <- r_spmm.py:13-126,148-164    r_spmm_kernel_row_maj_row_comp / rspmm_launcher
+ *   splat_attention_fwd   <- r_attention.py:77-100    RegularAttention.forward (the three launches fused)
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer unless its comment says "host".
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls only enqueue
+ *     work; they never synchronise, never allocate or free device memory and never throw.
+ *   - Return value: 0 on success; negative SPLAT_E_* for rejected arguments (nothing was
+ *     launched); positive = the hipError_t reported by the launch.  splat_last_error() returns a
+ *     thread-local, human readable description of the last non-zero return on this thread.
+ *   - All metadata arrays are float32, exactly as acsr_helpers.py:148-156 stores them.
+ *   - Compressed layout (r_sddmm.py:57-115, acsr_helpers.py:122-124): slot s of row r holds dense
+ *     column c = sTod_lin[r] * (s + sTod_trans[r]); slots s >= nnz[r] are never written and never
+ *     read.  A row's compressed slots may be the concatenation of several affine segments; segment
+ *     k owns slots [slot_offset_k, slot_offset_k + nnz_k[r]).
+ */
+#ifndef SPLAT_HIP_H
+#define SPLAT_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SPLAT_VERSION 100 /* major*10000 + minor*100 + patch */
+
+/* element types of q/k/v/score/output buffers */
+#define SPLAT_F32 0
+#define SPLAT_F16 1
+#define SPLAT_BF16 2
+
+/* negative return codes */
+#define SPLAT_E_NULL (-1)        /* a required pointer is NULL */
+#define SPLAT_E_SHAPE (-2)       /* a size is non-positive or out of the supported range */
+#define SPLAT_E_DTYPE (-3)       /* unknown element type */
+#define SPLAT_E_ALIGN (-4)       /* a pointer or stride is not aligned as the kernel requires */
+#define SPLAT_E_UNSUPPORTED (-5) /* valid request that this build has no kernel for */
+
+#define SPLAT_MAX_SEGMENTS 4
+
+/* mask patterns for splat_mask_generate */
+#define SPLAT_MASK_BLOCKED 0         /* acsr_helpers.py:18-34, p0 = p */
+#define SPLAT_MASK_WINDOWED 1        /* acsr_helpers.py:36-44, p0 = p */
+#define SPLAT_MASK_CAUSAL_WINDOWED 2 /* acsr_helpers.py:46-55, p0 = p */
+#define SPLAT_MASK_DILATED 3         /* columns i - p0*p1/2 + p1*t, t in [0,p0): p0 = window, p1 = dilation */
+#define SPLAT_MASK_STRIDED_LOCAL 4   /* columns (i-p0, i]: p0 = local width */
+#define SPLAT_MASK_STRIDED_FAR 5     /* columns j <= i-p0 with j % p1 == p1-1: p0 = local width, p1 = stride */
+
+/* One affine segment of an ACSR: the five per-row arrays create_acsr returns
+ * (acsr_helpers.py:148-152) plus where the segment's slots start in a compressed row. */
+typedef struct splat_acsr_seg {
+    const float* dTos_lin;   /* [rows] dense->sparse linear term, 1/(b-a)            */
+    const float* dTos_trans; /* [rows] dense->sparse translation, -a/(b-a)           */
+    const float* sTod_lin;   /* [rows] sparse->dense linear term, b-a                */
+    const float* sTod_trans; /* [rows] sparse->dense translation, a/(b-a)            */
+    const float* nnz;        /* [rows] live slots of the row                          */
+    const int32_t* first_col; /* [rows] optional (may be NULL): first live dense column of the
+                                 row.  Used for rows with exactly one live column, whose stored
+                                 translation acsr_helpers.py:126-130 hard-codes to 0.   */
+    int32_t slot_offset;     /* first compressed slot of this segment (0 for one segment) */
+    int32_t reserved;
+} splat_acsr_seg;
+
+int splat_version(void);
+const char* splat_last_error(void);
+
+/* Build the ACSR of a rows x cols 0/1 byte mask (row pitch `ld` bytes).
+ * Replaces instantiate_metadata/create_acsr, acsr_helpers.py:99-160; the float32 arrays are
+ * bit-identical to what that code stores.
+ *   dTos_lin..nnz      [rows]  float32 outputs
+ *   span_start/end     [ceil(rows/block_height)] float32 outputs (acsr_helpers.py:135-140)
+ *   row_first/row_last [rows]  int32 outputs, optional (NULL to skip): first / last nonzero
+ *                      column (cols / -1 for an empty row); the tiling of r_sddmm.py:117-146 and
+ *                      splat_acsr_seg.first_col are derived from them
+ *   summary            [8] int32 output: [0] T = max row sum (acsr_helpers.py:153), [1] number of
+ *                      rows that trip the reference's "Incorrect unpacking of affine-indices."
+ *                      assertion (nnz > 1 but fewer than two entries equal to 1), [2..7] reserved.
+ * Reads rows*ld bytes once; the caller reads `summary` back after synchronising the stream. */
+int splat_acsr_build(const uint8_t* mask, int64_t rows, int64_t cols, int64_t ld,
+                     int32_t block_height, float* dTos_lin, float* dTos_trans, float* sTod_lin,
+                     float* sTod_trans, float* nnz, float* span_start, float* span_end,
+                     int32_t* row_first, int32_t* row_last, int32_t* summary, void* stream);
+
+/* Fill a rows x cols byte mask (row pitch ld) with one of the SPLAT_MASK_* patterns.
+ * Device-side equivalent of the O(s^2) Python loops at acsr_helpers.py:18-55. */
+int splat_mask_generate(uint8_t* mask, int64_t rows, int64_t cols, int64_t ld, int32_t pattern,
+                        int64_t p0, int64_t p1, void* stream);
+
+/* SDDMM: out[b,h,r,off+s] = scale * sum_k q[b,h,r,k] * kT[b,h,k,c(r,s)], s < nnz[r], per segment.
+ * Replaces rsddmm_launcher / rsddmm_kernel, r_sddmm.py:15-115,171-184 (x = q, y = kT).
+ *   q    element (b,h,r,k) at q   + b*q_sb + h*q_sh + r*q_sl + k            (unit stride in k)
+ *   kT   element (b,h,k,c) at kT  + b*k_sb + h*k_sh + k*k_sd + c*k_sl       (k_sd==1 or k_sl==1)
+ *   out  [B,H,L,T] contiguous, dtype `out_dtype`; q and kT have dtype `in_dtype`
+ * Strides are in elements. */
+int splat_sddmm(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT,
+                int64_t k_sb, int64_t k_sh, int64_t k_sd, int64_t k_sl, void* out,
+                const splat_acsr_seg* segs /* host */, int32_t n_seg, int32_t B, int32_t H,
+                int32_t L, int32_t n_keys, int32_t d, int32_t T, float scale, int32_t in_dtype,
+                int32_t out_dtype, void* stream);
+
+/* Row softmax over the live slots of compressed rows: y[bh,r,s] = exp(x[bh,r,s]-max_r)/sum_r.
+ * Replaces rsoftmax_launcher / r_softmax_1d_kernel, r_softmax.py:16-59,126-150, applied to every
+ * row.  x, y: [BH, L, T] contiguous; x may equal y (in place). */
+int splat_softmax(const void* x, void* y, const splat_acsr_seg* segs /* host */, int32_t n_seg,
+                  int64_t BH, int32_t L, int32_t T, int32_t in_dtype, int32_t out_dtype,
+                  void* stream);
+
+/* SpMM: out[b,h,r,:] = sum_{s<nnz[r]} p[b,h,r,off+s] * v[b,h,c(r,s),:], summed over segments.
+ * Replaces rspmm_launcher / r_spmm_kernel_row_maj_row_comp, r_spmm.py:13-126,148-164.
+ *   p    [B,H,L,T] contiguous compressed probabilities, dtype in_dtype
+ *   v    element (b,h,c,n) at v + b*v_sb + h*v_sh + c*v_sl + n, dtype in_dtype
+ *   out  [B,H,L,n_out] contiguous, dtype out_dtype */
+int splat_spmm(const void* p, const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sl, void* out,
+               const splat_acsr_seg* segs /* host */, int32_t n_seg, int32_t B, int32_t H,
+               int32_t L, int32_t n_keys, int32_t n_out, int32_t T, int32_t in_dtype,
+               int32_t out_dtype, void* stream);
+
+/* Fused forward: out = softmax_over_live_columns(scale * q.kT) . v with online softmax; the
+ * compressed score matrix is never written to memory.  Equals the composition
+ * rsddmm_launcher -> rsoftmax_launcher -> rspmm_launcher of RegularAttention.forward
+ * (r_attention.py:77-100).  d must be 64 or 128.  q, kT, v, out share `dtype`; layouts as in
+ * splat_sddmm / splat_spmm, out element (b,h,r,n) at out + b*o_sb + h*o_sh + r*o_sl + n. */
+int splat_attention_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT,
+                        int64_t k_sb, int64_t k_sh, int64_t k_sd, int64_t k_sl, const void* v,
+                        int64_t v_sb, int64_t v_sh, int64_t v_sl, void* out, int64_t o_sb,
+                        int64_t o_sh, int64_t o_sl, const splat_acsr_seg* segs /* host */,
+                        int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t d, float scale,
+                        int32_t dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPLAT_HIP_H */

@@ -1,0 +1,73 @@
+"""No-GPU checks of the product: the C-ABI library loads and exports every symbol the header declares,
+rejects bad arguments before touching the device, and the Python operator layer refuses to run
+without a HIP device (there is no host fallback)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import _splat_hip as hip
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "splat_hip.h")
+
+
+def header_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(splat_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    syms = header_symbols()
+    assert {"splat_acsr_build", "splat_mask_generate", "splat_sddmm", "splat_softmax", "splat_spmm",
+            "splat_attention_fwd", "splat_version", "splat_last_error"} <= set(syms)
+    handle = ctypes.CDLL(hip.LIB_PATH)
+    for s in syms:
+        assert hasattr(handle, s), s
+    assert sorted(hip.EXPORTS) == syms
+
+
+def test_version_matches_header():
+    want = int(re.search(r"#define SPLAT_VERSION (\d+)", open(HEADER).read()).group(1))
+    assert hip.lib().splat_version() == want
+
+
+def test_null_and_shape_arguments_are_rejected_without_a_device():
+    lib = hip.lib()
+    assert lib.splat_softmax(None, None, None, 1, 1, 1, 1, 0, 0, None) == -1
+    assert b"null" in lib.splat_last_error()
+    seg = (hip.AcsrSeg * 1)()
+    assert lib.splat_softmax(8, 8, seg, 0, 1, 1, 1, 0, 0, None) == -2          # n_seg = 0
+    assert lib.splat_softmax(8, 8, seg, 1, 1, 1, 0, 0, 0, None) == -2          # T = 0
+    assert lib.splat_acsr_build(None, 4, 4, 4, 2, *([None] * 10), None) == -1
+    assert lib.splat_acsr_build(8, 4, 4, 2, 2, *([8] * 7), None, None, 8, None) == -2  # ld < cols
+    assert lib.splat_mask_generate(8, 4, 4, 4, 99, 1, 1, None) == -5
+    assert lib.splat_attention_fwd(8, 0, 0, 64, 8, 0, 0, 1, 64, 8, 0, 0, 64, 8, 0, 0, 64, seg, 1, 1, 1, 16, 48, 1.0, 2,
+                                   None) == -5                                   # d = 48 unsupported
+    assert b"64 or 128" in lib.splat_last_error()
+    assert lib.splat_sddmm(8, 0, 0, 8, 8, 0, 0, 3, 5, 8, seg, 1, 1, 1, 4, 4, 8, 4, 1.0, 0, 0, None) == -4  # no unit stride
+    assert lib.splat_spmm(8, 8, 0, 0, 8, 8, seg, 1, 1, 1, 4, 4, 8, 4, 7, 0, None) == -3                    # bad dtype
+
+
+def test_operators_refuse_the_host():
+    import acsr_helpers as A
+    import r_attention
+    with pytest.raises(hip.SplatError):
+        A.create_acsr(A.create_blocked_mask(10, 2), 2, "cpu")
+    with pytest.raises(hip.SplatError):
+        r_attention.RegularAttention(1, 16, 1, 64, A.create_causal_windowed_mask(16, 3), 16, 16, "cpu", torch.float32)
+    if not torch.cuda.is_available():
+        with pytest.raises(hip.SplatError):
+            A.create_acsr(A.create_blocked_mask(10, 2), 2, 0)
+
+
+def test_product_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "triton-fun_amd")
+    for base, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".cpp", ".h")):
+                text = open(os.path.join(base, f)).read()
+                assert "oracle" not in text, os.path.join(base, f)

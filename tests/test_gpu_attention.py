@@ -1,0 +1,156 @@
+"""Fused forward and the three-kernel composition against fp32 dense masked attention (the oracle), at
+BASELINE's configurations: small ones whole, large ones through a head subset plus size-independent
+properties at full size."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import splat_oracle as O
+import acsr_helpers as A
+from r_attention import RegularAttention, attention_launcher, unit
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.float16: 1e-2, torch.bfloat16: 2e-2}
+
+
+def run_module(mask, B, H, L, d, dtype, dev, q, k, v, scale, fused, contig_kT=False):
+    attn = RegularAttention(B, L, H, d, mask, 16, 16, dev, dtype, scale=scale, fused=fused)
+    kT = k.to(dev).transpose(2, 3)
+    if contig_kT:
+        kT = kT.contiguous()
+    out = attn([q.to(dev), kT, v.to(dev)])
+    assert out is attn.rspmm_output
+    return out.float().cpu()
+
+
+def test_config1_fp32_whole(dev):
+    """B=1, H=1, L=512, d=64, fp32, causal window 64, scale 1/sqrt(d)."""
+    L, d = 512, 64
+    mask = A.create_causal_windowed_mask(L, 63)  # list of lists, the reference's argument type
+    q, k, v = O.make_inputs(1001, 1, 1, L, d, torch.float32)
+    want = O.dense_masked_attention(q, k.transpose(2, 3), v, np.asarray(mask), d ** -0.5)
+    for fused in (True, False):
+        for contig in (False, True):
+            got = run_module(mask, 1, 1, L, d, torch.float32, dev, q, k, v, d ** -0.5, fused, contig)
+            assert float((got - want).abs().max()) <= TOL[torch.float32], (fused, contig)
+
+
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("contig", [False, True])
+def test_config2_fp16(dev, fused, contig):
+    """B=4, H=16, L=4096, d=64, fp16, causal window 256, inputs * 0.5: run whole on the GPU, checked on the
+    first and last (batch, head) pairs."""
+    B, H, L, d = 4, 16, 4096, 64
+    q, k, v = O.make_inputs(1002, B, H, L, d, torch.float16, mul=0.5)
+    mask = A.causal_windowed_pattern(L, 255)
+    got = run_module(mask, B, H, L, d, torch.float16, dev, q, k, v, d ** -0.5, fused, contig)
+    m = O.create_causal_windowed_mask(L, 255)
+    for b, h in ((0, 0), (3, 15)):
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        want = O.dense_masked_attention_chunked(q[sl], k[sl].transpose(2, 3), v[sl], lambda a, c: m[a:c] != 0, d ** -0.5)
+        assert float((got[sl] - want).abs().max()) <= TOL[torch.float16]
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_config3_strided_two_segments(dev, fused):
+    """B=2, H=16, L=8192, d=64, bf16, local 128 + every 128th column: two affine segments per row.  Run at
+    H=2 (the per-head work is what scales), checked whole."""
+    B, H, L, d = 1, 2, 8192, 64
+    q, k, v = O.make_inputs(1003, B, H, L, d, torch.bfloat16)
+    got = run_module(A.strided_patterns(L, 128, 128), B, H, L, d, torch.bfloat16, dev, q, k, v, d ** -0.5, fused)
+    segs = O.create_strided_segment_masks(L, 128, 128)
+    union = segs[0] | segs[1]
+    want = O.dense_masked_attention_chunked(q, k.transpose(2, 3), v, lambda a, c: union[a:c] != 0, d ** -0.5)
+    assert float((got - want).abs().max()) <= TOL[torch.bfloat16]
+
+
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("contig", [False, True])
+def test_config4_dilated(dev, fused, contig):
+    """B=2, H=32, L=8192, d=128, bf16, 512 keys centred on i with dilation 2.  Run at B=1, H=2."""
+    B, H, L, d = 1, 2, 8192, 128
+    q, k, v = O.make_inputs(1004, B, H, L, d, torch.bfloat16)
+    got = run_module(A.dilated_pattern(L, 512, 2), B, H, L, d, torch.bfloat16, dev, q, k, v, d ** -0.5, fused, contig)
+    m = O.create_dilated_mask(L, 512, 2)
+    want = O.dense_masked_attention_chunked(q, k.transpose(2, 3), v, lambda a, c: m[a:c] != 0, d ** -0.5)
+    assert float((got - want).abs().max()) <= TOL[torch.bfloat16]
+
+
+def test_config5_headline_full_size(dev):
+    """B=4, H=16, L=16384, d=128, bf16, causal window 512, fused only: the full problem runs on the GPU;
+    two (batch, head) pairs are checked against the oracle, the rest through properties that do not depend on
+    size: V = 1 gives 1 (the weights of a row sum to one), and the output is linear in V."""
+    B, H, L, d = 4, 16, 16384, 128
+    scale = d ** -0.5
+    q, k, v = O.make_inputs(1005, B, H, L, d, torch.bfloat16)
+    attn = RegularAttention(B, L, H, d, A.causal_windowed_pattern(L, 511), 16, 16, dev, torch.bfloat16, scale=scale)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    for contig in (False, True):
+        kT = kd.transpose(2, 3).contiguous() if contig else kd.transpose(2, 3)
+        got = attn([qd, kT, vd]).float().cpu()
+        m_rows = lambda a, c: ((np.arange(a, c)[:, None] >= np.arange(L)[None, :]) &
+                               (np.arange(a, c)[:, None] - 511 <= np.arange(L)[None, :]))
+        for b, h in ((0, 0), (3, 15)):
+            sl = (slice(b, b + 1), slice(h, h + 1))
+            want = O.dense_masked_attention_chunked(q[sl], k[sl].transpose(2, 3), v[sl], m_rows, scale)
+            assert float((got[sl] - want).abs().max()) <= TOL[torch.bfloat16], (contig, b, h)
+        assert torch.isfinite(got).all()
+    kT = kd.transpose(2, 3)
+    ones = attn([qd, kT, torch.ones_like(vd)]).float()
+    assert float((ones - 1).abs().max()) <= 2e-2
+    base = attn([qd, kT, vd]).float().clone()
+    v2 = torch.randn(B, H, L, d, generator=torch.Generator().manual_seed(7)).to(torch.bfloat16).to(dev)
+    o2 = attn([qd, kT, v2]).float().clone()
+    o12 = attn([qd, kT, (vd.float() + v2.float()).to(torch.bfloat16)]).float()
+    assert float((o12 - (base + o2)).abs().max()) <= 6e-2  # three bf16 roundings of O(1) values
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("make", [
+    lambda: O.create_blocked_mask(128, 57), lambda: O.create_windowed_mask(333, 40),
+    lambda: O.create_causal_windowed_mask(1000, 100), lambda: O.create_dilated_mask(520, 64, 3),
+    lambda: O.create_blocked_mask(1024, 328)])
+def test_fused_small_patterns(dev, dtype, d, make):
+    mask = make()
+    L = mask.shape[0]
+    if dtype != torch.float32 and L % 8:
+        contigs = (False,)  # K^T contiguous along keys needs 16-byte rows
+    elif dtype == torch.float32 and L % 4:
+        contigs = (False,)
+    else:
+        contigs = (False, True)
+    q, k, v = O.make_inputs(L + d, 2, 2, L, d, dtype)
+    want = O.dense_masked_attention(q, k.transpose(2, 3), v, mask, d ** -0.5)
+    for contig in contigs:
+        got = run_module(mask, 2, 2, L, d, dtype, dev, q, k, v, d ** -0.5, True, contig)
+        assert float((got - want).abs().max()) <= TOL[dtype], contig
+
+
+def test_empty_and_single_column_rows(dev):
+    L, d = 256, 64
+    mask = O.create_causal_windowed_mask(L, 31).copy()
+    mask[7] = 0          # empty row -> zero output
+    mask[100] = 0
+    mask[100, 40] = 1    # single live column that is not column 0
+    q, k, v = O.make_inputs(5, 1, 2, L, d, torch.float16)
+    want = O.dense_masked_attention(q, k.transpose(2, 3), v, mask, 0.125)
+    for fused in (True, False):
+        got = run_module(mask, 1, 2, L, d, torch.float16, dev, q, k, v, 0.125, fused)
+        assert float((got - want).abs().max()) <= TOL[torch.float16]
+        assert torch.all(got[:, :, 7] == 0)
+
+
+def test_unit_projection_wrapper(dev):
+    """r_attention.py:102-110: project then attend (reference smoke test shape scaled down), default scale 1."""
+    B, S, N, Hd = 2, 256, 4, 64
+    g = torch.Generator().manual_seed(9)
+    x = [torch.rand(B, S, N * Hd, generator=g) * 0.1 for _ in range(3)]
+    w = [torch.rand(N * Hd, N, Hd, generator=g) * 0.1 for _ in range(3)]
+    mask = A.create_windowed_mask(S, 32)
+    attn = RegularAttention(B, S, N, Hd, mask, 16, 16, dev, torch.float32)
+    got = unit(*[t.to(dev) for t in x], *[t.to(dev) for t in w], attn).cpu()
+    q, k, v = [torch.einsum("bsd,dnh->bnsh", a, b) for a, b in zip(x, w)]
+    want = O.dense_masked_attention(q, k.transpose(2, 3), v, np.asarray(mask), 1.0)
+    assert float((got - want).abs().max()) <= 1e-5

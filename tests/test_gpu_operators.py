@@ -1,0 +1,165 @@
+"""SDDMM, softmax and SpMM HIP kernels against the oracle on identical seeded inputs."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import splat_oracle as O
+import acsr_helpers as A
+import r_sddmm
+import r_softmax
+import r_spmm
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.float16: 1e-2, torch.bfloat16: 2e-2}
+SENTINEL = 777.0
+
+
+def acsr_pair(mask, BH, dev):
+    return A.create_acsr(mask, BH, dev), O.create_acsr(np.asarray(mask), BH)
+
+
+def live(acsr_np):
+    return torch.from_numpy(O.slot_columns(acsr_np)[1])
+
+
+REF_SMALL = [(10, 2), (10, 5), (10, 7), (16, 5), (16, 16), (32, 10), (32, 20), (32, 32), (128, 57)]
+
+
+# ---------------------------------------------------------------- SDDMM
+@pytest.mark.parametrize("n,p", REF_SMALL)
+def test_sddmm_reference_cases(dev, n, p):
+    """r_sddmm.py:224-256 with its masks: m = k = n, B = H = 2, 16x16 blocks, integer-valued inputs, the
+    reference's acceptance rule |out[r, s] - truth[r, c(r, s)]| <= 1e-3 on live slots (exact here: integer
+    products below 2^24 summed in fp32)."""
+    mask = A.create_blocked_mask(n, p)
+    g = torch.Generator().manual_seed(n * 100 + p)
+    left = torch.randint(0, 100, (2, 2, n, n), generator=g).float()
+    right = torch.randint(0, 100, (2, 2, n, n), generator=g).float()
+    acsr, acsr_np = acsr_pair(mask, 16, dev)
+    out, grid, tx, ty = r_sddmm.rsddmm_preamble(mask, (2, 2, n, acsr[5]), 16, 16, dev, torch.float32)
+    out.fill_(SENTINEL)
+    res = r_sddmm.rsddmm_launcher(left.to(dev), right.to(dev), out, acsr[0], acsr[1], acsr[2], acsr[3], acsr[5], acsr[4],
+                                  grid, tx, ty, 16, 16)
+    assert res[0] is out and res[1] is acsr[2] and res[2] is acsr[3] and res[3] is acsr[4]
+    want = O.sddmm(left, right, acsr_np)
+    lv = live(acsr_np)
+    got = out.cpu()
+    assert torch.all(torch.abs(got - want)[..., lv] <= 1e-3)
+    assert torch.all(got[..., ~lv] == SENTINEL), "dead slots must not be written"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("layout", ["view", "contig"])
+@pytest.mark.parametrize("make,d", [
+    (lambda: O.create_causal_windowed_mask(512, 63), 64), (lambda: O.create_windowed_mask(300, 20), 40),
+    (lambda: O.create_dilated_mask(256, 32, 2), 128), (lambda: O.create_blocked_mask(200, 33), 200),
+    (lambda: O.create_causal_windowed_mask(130, 9), 10)])
+def test_sddmm_patterns(dev, dtype, layout, make, d):
+    mask = make()
+    L = mask.shape[0]
+    q, k, _ = O.make_inputs(11, 2, 3, L, d, dtype)
+    kT = k.transpose(2, 3)
+    acsr, acsr_np = acsr_pair(mask, 16, dev)
+    scale = d ** -0.5
+    want = O.sddmm(q, kT, acsr_np, scale)
+    kT_dev = k.to(dev).transpose(2, 3)
+    if layout == "contig":
+        kT_dev = kT_dev.contiguous()
+    out = torch.full((2, 3, L, acsr[5]), SENTINEL, dtype=dtype, device=dev)
+    r_sddmm.rsddmm_launcher(q.to(dev), kT_dev, out, acsr[0], acsr[1], acsr[2], acsr[3], acsr[5], acsr[4], (1, 1),
+                            None, None, 16, 16, scale=scale)
+    got = out.float().cpu()
+    lv = live(acsr_np)
+    tol = TOL[dtype] * max(1.0, float(want.abs().max()))
+    assert float((got - want)[..., lv].abs().max()) <= tol
+    assert torch.all(got[..., ~lv] == SENTINEL)
+
+
+# ---------------------------------------------------------------- softmax
+@pytest.mark.parametrize("n,p", REF_SMALL)
+def test_softmax_reference_cases(dev, n, p):
+    """r_softmax.py:188-224 with its masks: fp32 integer-valued input, bf16 output; live slots of every
+    row sum to 1 +- 1e-2 (the reference's rule) and match the oracle's values."""
+    mask = A.create_blocked_mask(n, p)
+    acsr, acsr_np = acsr_pair(mask, 16, dev)
+    grid, out, full, pow2 = r_softmax.rsoftmax_preamble(mask, (2, 2, n, acsr[5]), 16, dev, torch.bfloat16)
+    g = torch.Generator().manual_seed(n + p)
+    inp = torch.randint(0, 100, full, generator=g).float()
+    out.fill_(SENTINEL)
+    res = r_softmax.rsoftmax_launcher(inp.to(dev), out, acsr[0], acsr[1], acsr[2], acsr[3], acsr[5], pow2, acsr[4], grid, 16)
+    assert res[0] is out
+    lv = live(acsr_np)
+    got = out.float().cpu()
+    sums = torch.where(lv, got, torch.zeros(())).sum(-1)
+    assert torch.all(torch.abs(sums - 1) < 1e-2)
+    want = O.softmax_compressed(inp, lv)
+    assert float((got - want)[..., lv].abs().max()) <= TOL[torch.bfloat16]
+    assert torch.all(got[..., ~lv] == SENTINEL)
+
+
+@pytest.mark.parametrize("in_dt,out_dt", [(torch.float32, torch.float32), (torch.float16, torch.float16),
+                                          (torch.bfloat16, torch.bfloat16), (torch.float32, torch.float16)])
+@pytest.mark.parametrize("make", [lambda: O.create_causal_windowed_mask(512, 255), lambda: O.create_windowed_mask(200, 50),
+                                  lambda: O.create_dilated_mask(700, 512, 2), lambda: O.create_blocked_mask(3000, 1300)])
+def test_softmax_patterns(dev, in_dt, out_dt, make):
+    mask = make()
+    L = mask.shape[0]
+    acsr, acsr_np = acsr_pair(mask, 16, dev)
+    T = acsr[5]
+    g = torch.Generator().manual_seed(T)
+    x = (torch.randn(2, 2, L, T, generator=g) * 3).to(in_dt)
+    lv = live(acsr_np)
+    want = O.softmax_compressed(x.float(), lv)
+    out = torch.full((2, 2, L, T), SENTINEL, dtype=out_dt, device=dev)
+    r_softmax.rsoftmax_launcher(x.to(dev), out, acsr[0], acsr[1], acsr[2], acsr[3], T, O.rsoftmax_pow2(T), acsr[4], (1, 1), 16)
+    got = out.float().cpu()
+    assert float((got - want)[..., lv].abs().max()) <= TOL[out_dt]
+    assert torch.all(got[..., ~lv] == SENTINEL)
+    # in place
+    xd = x.to(dev)
+    if in_dt == out_dt:
+        r_softmax.rsoftmax_launcher(xd, xd, acsr[0], acsr[1], acsr[2], acsr[3], T, O.rsoftmax_pow2(T), acsr[4], (1, 1), 16)
+        assert float((xd.float().cpu() - want)[..., lv].abs().max()) <= TOL[out_dt]
+
+
+# ---------------------------------------------------------------- SpMM
+@pytest.mark.parametrize("n,p", REF_SMALL)
+def test_spmm_reference_cases(dev, n, p):
+    """r_spmm.py:219-261 with its masks: fp32 integer-valued P [.., n, T] and V [.., n, n], every output element
+    within 1e-3 of the dot product over live slots (exact here)."""
+    mask = A.create_blocked_mask(n, p)
+    acsr, acsr_np = acsr_pair(mask, 16, dev)
+    g = torch.Generator().manual_seed(n * 7 + p)
+    left = torch.randint(0, 100, (2, 2, n, acsr[5]), generator=g).float()
+    right = torch.randint(0, 100, (2, 2, n, n), generator=g).float()
+    out, grid, T = r_spmm.rspmm_preamble(mask, (2, 2, n, n), 16, 16, dev, torch.float32)
+    assert T == acsr[5]
+    res = r_spmm.rspmm_launcher(left.to(dev), right.to(dev), out, acsr[0], acsr[1], acsr[2], acsr[3], acsr[6], acsr[7], T,
+                                acsr[4], grid, 16, 16)
+    assert res[0] is out
+    want = O.spmm(left, right, acsr_np)
+    assert float((out.cpu() - want).abs().max()) <= 1e-3 * max(1.0, float(want.abs().max()) * 1e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("make,n_out", [
+    (lambda: O.create_causal_windowed_mask(512, 63), 64), (lambda: O.create_windowed_mask(300, 20), 40),
+    (lambda: O.create_dilated_mask(256, 32, 2), 128), (lambda: O.create_blocked_mask(200, 33), 200),
+    (lambda: O.create_causal_windowed_mask(130, 9), 10)])
+def test_spmm_patterns(dev, dtype, make, n_out):
+    mask = make()
+    L = mask.shape[0]
+    acsr, acsr_np = acsr_pair(mask, 16, dev)
+    T = acsr[5]
+    g = torch.Generator().manual_seed(T + n_out)
+    lv = live(acsr_np)
+    p = torch.rand(2, 3, L, T, generator=g)
+    p = (p / torch.where(lv, p, torch.zeros(())).sum(-1, keepdim=True)).to(dtype)
+    p = torch.where(lv, p, torch.full((), float("nan"), dtype=dtype))  # dead slots hold garbage
+    v = torch.randn(2, 3, L, n_out, generator=g).to(dtype)
+    want = O.spmm(torch.nan_to_num(p.float()), v, acsr_np)
+    out = torch.empty(2, 3, L, n_out, dtype=dtype, device=dev)
+    r_spmm.rspmm_launcher(p.to(dev), v.to(dev), out, acsr[0], acsr[1], acsr[2], acsr[3], acsr[6], acsr[7], T, acsr[4],
+                          (1, 1, 1), 16, 16)
+    assert float((out.float().cpu() - want).abs().max()) <= TOL[dtype]

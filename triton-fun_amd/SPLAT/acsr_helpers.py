@@ -1,0 +1,302 @@
+"""ACSR (affine-compressed sparse row) metadata for SPLAT's regular sparse kernels, built on the GPU.
+
+Mirrors the interface of the reference's ``SPLAT/acsr_helpers.py`` (mask generators :18-55, ACSR
+containers :58-96, ``instantiate_metadata`` :99-142, ``create_acsr`` :145-160): same names, same
+positional arguments, same return tuples, every metadata tensor float32.  The O(L^2) Python passes of
+the reference are replaced by one streaming HIP kernel over a byte mask (``splat_acsr_build``).
+
+Additions that keep the reference behaviour as the default:
+  * masks may also be numpy arrays, torch tensors (host or device) or :class:`MaskPattern` descriptors
+    that are rasterised on the device, so L = 16384 never needs a Python list of lists;
+  * ``create_acsr_segments`` builds several disjoint affine segments per row (e.g. a local window plus
+    a strided far field), which one affine map per row cannot express.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from math import ceil
+from typing import Any, Sequence, Type
+
+import numpy as np
+import torch
+
+import _splat_hip as _hip
+
+# ---------------------------------------------------------------------------------------------
+# Mask generators (s = sequence length, p = sparsity parameter); list-of-lists like the reference.
+# ---------------------------------------------------------------------------------------------
+
+
+def _row(s: int, lo: int, hi: int) -> list[int]:
+    lo, hi = max(lo, 0), min(hi, s)
+    if hi <= lo:
+        return [0] * s
+    return [0] * lo + [1] * (hi - lo) + [0] * (s - hi)
+
+
+def create_blocked_mask(s: int, p: int, device: Any = None):
+    """Rows of the first block see columns [0, p); row i of a later block sees the previous block and
+    its own: [(i//p - 1)*p, (i//p + 1)*p).  With ``device`` set, returns a uint8 tensor rasterised there."""
+    if device is not None:
+        return MaskPattern(_hip.MASK_BLOCKED, s, p).device_mask(device)
+    return [_row(s, 0, p) if i < p else _row(s, (i // p - 1) * p, (i // p + 1) * p) for i in range(s)]
+
+
+def create_windowed_mask(s: int, p: int, device: Any = None):
+    """|i - j| <= p."""
+    if device is not None:
+        return MaskPattern(_hip.MASK_WINDOWED, s, p).device_mask(device)
+    return [_row(s, i - p, i + p + 1) for i in range(s)]
+
+
+def create_causal_windowed_mask(s: int, p: int, device: Any = None):
+    """i - p <= j <= i."""
+    if device is not None:
+        return MaskPattern(_hip.MASK_CAUSAL_WINDOWED, s, p).device_mask(device)
+    return [_row(s, i - p, i + 1) for i in range(s)]
+
+
+@dataclass(frozen=True)
+class MaskPattern:
+    """A closed-form s x s mask that is rasterised on the device instead of in Python."""
+    kind: int
+    s: int
+    p0: int
+    p1: int = 1
+
+    def device_mask(self, device: Any) -> torch.Tensor:
+        dev = _hip.resolve_device(device)
+        out = torch.empty((self.s, self.s), dtype=torch.uint8, device=dev)
+        with torch.cuda.device(dev):
+            rc = _hip.lib().splat_mask_generate(out.data_ptr(), self.s, self.s, self.s, self.kind, self.p0, self.p1,
+                                                _hip.stream_ptr(dev))
+        _hip.check(rc, "splat_mask_generate")
+        return out
+
+
+def blocked_pattern(s: int, p: int) -> MaskPattern:
+    return MaskPattern(_hip.MASK_BLOCKED, s, p)
+
+
+def windowed_pattern(s: int, p: int) -> MaskPattern:
+    return MaskPattern(_hip.MASK_WINDOWED, s, p)
+
+
+def causal_windowed_pattern(s: int, p: int) -> MaskPattern:
+    return MaskPattern(_hip.MASK_CAUSAL_WINDOWED, s, p)
+
+
+def dilated_pattern(s: int, window: int, dilation: int) -> MaskPattern:
+    """Row i sees columns i - window*dilation//2 + dilation*t, t in [0, window), clipped to [0, s)."""
+    return MaskPattern(_hip.MASK_DILATED, s, window, dilation)
+
+
+def strided_patterns(s: int, local: int, stride: int) -> list[MaskPattern]:
+    """Sparse-Transformer style rows as two disjoint affine segments: the local causal window
+    (i - local, i] and the far columns j <= i - local with j % stride == stride - 1."""
+    return [MaskPattern(_hip.MASK_STRIDED_LOCAL, s, local), MaskPattern(_hip.MASK_STRIDED_FAR, s, local, stride)]
+
+
+# ---------------------------------------------------------------------------------------------
+# Host containers, as in the reference.
+# ---------------------------------------------------------------------------------------------
+
+
+@dataclass
+class AffineIndices:
+    """Dense -> sparse map of one row: slot = linear_transformation * column + translation."""
+    linear_transformation: float
+    translation: int
+    nnz: int
+
+
+@dataclass
+class AffineIndicesInt:
+    """Sparse -> dense map of one row: column = linear_transformation * (slot + translation)."""
+    linear_transformation: int
+    translation: int
+    nnz: int
+
+
+class ACSR:
+    def __init__(self, affine_indices: list[Type[AffineIndices]], affine_indices_int: list[Type[AffineIndicesInt]],
+                 span_specialised_loop_idxs: list[tuple[int]]):
+        self.affine_indices = affine_indices
+        self.affine_indices_int = affine_indices_int
+        self.span_specialised_loop_idxs = span_specialised_loop_idxs
+
+    def get_dTos_linear_transformations(self) -> list[float]:
+        return [x.linear_transformation for x in self.affine_indices]
+
+    def get_sTod_linear_transformations(self) -> list[int]:
+        return [x.linear_transformation for x in self.affine_indices_int]
+
+    def get_dTos_translations(self) -> list[float]:
+        return [x.translation for x in self.affine_indices]
+
+    def get_sTod_translations(self) -> list[int]:
+        return [x.translation for x in self.affine_indices_int]
+
+    def get_nnzs(self) -> list[float]:
+        return [x.nnz for x in self.affine_indices]
+
+    def get_span_specialised_data(self) -> list[tuple[int]]:
+        return self.span_specialised_loop_idxs
+
+
+# ---------------------------------------------------------------------------------------------
+# Device masks and the GPU builder.
+# ---------------------------------------------------------------------------------------------
+
+
+class _MaskEntry:
+    __slots__ = ("key_obj", "mask", "builds")
+
+    def __init__(self, key_obj, mask):
+        self.key_obj = key_obj  # keeps the caller's object alive so that its id() stays unique
+        self.mask = mask
+        self.builds = {}
+
+
+_MASK_CACHE: list[_MaskEntry] = []
+_MASK_CACHE_SIZE = 4
+
+
+def _cache_key(mask) -> tuple:
+    if isinstance(mask, torch.Tensor):
+        return ("t", mask.data_ptr(), mask._version, tuple(mask.shape), str(mask.device))
+    if isinstance(mask, MaskPattern):
+        return ("p", mask)
+    return ("o", id(mask))
+
+
+def _mask_entry(mask, dev: torch.device) -> _MaskEntry:
+    """The uint8 [rows, cols] device copy of ``mask`` (shared by create_acsr and the three preambles,
+    which the reference hands the same mask object)."""
+    key = (_cache_key(mask), str(dev))
+    for e in _MASK_CACHE:
+        if e.key_obj[0] == key:
+            return e
+    if isinstance(mask, MaskPattern):
+        dm = mask.device_mask(dev)
+    elif isinstance(mask, torch.Tensor):
+        dm = mask.to(device=dev, dtype=torch.uint8).contiguous()
+    else:
+        arr = np.asarray(mask)
+        if arr.ndim != 2:
+            raise ValueError("mask must be a 2-D 0/1 array")
+        if arr.size and (arr.min() < 0 or arr.max() > 255):
+            raise ValueError("mask entries must fit in a byte")
+        dm = torch.from_numpy(np.ascontiguousarray(arr, dtype=np.uint8)).to(dev)
+    if dm.dim() != 2:
+        raise ValueError("mask must be 2-D")
+    entry = _MaskEntry((key, mask), dm)
+    _MASK_CACHE.append(entry)
+    del _MASK_CACHE[:-_MASK_CACHE_SIZE]
+    return entry
+
+
+def mask_shape(mask) -> tuple[int, int]:
+    if isinstance(mask, MaskPattern):
+        return (mask.s, mask.s)
+    if isinstance(mask, torch.Tensor):
+        return tuple(mask.shape)
+    return (len(mask), len(mask[0]))
+
+
+class AcsrBuild:
+    """Everything one ``splat_acsr_build`` call produced for (mask, BLOCK_HEIGHT)."""
+    __slots__ = ("dTos_lin", "dTos_trans", "sTod_lin", "sTod_trans", "nnz", "T", "span_start", "span_end",
+                 "row_first", "row_last")
+
+
+def build_acsr(mask, BLOCK_HEIGHT: int, dev: torch.device) -> AcsrBuild:
+    entry = _mask_entry(mask, dev)
+    if BLOCK_HEIGHT in entry.builds:
+        return entry.builds[BLOCK_HEIGHT]
+    dm = entry.mask
+    rows, cols = dm.shape
+    n_blocks = ceil(rows / BLOCK_HEIGHT)
+    f32 = dict(dtype=torch.float32, device=dev)
+    b = AcsrBuild()
+    b.dTos_lin, b.dTos_trans = torch.empty(rows, **f32), torch.empty(rows, **f32)
+    b.sTod_lin, b.sTod_trans = torch.empty(rows, **f32), torch.empty(rows, **f32)
+    b.nnz = torch.empty(rows, **f32)
+    b.span_start, b.span_end = torch.empty(n_blocks, **f32), torch.empty(n_blocks, **f32)
+    b.row_first = torch.empty(rows, dtype=torch.int32, device=dev)
+    b.row_last = torch.empty(rows, dtype=torch.int32, device=dev)
+    summary = torch.empty(8, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _hip.lib().splat_acsr_build(dm.data_ptr(), rows, cols, dm.stride(0), BLOCK_HEIGHT, b.dTos_lin.data_ptr(),
+                                         b.dTos_trans.data_ptr(), b.sTod_lin.data_ptr(), b.sTod_trans.data_ptr(),
+                                         b.nnz.data_ptr(), b.span_start.data_ptr(), b.span_end.data_ptr(),
+                                         b.row_first.data_ptr(), b.row_last.data_ptr(), summary.data_ptr(),
+                                         _hip.stream_ptr(dev))
+    _hip.check(rc, "splat_acsr_build")
+    host = summary.cpu()  # the one synchronisation: T is returned as a Python int, like the reference
+    assert int(host[1]) == 0, "Incorrect unpacking of affine-indices."
+    b.T = int(host[0])
+    entry.builds[BLOCK_HEIGHT] = b
+    return b
+
+
+def instantiate_metadata(mask, BLOCK_HEIGHT: int, GPU_ID: Any = 0) -> ACSR:
+    """Host containers of the ACSR (values as stored, i.e. rounded to float32)."""
+    b = build_acsr(mask, BLOCK_HEIGHT, _hip.resolve_device(GPU_ID))
+    a0, a1 = b.dTos_lin.tolist(), b.dTos_trans.tolist()
+    s0, s1 = b.sTod_lin.tolist(), b.sTod_trans.tolist()
+    nz = [int(x) for x in b.nnz.tolist()]
+    d2s = [AffineIndices(a0[i], a1[i], nz[i]) for i in range(len(nz))]
+    s2d = [AffineIndicesInt(int(s0[i]), s1[i], nz[i]) for i in range(len(nz))]
+    return ACSR(d2s, s2d, list(zip(b.span_start.tolist(), b.span_end.tolist())))
+
+
+def create_acsr(mask, BLOCK_HEIGHT: int, GPU_ID: Any):
+    """(dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnzs, T, span_loop_start, span_loop_end): seven float32
+    device tensors and the trailing dimension T = max row nnz as an int.
+
+    The returned ``sTod_translations`` tensor carries an attribute ``splat_first_col`` (int32 tensor, first
+    live column per row) that the launchers pick up: rows with a single live column store translation 0
+    whatever that column is, so the column itself has to travel separately."""
+    dev = _hip.resolve_device(GPU_ID)
+    b = build_acsr(mask, BLOCK_HEIGHT, dev)
+    b.sTod_trans.splat_first_col = b.row_first
+    return (b.dTos_lin, b.dTos_trans, b.sTod_lin, b.sTod_trans, b.nnz, b.T, b.span_start, b.span_end)
+
+
+class ACSRSegments:
+    """Several disjoint affine segments per row.  Segment k owns compressed slots
+    [offsets[k], offsets[k] + T_k); ``T`` is the total trailing dimension."""
+
+    def __init__(self, tuples: Sequence[tuple], first_cols: Sequence[torch.Tensor | None]):
+        self.tuples = list(tuples)
+        self.first_cols = list(first_cols)
+        self.offsets = []
+        off = 0
+        for t in self.tuples:
+            self.offsets.append(off)
+            off += int(t[5])
+        self.T = off
+
+    def __len__(self) -> int:
+        return len(self.tuples)
+
+    def seg_args(self) -> list[tuple]:
+        return [(t[0], t[1], t[2], t[3], t[4], fc, off) for t, fc, off in zip(self.tuples, self.first_cols, self.offsets)]
+
+    @staticmethod
+    def single(dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnzs, T) -> "ACSRSegments":
+        fc = getattr(sTod_trans, "splat_first_col", None)
+        return ACSRSegments([(dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnzs, T, None, None)], [fc])
+
+
+def create_acsr_segments(masks: Sequence, BLOCK_HEIGHT: int, GPU_ID: Any) -> ACSRSegments:
+    """One ``create_acsr`` per segment mask; the masks must be pairwise disjoint."""
+    tuples = [create_acsr(m, BLOCK_HEIGHT, GPU_ID) for m in masks]
+    return ACSRSegments(tuples, [t[3].splat_first_col for t in tuples])
+
+
+def row_extents(mask, GPU_ID: Any) -> tuple[torch.Tensor, torch.Tensor]:
+    """(first, last) nonzero column per row as int32 device tensors (cols / -1 for an empty row)."""
+    b = build_acsr(mask, 16, _hip.resolve_device(GPU_ID))
+    return b.row_first, b.row_last

@@ -1,0 +1,170 @@
+"""Regular (ACSR) sparse attention: SDDMM -> softmax -> SpMM, or the three fused into one kernel.
+
+Mirrors the reference's ``SPLAT/r_attention.py``: ``RegularAttention`` (:12-100) keeps its constructor
+signature, attribute names and ``forward([q, kT, v])``; ``unit`` (:102-110) keeps its signature.
+
+Differences, all opt-in or invisible to a caller of the reference:
+  * ``forward`` runs the fused online-softmax kernel by default (``fused=False`` gives the three launches);
+    the two [B, H, L, T] intermediates are therefore allocated on first use, not in ``__init__``;
+  * ``scale`` (default 1.0: the reference applies no softmax scale) multiplies the scores;
+  * ``mask`` may be a list of lists (reference), an array / tensor, a ``MaskPattern`` or a list of
+    ``MaskPattern`` segments (several affine segments per row).
+"""
+from __future__ import annotations
+
+from typing import Any
+
+import torch
+import torch.nn as nn
+
+import _splat_hip as _hip
+from acsr_helpers import (ACSRSegments, MaskPattern, create_acsr, create_acsr_segments, create_blocked_mask,  # noqa: F401
+                          create_causal_windowed_mask, create_windowed_mask, mask_shape)
+from r_sddmm import rsddmm_launcher, rsddmm_preamble
+from r_softmax import rsoftmax_launcher, rsoftmax_preamble
+from r_spmm import rspmm_launcher, rspmm_preamble
+
+
+def _is_segment_list(mask) -> bool:
+    return isinstance(mask, (list, tuple)) and len(mask) > 0 and isinstance(mask[0], (MaskPattern, torch.Tensor))
+
+
+def attention_launcher(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor, output: torch.Tensor,
+                       segments: ACSRSegments, scale: float = 1.0) -> torch.Tensor:
+    """Fused forward: output[b, h, r, :] = softmax over the live columns of (scale * q.kT)[b, h, r, :] times v.
+    q [B, H, L, d], kT [B, H, d, L] (unit stride along d or along L), v [B, H, L, d], output [B, H, L, d];
+    d in {64, 128}; one dtype for all four."""
+    for name, t in (("q", q), ("kT", kT), ("v", v), ("output", output)):
+        _hip.require_device_tensor(t, name)
+        if t.dim() != 4:
+            raise _hip.SplatError(f"{name} must be 4-D")
+    if not (q.dtype == kT.dtype == v.dtype == output.dtype):
+        raise _hip.SplatError("q, kT, v and output must share a dtype")
+    B, H, L, d = q.shape
+    if tuple(kT.shape) != (B, H, d, L) or tuple(v.shape) != (B, H, L, d) or tuple(output.shape) != (B, H, L, d):
+        raise _hip.SplatError(f"expected kT {(B, H, d, L)}, v and output {(B, H, L, d)}; got {tuple(kT.shape)}, "
+                              f"{tuple(v.shape)}, {tuple(output.shape)}")
+    if q.stride(3) != 1:
+        q = q.contiguous()
+    if v.stride(3) != 1:
+        v = v.contiguous()
+    if kT.stride(2) != 1 and kT.stride(3) != 1:
+        kT = kT.contiguous()
+    if output.stride(3) != 1:
+        raise _hip.SplatError("output needs unit stride along d")
+    qs, ks, vs, os_ = q.stride(), kT.stride(), v.stride(), output.stride()
+    dev = q.device
+    arr = _hip.seg_array(segments.seg_args())
+    with torch.cuda.device(dev):
+        rc = _hip.lib().splat_attention_fwd(q.data_ptr(), qs[0], qs[1], qs[2], kT.data_ptr(), ks[0], ks[1], ks[2], ks[3],
+                                            v.data_ptr(), vs[0], vs[1], vs[2], output.data_ptr(), os_[0], os_[1], os_[2],
+                                            arr, len(segments), B, H, L, d, float(scale), _hip.dtype_code(q.dtype),
+                                            _hip.stream_ptr(dev))
+    _hip.check(rc, "splat_attention_fwd")
+    return output
+
+
+class RegularAttention(nn.Module):
+
+    def __init__(self, batch: int, seq_length: int, num_heads: int, head_dim: int, mask,
+                 BLOCK_SIZE_Y: int, BLOCK_SIZE_X: int, GPU_ID: Any, out_dtype: torch.dtype,
+                 *, scale: float | None = None, fused: bool = True):
+        super().__init__()
+        self._device = _hip.resolve_device(GPU_ID)
+        self._mask = mask
+        self._shape = (batch, num_heads, seq_length, head_dim)
+        self._out_dtype = out_dtype
+        self._GPU_ID = GPU_ID
+        self.scale = 1.0 if scale is None else float(scale)
+        self.fused = fused
+
+        if _is_segment_list(mask):
+            self.segments = create_acsr_segments(mask, BLOCK_SIZE_Y, GPU_ID)
+        else:
+            t = create_acsr(mask, BLOCK_SIZE_Y, GPU_ID)
+            self.segments = ACSRSegments([t], [t[3].splat_first_col])
+        first = self.segments.tuples[0]
+
+        # ACSR metadata of the (first) segment under the reference's attribute names.
+        self.dTos_linear_transformations = first[0]
+        self.dTos_translations = first[1]
+        self.sTod_linear_transformations = first[2]
+        self.sTod_translations = first[3]
+        self.acsr_trailing_dim = self.segments.T
+        self.nnzs = first[4]
+        self.span_loop_start = first[6]
+        self.span_loop_end = first[7]
+
+        self.BLOCK_SIZE_Y = BLOCK_SIZE_Y
+        self.BLOCK_SIZE_X = BLOCK_SIZE_X
+
+        self.rspmm_output = torch.empty(self._shape, dtype=out_dtype, device=self._device)
+        self.rspmm_grid_dim = (-(-head_dim // BLOCK_SIZE_X), -(-seq_length // BLOCK_SIZE_Y), batch * num_heads)
+        self._unfused_ready = False
+
+    # The two [B, H, L, T] intermediates and the reference's launch geometry exist only for the unfused path.
+    def _prepare_unfused(self):
+        if self._unfused_ready:
+            return
+        B, H, L, _ = self._shape
+        T = self.acsr_trailing_dim
+        tile_mask = self._mask[0] if _is_segment_list(self._mask) else self._mask
+        (self._rsddmm_output, self._rsddmm_grid_dim, self._rsddmm_tb_map_x,
+         self._rsddmm_tb_map_y) = rsddmm_preamble(tile_mask, (B, H, L, T), self.BLOCK_SIZE_X, self.BLOCK_SIZE_Y,
+                                                  self._GPU_ID, self._out_dtype)
+        (self._rsoftmax_grid_dim, self._rsoftmax_output, _,
+         self._rsoftmax_trailing_dim_pow_two) = rsoftmax_preamble(tile_mask, (B, H, L, T), self.BLOCK_SIZE_X,
+                                                                  self._GPU_ID, self._out_dtype)
+        self._unfused_ready = True
+
+    def _lazy(name):  # noqa: N805
+        def get(self):
+            self._prepare_unfused()
+            return getattr(self, "_" + name)
+        return property(get)
+
+    rsddmm_output = _lazy("rsddmm_output")
+    rsddmm_grid_dim = _lazy("rsddmm_grid_dim")
+    rsddmm_tb_map_x = _lazy("rsddmm_tb_map_x")
+    rsddmm_tb_map_y = _lazy("rsddmm_tb_map_y")
+    rsoftmax_output = _lazy("rsoftmax_output")
+    rsoftmax_grid_dim = _lazy("rsoftmax_grid_dim")
+    rsoftmax_trailing_dim_pow_two = _lazy("rsoftmax_trailing_dim_pow_two")
+    del _lazy
+
+    def forward(self, x):
+        """x = [q, kT, v] after RoPE: q [B, H, L, d], kT [B, H, d, L], v [B, H, L, d].  Returns the module's
+        output buffer (reused by every call)."""
+        q, k, v = x
+        fusable = self.fused and q.shape[-1] in (64, 128) and q.dtype == k.dtype == v.dtype == self._out_dtype
+        if fusable:
+            return attention_launcher(q, k, v, self.rspmm_output, self.segments, self.scale)
+
+        multi = self.segments if len(self.segments) > 1 else None
+        rsddmm_launcher(q, k, self.rsddmm_output,
+                        self.dTos_linear_transformations, self.dTos_translations,
+                        self.sTod_linear_transformations, self.sTod_translations,
+                        self.acsr_trailing_dim, self.nnzs,
+                        self.rsddmm_grid_dim, self.rsddmm_tb_map_x,
+                        self.rsddmm_tb_map_y, self.BLOCK_SIZE_Y, self.BLOCK_SIZE_X, scale=self.scale, segments=multi)
+        rsoftmax_launcher(self.rsddmm_output, self.rsoftmax_output,
+                          self.dTos_linear_transformations, self.dTos_translations,
+                          self.sTod_linear_transformations, self.sTod_translations,
+                          self.acsr_trailing_dim, self.rsoftmax_trailing_dim_pow_two, self.nnzs,
+                          self.rsoftmax_grid_dim, self.BLOCK_SIZE_X, segments=multi)
+        rspmm_launcher(self.rsoftmax_output, v, self.rspmm_output,
+                       self.dTos_linear_transformations, self.dTos_translations,
+                       self.sTod_linear_transformations, self.sTod_translations,
+                       self.span_loop_start, self.span_loop_end, self.acsr_trailing_dim,
+                       self.nnzs, self.rspmm_grid_dim, self.BLOCK_SIZE_Y, self.BLOCK_SIZE_X, segments=multi)
+        return self.rspmm_output
+
+
+def unit(q, k, v, w_q, w_k, w_v, attn: RegularAttention):
+    """Project [B, S, D] activations with [D, N, H] weights and attend.  The projections are laid out
+    [B, N, S, H] (heads before sequence), which is the layout ``RegularAttention.forward`` documents;
+    K is handed over as a transposed view, not a copy."""
+    q = torch.einsum('bsd, dnh -> bnsh', q, w_q)
+    k = torch.einsum('bsd, dnh -> bnsh', k, w_k)
+    v = torch.einsum('bsd, dnh -> bnsh', v, w_v)
+    return attn([q, k.transpose(2, 3), v])

@@ -1,0 +1,102 @@
+"""R-SDDMM: Q.K^T sampled onto the live slots of an ACSR.
+
+Mirrors the reference's ``SPLAT/r_sddmm.py``: ``gen_block_mappings`` / ``naive_block_mappings`` (:117-151),
+``rsddmm_preamble`` (:154-169) and ``rsddmm_launcher`` (:171-184) keep their names, positional parameters
+and return tuples.  The Triton kernel (:15-115) is replaced by ``splat_sddmm`` (MFMA, gfx950).
+"""
+from __future__ import annotations
+
+from typing import Any
+
+import numpy as np
+import torch
+
+import _splat_hip as _hip
+from acsr_helpers import ACSRSegments, create_acsr, create_blocked_mask, mask_shape, row_extents  # noqa: F401
+
+
+def naive_block_mappings(mask, BLOCK_HEIGHT: int, BLOCK_WIDTH: int, GPU_ID: Any) -> tuple[torch.Tensor, torch.Tensor]:
+    """Anchor points (x = column, y = row) of the BLOCK_HEIGHT x BLOCK_WIDTH tiles that cover each row block's
+    nonzero column range, as int32 device tensors -- the tiling the reference's launch grid is derived from.
+    Its conventions are kept: max(rows // BLOCK_HEIGHT, 1) row blocks, anchors from the block's first
+    nonzero column while strictly below its last one."""
+    dev = _hip.resolve_device(GPU_ID)
+    rows, cols = mask_shape(mask)
+    first, last = row_extents(mask, dev)
+    first, last = first.cpu().numpy().astype(np.int64), last.cpu().numpy().astype(np.int64)
+    n_blocks = max(rows // BLOCK_HEIGHT, 1)
+    pad = n_blocks * BLOCK_HEIGHT - min(rows, n_blocks * BLOCK_HEIGHT)
+    f = np.concatenate([first[:n_blocks * BLOCK_HEIGHT], np.full(pad, cols)]).reshape(n_blocks, BLOCK_HEIGHT)
+    l = np.concatenate([last[:n_blocks * BLOCK_HEIGHT], np.full(pad, -1)]).reshape(n_blocks, BLOCK_HEIGHT)
+    lo = np.minimum(f.min(axis=1), cols)
+    hi = np.maximum(l.max(axis=1), 0)
+    counts = np.where(hi > lo, -(-(hi - lo) // BLOCK_WIDTH), 0)
+    total = int(counts.sum())
+    assert total > 0, "Issues with generating arrangement!"
+    blk = np.repeat(np.arange(n_blocks), counts)
+    within = np.arange(total) - np.repeat(np.cumsum(counts) - counts, counts)
+    xs = (lo[blk] + within * BLOCK_WIDTH).astype(np.int32)
+    ys = (blk * BLOCK_HEIGHT).astype(np.int32)
+    return torch.from_numpy(xs).to(dev), torch.from_numpy(ys).to(dev)
+
+
+def gen_block_mappings(mask, BLOCK_HEIGHT: int, BLOCK_WIDTH: int, GPU_ID: Any,
+                       is_naive: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
+    return naive_block_mappings(mask, BLOCK_HEIGHT, BLOCK_WIDTH, GPU_ID)
+
+
+def rsddmm_preamble(mask, output_shape: tuple[int], BLOCK_SIZE_X: int, BLOCK_SIZE_Y: int, GPU_ID: Any,
+                    out_dtype: torch.dtype):
+    """-> (output [B, H, L, T] uninitialised, grid_dim = (n_tiles, B*H), tb_map_x, tb_map_y)."""
+    dev = _hip.resolve_device(GPU_ID)
+    output = torch.empty(tuple(output_shape), dtype=out_dtype, device=dev)
+    tb_map_x, tb_map_y = gen_block_mappings(mask, BLOCK_SIZE_Y, BLOCK_SIZE_X, GPU_ID)
+    assert tb_map_x.shape == tb_map_y.shape, "Incorrect tiling arrangement!"
+    grid_dim = (tb_map_x.shape[0], output_shape[0] * output_shape[1])
+    return (output, grid_dim, tb_map_x, tb_map_y)
+
+
+def _strides4(t: torch.Tensor, name: str):
+    if t.dim() != 4:
+        raise _hip.SplatError(f"{name} must be 4-D [batch, heads, ., .]")
+    return t.stride()
+
+
+def rsddmm_launcher(x: torch.Tensor, y: torch.Tensor, output: torch.Tensor,
+                    dTos_linear_transformations: torch.Tensor, dTos_translations: torch.Tensor,
+                    sTod_linear_transformations: torch.Tensor, sTod_translations: torch.Tensor,
+                    trailing_dim: int, nnzs: torch.Tensor, grid_dim: tuple[int],
+                    tb_map_x: torch.Tensor, tb_map_y: torch.Tensor,
+                    BLOCK_SIZE_Y: int, BLOCK_SIZE_X: int, *, scale: float | None = None,
+                    segments: ACSRSegments | None = None):
+    """x = Q [B, H, L, d]; y = K^T [B, H, d, L] (any strides with unit stride along d or along L, so
+    ``k.transpose(2, 3)`` of a [B, H, L, d] tensor needs no copy); output [B, H, L, T] is written in place for
+    the live slots only.  ``grid_dim`` / ``tb_map_*`` / ``BLOCK_SIZE_*`` describe the reference's launch
+    geometry and are accepted unchanged; the HIP kernel tiles by itself from the row maps.
+    Returns (output, sTod_linear_transformations, sTod_translations, nnzs)."""
+    for name, t in (("x", x), ("y", y), ("output", output)):
+        _hip.require_device_tensor(t, name)
+    if x.dtype != y.dtype:
+        raise _hip.SplatError("x and y must share a dtype")
+    segs = segments or ACSRSegments.single(dTos_linear_transformations, dTos_translations,
+                                           sTod_linear_transformations, sTod_translations, nnzs, trailing_dim)
+    B, H, L, d = x.shape
+    if y.shape[0] != B or y.shape[1] != H or y.shape[2] != d:
+        raise _hip.SplatError(f"y must be [B, H, d, n] = [{B}, {H}, {d}, n], got {tuple(y.shape)}")
+    n_keys = y.shape[3]
+    if x.stride(3) != 1 and d > 1:
+        x = x.contiguous()
+    if y.stride(2) != 1 and y.stride(3) != 1:
+        y = y.contiguous()
+    if not output.is_contiguous() or tuple(output.shape) != (B, H, L, trailing_dim):
+        raise _hip.SplatError(f"output must be a contiguous [B, H, L, T] = {(B, H, L, trailing_dim)} tensor")
+    qs, ks = _strides4(x, "x"), _strides4(y, "y")
+    dev = x.device
+    arr = _hip.seg_array(segs.seg_args())
+    with torch.cuda.device(dev):
+        rc = _hip.lib().splat_sddmm(x.data_ptr(), qs[0], qs[1], qs[2], y.data_ptr(), ks[0], ks[1], ks[2], ks[3],
+                                    output.data_ptr(), arr, len(segs), B, H, L, n_keys, d, trailing_dim,
+                                    1.0 if scale is None else float(scale), _hip.dtype_code(x.dtype),
+                                    _hip.dtype_code(output.dtype), _hip.stream_ptr(dev))
+    _hip.check(rc, "splat_sddmm")
+    return (output, sTod_linear_transformations, sTod_translations, nnzs)

@@ -1,0 +1,258 @@
+// ACSR builder and mask generators.
+//
+// splat_acsr_build: one wavefront per mask row streams the row once (16-byte loads), reducing the
+// byte sum (nnz), the first two columns whose byte equals 1 (the affine map's anchors a < b) and the
+// first/last nonzero column.  Lane 0 then evaluates the 2x2 solve of acsr_helpers.py:122 in closed
+// form in double precision and rounds to float32, which is what the reference's
+// float64 -> torch.FloatTensor conversion stores.  A second, tiny kernel folds rows into the
+// per-row-block span pairs (acsr_helpers.py:135-140).  HBM-bound: rows*ld bytes in, 28*rows out.
+#include "splat_common.hpp"
+
+namespace splat {
+
+constexpr int kInf = 0x7fffffff;
+
+// 0x80 in every byte of y that is zero (exact, no borrow artefacts).
+__device__ __forceinline__ uint32_t zero_bytes(uint32_t y) {
+    return ~(((y & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | y | 0x7F7F7F7Fu);
+}
+
+struct RowScan {
+    uint32_t sum;  // sum of byte values
+    int m1, m2;    // two smallest columns whose byte == 1
+    int first, last;  // first / last nonzero column
+
+    __device__ __forceinline__ void init() {
+        sum = 0;
+        m1 = m2 = first = kInf;
+        last = -1;
+    }
+    __device__ __forceinline__ void add_one(int col) {
+        if (col < m1) {
+            m2 = m1;
+            m1 = col;
+        } else if (col < m2 && col != m1) {
+            m2 = col;
+        }
+    }
+    __device__ __forceinline__ void dword(uint32_t x, int col0) {
+        if (x == 0) return;
+        sum = __builtin_amdgcn_sad_u8(x, 0u, sum);
+        uint32_t nz = ~zero_bytes(x) & 0x80808080u;  // bytes that are nonzero
+        int lo = (__builtin_ctz(nz) >> 3), hi = ((31 - __builtin_clz(nz)) >> 3);
+        first = min(first, col0 + lo);
+        last = max(last, col0 + hi);
+        if (m2 == kInf) {
+            uint32_t eq = zero_bytes(x ^ 0x01010101u);  // bytes equal to 1
+            while (eq) {
+                int b = __builtin_ctz(eq) >> 3;
+                add_one(col0 + b);
+                eq &= eq - 1;
+            }
+        }
+    }
+    __device__ __forceinline__ void byte(uint32_t x, int col) {
+        if (x == 0) return;
+        sum += x;
+        first = min(first, col);
+        last = max(last, col);
+        if (x == 1) add_one(col);
+    }
+    __device__ __forceinline__ void wave_reduce() {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            uint32_t s2 = __shfl_xor(sum, o);
+            int a1 = __shfl_xor(m1, o), a2 = __shfl_xor(m2, o);
+            int f2 = __shfl_xor(first, o), l2 = __shfl_xor(last, o);
+            sum += s2;
+            int n1 = min(m1, a1);
+            int n2 = min(max(m1, a1), min(m2, a2));
+            m1 = n1;
+            m2 = n2;
+            first = min(first, f2);
+            last = max(last, l2);
+        }
+    }
+};
+
+__global__ void acsr_init_summary(int32_t* summary) {
+    if (threadIdx.x < 8) summary[threadIdx.x] = 0;
+}
+
+__global__ __launch_bounds__(256) void acsr_rows_kernel(const uint8_t* __restrict__ mask, int rows, int cols,
+                                                        int64_t ld, int vec_ok, float* __restrict__ dTos_lin,
+                                                        float* __restrict__ dTos_trans, float* __restrict__ sTod_lin,
+                                                        float* __restrict__ sTod_trans, float* __restrict__ nnz_out,
+                                                        int32_t* __restrict__ row_first,
+                                                        int32_t* __restrict__ row_last, int32_t* __restrict__ summary) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const uint8_t* p = mask + (int64_t)row * ld;
+    RowScan s;
+    s.init();
+    int done = 0;
+    if (vec_ok) {
+        const int nvec = cols >> 4;
+        const uint4* pv = reinterpret_cast<const uint4*>(p);
+        int i = lane;
+        // four independent 16-byte loads in flight per lane
+        for (; i + 192 < nvec; i += 256) {
+            uint4 x0 = pv[i], x1 = pv[i + 64], x2 = pv[i + 128], x3 = pv[i + 192];
+            const uint4 xs[4] = {x0, x1, x2, x3};
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                int c = (i + 64 * u) << 4;
+                if ((xs[u].x | xs[u].y | xs[u].z | xs[u].w) == 0) continue;
+                s.dword(xs[u].x, c);
+                s.dword(xs[u].y, c + 4);
+                s.dword(xs[u].z, c + 8);
+                s.dword(xs[u].w, c + 12);
+            }
+        }
+        for (; i < nvec; i += 64) {
+            uint4 x = pv[i];
+            int c = i << 4;
+            s.dword(x.x, c);
+            s.dword(x.y, c + 4);
+            s.dword(x.z, c + 8);
+            s.dword(x.w, c + 12);
+        }
+        done = nvec << 4;
+    }
+    for (int c = done + lane; c < cols; c += 64) s.byte(p[c], c);
+    s.wave_reduce();
+    if (lane != 0) return;
+
+    const int nnz = (int)s.sum;
+    double x0 = 1.0, x1 = 0.0;
+    int step = 1;
+    if (nnz > 1) {
+        if (s.m1 == kInf || s.m2 == kInf) {
+            atomicAdd(&summary[1], 1);  // the reference asserts here (acsr_helpers.py:119)
+        } else {
+            step = s.m2 - s.m1;
+            x0 = 1.0 / (double)step;
+            // the solve yields +0.0 (not -0.0) for a == 0
+            x1 = (s.m1 == 0) ? 0.0 : -(double)s.m1 / (double)step;
+        }
+    }
+    dTos_lin[row] = (float)x0;
+    dTos_trans[row] = (float)x1;
+    sTod_lin[row] = (float)step;
+    sTod_trans[row] = (float)fabs(x1);
+    nnz_out[row] = (float)nnz;
+    if (row_first) row_first[row] = (s.first == kInf) ? cols : s.first;
+    if (row_last) row_last[row] = s.last;
+    atomicMax(&summary[0], nnz);
+}
+
+// One thread per row block: span_start = min(cols, min_r trans_r), span_end = max(-1, max_r nnz_r*lin_r + trans_r)
+// evaluated in double from the exact integers (a, lin, nnz) and rounded once to float32.
+__global__ void acsr_spans_kernel(const float* __restrict__ sTod_lin, const float* __restrict__ sTod_trans,
+                                  const float* __restrict__ nnz, int rows, int cols, int block_height,
+                                  float* __restrict__ span_start, float* __restrict__ span_end) {
+    const int g = blockIdx.x * blockDim.x + threadIdx.x;
+    const int n_blocks = (rows + block_height - 1) / block_height;
+    if (g >= n_blocks) return;
+    double lo = (double)cols, hi = -1.0;
+    const int r1 = min(rows, (g + 1) * block_height);
+    for (int r = g * block_height; r < r1; ++r) {
+        const float linf = sTod_lin[r];
+        const int lin = (int)linf;
+        const int a = (int)rintf(linf * sTod_trans[r]);
+        const double t = (double)a / (double)lin;
+        lo = fmin(lo, t);
+        hi = fmax(hi, (double)((int64_t)nnz[r] * lin) + t);
+    }
+    span_start[g] = (float)lo;
+    span_end[g] = (float)hi;
+}
+
+__device__ __forceinline__ bool mask_pred(int pattern, int64_t i, int64_t j, int64_t p0, int64_t p1) {
+    switch (pattern) {
+        case SPLAT_MASK_BLOCKED: {
+            if (i < p0) return j < p0;
+            int64_t start = (i / p0 - 1) * p0;
+            return start <= j && j < start + 2 * p0;
+        }
+        case SPLAT_MASK_WINDOWED:
+            return i - p0 <= j && j <= i + p0;
+        case SPLAT_MASK_CAUSAL_WINDOWED:
+            return i - p0 <= j && j <= i;
+        case SPLAT_MASK_DILATED: {
+            int64_t rel = j - (i - (p0 * p1) / 2);
+            return rel >= 0 && rel < p0 * p1 && rel % p1 == 0;
+        }
+        case SPLAT_MASK_STRIDED_LOCAL:
+            return j <= i && j > i - p0;
+        case SPLAT_MASK_STRIDED_FAR:
+            return j <= i - p0 && j % p1 == p1 - 1;
+    }
+    return false;
+}
+
+__global__ __launch_bounds__(256) void mask_generate_kernel(uint8_t* __restrict__ mask, int rows, int cols,
+                                                            int64_t ld, int pattern, int64_t p0, int64_t p1,
+                                                            int vec_ok) {
+    const int chunks = (cols + 15) >> 4;
+    const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (id >= (int64_t)rows * chunks) return;
+    const int i = (int)(id / chunks);
+    const int c0 = (int)(id % chunks) << 4;
+    uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int b = 0; b < 16; ++b) {
+        int j = c0 + b;
+        if (j < cols && mask_pred(pattern, i, j, p0, p1)) w[b >> 2] |= 1u << ((b & 3) * 8);
+    }
+    uint8_t* dst = mask + (int64_t)i * ld + c0;
+    if (vec_ok && c0 + 16 <= cols) {
+        *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
+    } else {
+        for (int b = 0; b < 16 && c0 + b < cols; ++b) dst[b] = (uint8_t)((w[b >> 2] >> ((b & 3) * 8)) & 0xff);
+    }
+}
+
+}  // namespace splat
+
+using namespace splat;
+
+extern "C" int splat_acsr_build(const uint8_t* mask, int64_t rows, int64_t cols, int64_t ld, int32_t block_height,
+                                float* dTos_lin, float* dTos_trans, float* sTod_lin, float* sTod_trans, float* nnz,
+                                float* span_start, float* span_end, int32_t* row_first, int32_t* row_last,
+                                int32_t* summary, void* stream) {
+    if (!mask || !dTos_lin || !dTos_trans || !sTod_lin || !sTod_trans || !nnz || !span_start || !span_end || !summary)
+        return fail(SPLAT_E_NULL, "splat_acsr_build: null pointer argument");
+    if (rows <= 0 || cols <= 0 || ld < cols || block_height <= 0)
+        return fail(SPLAT_E_SHAPE, "splat_acsr_build: need rows > 0, cols > 0, ld >= cols, block_height > 0 (got %lld, %lld, %lld, %d)",
+                    (long long)rows, (long long)cols, (long long)ld, block_height);
+    // a row sum must fit int32 and columns must be exactly representable in float32 metadata
+    if (rows > (1 << 23) || cols > (1 << 23))
+        return fail(SPLAT_E_SHAPE, "splat_acsr_build: rows and cols are limited to 2^23 (got %lld, %lld)", (long long)rows, (long long)cols);
+    hipStream_t st = (hipStream_t)stream;
+    const int vec_ok = ((reinterpret_cast<uintptr_t>(mask) & 15) == 0 && (ld & 15) == 0) ? 1 : 0;
+    acsr_init_summary<<<1, 64, 0, st>>>(summary);
+    acsr_rows_kernel<<<(unsigned)((rows + 3) / 4), 256, 0, st>>>(mask, (int)rows, (int)cols, ld, vec_ok, dTos_lin, dTos_trans,
+                                                                 sTod_lin, sTod_trans, nnz, row_first, row_last, summary);
+    const int n_blocks = (int)((rows + block_height - 1) / block_height);
+    acsr_spans_kernel<<<(n_blocks + 255) / 256, 256, 0, st>>>(sTod_lin, sTod_trans, nnz, (int)rows, (int)cols, block_height,
+                                                               span_start, span_end);
+    return check_launch("splat_acsr_build");
+}
+
+extern "C" int splat_mask_generate(uint8_t* mask, int64_t rows, int64_t cols, int64_t ld, int32_t pattern, int64_t p0,
+                                   int64_t p1, void* stream) {
+    if (!mask) return fail(SPLAT_E_NULL, "splat_mask_generate: null mask");
+    if (rows <= 0 || cols <= 0 || ld < cols || rows > (1 << 23) || cols > (1 << 23))
+        return fail(SPLAT_E_SHAPE, "splat_mask_generate: bad shape rows=%lld cols=%lld ld=%lld", (long long)rows, (long long)cols, (long long)ld);
+    if (pattern < SPLAT_MASK_BLOCKED || pattern > SPLAT_MASK_STRIDED_FAR)
+        return fail(SPLAT_E_UNSUPPORTED, "splat_mask_generate: unknown pattern %d", pattern);
+    const bool needs_p1 = pattern == SPLAT_MASK_DILATED || pattern == SPLAT_MASK_STRIDED_FAR;
+    if (p0 < 0 || (pattern == SPLAT_MASK_BLOCKED && p0 <= 0) || (needs_p1 && p1 <= 0))
+        return fail(SPLAT_E_SHAPE, "splat_mask_generate: bad pattern parameters p0=%lld p1=%lld", (long long)p0, (long long)p1);
+    const int vec_ok = ((reinterpret_cast<uintptr_t>(mask) & 15) == 0 && (ld & 15) == 0) ? 1 : 0;
+    const int64_t n = rows * ((cols + 15) >> 4);
+    mask_generate_kernel<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(mask, (int)rows, (int)cols, ld, pattern, p0, p1, vec_ok);
+    return check_launch("splat_mask_generate");
+}

@@ -1,0 +1,233 @@
+// Per-workgroup planning shared by the SDDMM, SpMM and fused attention kernels: from the affine maps of
+// the workgroup's rows decide which key positions the tiles enumerate and how a row tests validity.
+#pragma once
+#include "splat_common.hpp"
+
+namespace splat {
+
+constexpr int kBN = 64;  // key positions per tile
+
+// Device pointers of one segment (kernel-argument form of splat_acsr_seg).
+struct SegPtrs {
+    const float* sTod_lin;
+    const float* sTod_trans;
+    const float* nnz;
+    const int32_t* first_col;
+    int slot_offset;
+    int pad_;
+};
+
+// Per-workgroup plan of one segment.
+struct SegPlan {
+    int c0;       // dense column of tile position j = 0
+    int cs;       // column step between consecutive tile positions
+    int n_tiles;  // kBN-position tiles to walk
+    int uniform;  // 1: all rows share step and phase -> position j of row r is slot j - lo_r;
+                  // 0: positions are dense columns and a row applies the full affine test
+};
+
+__device__ __forceinline__ RowMap load_row_map(const SegPtrs& s, int r) {
+    return load_row_map(s.sTod_lin, s.sTod_trans, s.nnz, s.first_col, r);
+}
+
+// Scratch the planner needs in LDS.
+struct PlanScratch {
+    int red[SPLAT_MAX_SEGMENTS][5];  // amin, cmax, linmin, linmax, nonuniform
+};
+
+// Fill plan[0..n_seg) for rows [r0, r0+BM) ∩ [0, n_rows).  All 256 threads of the workgroup call it; it
+// ends with a barrier.  `allow_gather` = false forces dense walks (column step 1).
+template <int BM>
+__device__ __forceinline__ void plan_segments(const SegPtrs* seg, int n_seg, int r0, int n_rows, bool allow_gather,
+                                              SegPlan* plan, PlanScratch* ps, int tid) {
+    if (tid < SPLAT_MAX_SEGMENTS) {
+        ps->red[tid][0] = 0x7fffffff;
+        ps->red[tid][1] = -1;
+        ps->red[tid][2] = 0x7fffffff;
+        ps->red[tid][3] = 0;
+        ps->red[tid][4] = 0;
+    }
+    __syncthreads();
+    for (int sg = 0; sg < n_seg; ++sg) {
+        for (int rr = tid; rr < BM; rr += 256) {
+            const int r = r0 + rr;
+            if (r < n_rows) {
+                RowMap m = load_row_map(seg[sg], r);
+                if (m.cnt > 0) {
+                    atomicMin(&ps->red[sg][0], m.a);
+                    atomicMax(&ps->red[sg][1], m.a + m.lin * (m.cnt - 1));
+                    if (m.cnt > 1) {
+                        atomicMin(&ps->red[sg][2], m.lin);
+                        atomicMax(&ps->red[sg][3], m.lin);
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+    for (int sg = 0; sg < n_seg; ++sg) {
+        const int amin = ps->red[sg][0], linmin = ps->red[sg][2], linmax = ps->red[sg][3];
+        const int step = (linmax == 0) ? 1 : linmin;  // no row with 2+ columns: any step fits
+        if (linmax != 0 && linmin != linmax) {
+            if (tid == 0) ps->red[sg][4] = 1;
+        } else if (step > 1) {
+            for (int rr = tid; rr < BM; rr += 256) {
+                const int r = r0 + rr;
+                if (r < n_rows) {
+                    RowMap m = load_row_map(seg[sg], r);
+                    if (m.cnt > 0 && ((m.a - amin) % step) != 0) atomicOr(&ps->red[sg][4], 1);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    if (tid < n_seg) {
+        const int sg = tid;
+        SegPlan pl;
+        const int amin = ps->red[sg][0], cmax = ps->red[sg][1], linmin = ps->red[sg][2], linmax = ps->red[sg][3];
+        if (cmax < 0) {
+            pl.c0 = 0;
+            pl.cs = 1;
+            pl.n_tiles = 0;
+            pl.uniform = 1;
+        } else {
+            const int step = (linmax == 0) ? 1 : linmin;
+            const bool uni = (ps->red[sg][4] == 0) && (allow_gather || step == 1);
+            pl.uniform = uni ? 1 : 0;
+            pl.cs = uni ? step : 1;
+            // dense walks start on a tile boundary (keeps 16-byte K^T loads aligned and lets neighbouring row
+            // blocks share cache lines); gathered walks start at the first live column
+            pl.c0 = (pl.cs == 1) ? (amin & ~(kBN - 1)) : amin;
+            const int n_pos = (cmax - pl.c0) / pl.cs + 1;
+            pl.n_tiles = (n_pos + kBN - 1) / kBN;
+        }
+        plan[sg] = pl;
+    }
+    __syncthreads();
+}
+
+// How one row tests a tile position j (relative to the plan's c0/cs).
+//   uniform plan: live iff 0 <= j - lo < cnt, slot = j - lo
+//   dense plan:   u = j - lo is the column offset from the row's first column; live iff 0 <= u < cnt
+//                 (cnt = extent in columns) and u % lin == 0, slot = u / lin
+struct RowWin {
+    int lo, cnt, lin;
+};
+
+__device__ __forceinline__ RowWin make_row_win(const RowMap& m, const SegPlan& pl) {
+    RowWin w;
+    if (m.cnt <= 0) {
+        w.lo = 0;
+        w.cnt = 0;
+        w.lin = 1;
+    } else if (pl.uniform) {
+        w.lo = (m.a - pl.c0) / pl.cs;
+        w.cnt = m.cnt;
+        w.lin = 1;
+    } else {
+        w.lo = m.a - pl.c0;
+        w.lin = (m.cnt > 1) ? m.lin : 1;
+        w.cnt = w.lin * (m.cnt - 1) + 1;
+    }
+    return w;
+}
+
+__device__ __forceinline__ bool win_live(const RowWin& w, int j) {
+    const int u = j - w.lo;
+    return (unsigned)u < (unsigned)w.cnt && (w.lin == 1 || ((unsigned)u % (unsigned)w.lin) == 0u);
+}
+__device__ __forceinline__ int win_slot(const RowWin& w, int j) {
+    const int u = j - w.lo;
+    return (w.lin == 1) ? u : u / w.lin;
+}
+
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+
+// Transposing LDS read: the 16 lanes of a block address 4 rows x 16 columns of 16-bit elements (lane s:
+// row s/4, columns 4*(s%4)..+3); lane i of the block receives column i of the 4 rows.
+__device__ __forceinline__ s16x4 lds_tr16(const char* p) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p));
+}
+
+template <typename T>
+__device__ __forceinline__ Frag<T> frag_from_tr(s16x4 lo, s16x4 hi) {
+    Frag<T> f;
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    s16x8 r = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    f.v = __builtin_bit_cast(typename Frag<T>::vec, r);
+    return f;
+}
+
+typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+
+// Fragment whose 8 contraction slots sit in 8 consecutive LDS elements.
+template <typename T>
+__device__ __forceinline__ Frag<T> lds_frag_rowmajor(const char* p) {
+    Frag<T> f;
+    if constexpr (sizeof(T) == 2) {
+        u32x4 r = *reinterpret_cast<const u32x4*>(p);
+        f.v = __builtin_bit_cast(typename Frag<T>::vec, r);
+    } else {
+        u32x4 r0 = *reinterpret_cast<const u32x4*>(p);
+        u32x4 r1 = *reinterpret_cast<const u32x4*>(p + 16);
+        u32x8 r = __builtin_shufflevector(r0, r1, 0, 1, 2, 3, 4, 5, 6, 7);
+        f.v = __builtin_bit_cast(typename Frag<T>::vec, r);
+    }
+    return f;
+}
+
+// Fragment whose contraction index runs down the rows of an LDS tile: slots 0..3 are rows r0..r0+3,
+// slots 4..7 rows r1..r1+3, all at column col0 + lane%32.  16-bit types use two transposing reads,
+// fp32 reads 8 scalars.
+template <typename T>
+__device__ __forceinline__ Frag<T> lds_frag_cols(const char* tile, int row_bytes, int r0, int r1, int col0, int lane) {
+    Frag<T> f;
+    if constexpr (sizeof(T) == 2) {
+        const int s = lane & 15;
+        const int col = col0 + 16 * ((lane >> 4) & 1) + 4 * (s & 3);
+        const char* p0 = tile + (r0 + (s >> 2)) * row_bytes + col * 2;
+        const char* p1 = tile + (r1 + (s >> 2)) * row_bytes + col * 2;
+        f = frag_from_tr<T>(lds_tr16(p0), lds_tr16(p1));
+    } else {
+        const int col = col0 + (lane & 31);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            f.v[e] = *reinterpret_cast<const float*>(tile + (r0 + e) * row_bytes + col * 4);
+            f.v[4 + e] = *reinterpret_cast<const float*>(tile + (r1 + e) * row_bytes + col * 4);
+        }
+    }
+    return f;
+}
+
+// 8 consecutive elements from global memory (16-byte aligned).
+template <typename T>
+__device__ __forceinline__ Frag<T> global_frag(const T* p) {
+    Frag<T> f;
+    if constexpr (sizeof(T) == 2) {
+        u32x4 r = *reinterpret_cast<const u32x4*>(p);
+        f.v = __builtin_bit_cast(typename Frag<T>::vec, r);
+    } else {
+        u32x4 r0 = *reinterpret_cast<const u32x4*>(p);
+        u32x4 r1 = *reinterpret_cast<const u32x4*>(p + 4);
+        u32x8 r = __builtin_shufflevector(r0, r1, 0, 1, 2, 3, 4, 5, 6, 7);
+        f.v = __builtin_bit_cast(typename Frag<T>::vec, r);
+    }
+    return f;
+}
+
+// Fill a SegPtrs array from the host-side segment descriptors; returns 0 or a negative code.
+inline int fill_segs(const char* who, const splat_acsr_seg* segs, int n_seg, SegPtrs* out, int T) {
+    if (n_seg < 1 || n_seg > SPLAT_MAX_SEGMENTS)
+        return fail(SPLAT_E_SHAPE, "%s: n_seg must be 1..%d (got %d)", who, SPLAT_MAX_SEGMENTS, n_seg);
+    for (int k = 0; k < SPLAT_MAX_SEGMENTS; ++k) out[k] = SegPtrs{nullptr, nullptr, nullptr, nullptr, 0, 0};
+    for (int k = 0; k < n_seg; ++k) {
+        if (!segs[k].sTod_lin || !segs[k].sTod_trans || !segs[k].nnz)
+            return fail(SPLAT_E_NULL, "%s: segment %d lacks sTod_lin / sTod_trans / nnz", who, k);
+        if (T >= 0 && (segs[k].slot_offset < 0 || segs[k].slot_offset >= T))
+            return fail(SPLAT_E_SHAPE, "%s: segment %d slot_offset %d outside [0, T=%d)", who, k, segs[k].slot_offset, T);
+        out[k] = SegPtrs{segs[k].sTod_lin, segs[k].sTod_trans, segs[k].nnz, segs[k].first_col, segs[k].slot_offset, 0};
+    }
+    return 0;
+}
+
+}  // namespace splat

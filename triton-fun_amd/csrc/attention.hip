@@ -1,0 +1,440 @@
+// Fused ACSR sparse-attention forward (online softmax), gfx950.
+//
+// A workgroup of 4 wavefronts owns BM = 128*MT consecutive query rows of one (batch, head).  It walks
+// the key range its rows' affine spans cover in tiles of 64 keys.  Per tile:
+//   * all 256 threads copy the K and V tiles global -> registers -> LDS (double buffered; the copy of
+//     tile t+1 overlaps the math of tile t);
+//   * every wavefront computes the TRANSPOSED score tile S^T = K . Q^T for its 32*MT rows with
+//     32x32x16 MFMA (A = K fragment from LDS, B = Q fragment held in registers for the whole kernel).
+//     In the transposed product one lane owns one query row, so masking, the running max and the
+//     running sum need no cross-lane traffic beyond one exchange with the lane that holds the other
+//     half of the row;
+//   * P^T (the exponentials, converted to the input type) is already laid out as the B operand of
+//     O^T += V^T . P^T, whose A operand (V^T fragments) is read from the row-major V tile in LDS with
+//     the transposing LDS read (ds_read_b64_tr_b16); K^T tiles ([d, keys] input layout) use the same read.
+// The compressed score matrix never exists in memory: traffic is Q + K + V + O.
+//
+// Which keys a tile holds is decided per workgroup from the rows' (a, lin, cnt) maps: if all rows
+// share the column step and phase, tiles enumerate exactly those columns (key index c0 + cs*j,
+// gathered rows of K/V) and validity is a per-row range test in j; otherwise tiles are dense columns
+// and validity is the full affine test (offset, step divisibility, count).  Each wavefront skips
+// tiles that lie outside all of its rows' spans and drops the mask on tiles inside all of them.
+#include "acsr_plan.hpp"
+
+namespace splat {
+
+constexpr float kNegBigA = -1.0e30f;
+
+struct AttnParams {
+    const void* q;
+    const void* k;
+    const void* v;
+    void* o;
+    int64_t q_sb, q_sh, q_sl;
+    int64_t k_sb, k_sh, k_sd, k_sl;
+    int64_t v_sb, v_sh, v_sl;
+    int64_t o_sb, o_sh, o_sl;
+    int B, H, L;
+    float scale_log2e;
+    int n_seg;
+    SegPtrs seg[SPLAT_MAX_SEGMENTS];
+    int n_row_blocks;
+    int total;
+};
+
+template <typename T, int D, bool KT>
+struct TileGeom {
+    static constexpr int ES = sizeof(T);
+    static constexpr int K_ROW = KT ? (kBN * ES + 64) : (D * ES + 16);  // bytes per LDS row of the K tile
+    static constexpr int K_ROWS = KT ? D : kBN;
+    static constexpr int K_BYTES = K_ROW * K_ROWS;
+    static constexpr int V_ROW = D * ES + 64;
+    static constexpr int V_BYTES = V_ROW * kBN;
+    static constexpr int STAGE = K_BYTES + V_BYTES;
+    static constexpr int CPT = kBN * D * ES / 16 / 256;  // 16-byte chunks per thread per tile (K or V)
+    static constexpr int CR = D * ES / 16;               // chunks per row-major row
+    static constexpr int CRK = kBN * ES / 16;            // chunks per K^T row
+    static constexpr int EPC = 16 / ES;                  // elements per chunk
+};
+
+template <typename T, int D, int MT, bool KT>
+__global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
+    using G = TileGeom<T, D, KT>;
+    constexpr int ES = G::ES;
+    constexpr int BM = 128 * MT;
+    constexpr int KS = D / 16;  // contraction steps of the score product
+    constexpr int DT = D / 32;  // 32-row tiles of O^T
+    constexpr int NT = kBN / 32;
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    __shared__ SegPlan s_plan[SPLAT_MAX_SEGMENTS];
+    __shared__ SegPtrs s_seg[SPLAT_MAX_SEGMENTS];  // indexable copy of the segment pointers
+    __shared__ PlanScratch s_ps;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lm = lane & 31, g = lane >> 5;
+
+    const int logical = xcd_remap(blockIdx.x, gridDim.x);
+    if (logical >= p.total) return;
+    const int bh = logical / p.n_row_blocks;
+    // later row blocks of causal patterns carry the most keys: hand them out first
+    const int rb = p.n_row_blocks - 1 - (logical % p.n_row_blocks);
+    const int b = bh / p.H, h = bh % p.H;
+    const int r0 = rb * BM;
+    const int L = p.L;
+
+    const T* qb = (const T*)p.q + b * p.q_sb + h * p.q_sh;
+    const T* kb = (const T*)p.k + b * p.k_sb + h * p.k_sh;
+    const T* vb = (const T*)p.v + b * p.v_sb + h * p.v_sh;
+    T* ob = (T*)p.o + b * p.o_sb + h * p.o_sh;
+
+    // ---- plan: per segment, the column range and step of this row block ------------------------
+    if (tid == 0) {
+#pragma unroll
+        for (int k = 0; k < SPLAT_MAX_SEGMENTS; ++k) s_seg[k] = p.seg[k];
+    }
+    __syncthreads();
+    plan_segments<BM>(s_seg, p.n_seg, r0, L, !KT, s_plan, &s_ps, tid);
+
+    int total_tiles = 0;
+    for (int sg = 0; sg < p.n_seg; ++sg) total_tiles += s_plan[sg].n_tiles;
+
+    // ---- Q fragments (B operand of S^T), resident for the whole kernel --------------------------
+    Frag<T> qf[MT][KS];
+    int my_row[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        my_row[mt] = r0 + (wave * MT + mt) * 32 + lm;
+        const T* qr = qb + (int64_t)min(my_row[mt], L - 1) * p.q_sl;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qf[mt][ks] = global_frag<T>(qr + 16 * ks + 8 * g);
+    }
+
+    f32x16 o_acc[MT][DT];
+    float m_run[MT], l_run[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        m_run[mt] = kNegBigA;
+        l_run[mt] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) o_acc[mt][dt][j] = 0.f;
+    }
+
+    // ---- tile walker -----------------------------------------------------------------------------
+    u32x4 kreg[G::CPT], vreg[G::CPT];
+
+#define SPLAT_GLOAD(sg_, tile_)                                                                          \
+    {                                                                                                    \
+        const SegPlan pl = s_plan[sg_];                                                                  \
+        const int j0_ = (tile_) * kBN;                                                                   \
+        _Pragma("unroll") for (int i = 0; i < G::CPT; ++i) {                                             \
+            const int idx = tid + 256 * i;                                                               \
+            {                                                                                            \
+                const int row = idx / G::CR, cc = idx % G::CR;                                           \
+                const int n = min(max(pl.c0 + pl.cs * (j0_ + row), 0), L - 1);                           \
+                vreg[i] = *reinterpret_cast<const u32x4*>(vb + (int64_t)n * p.v_sl + cc * G::EPC);       \
+            }                                                                                            \
+            if constexpr (KT) {                                                                          \
+                const int drow = idx / G::CRK, cc = idx % G::CRK;                                        \
+                const int c = min(pl.c0 + j0_ + cc * G::EPC, L - G::EPC);                                \
+                kreg[i] = *reinterpret_cast<const u32x4*>(kb + (int64_t)drow * p.k_sd + c);              \
+            } else {                                                                                     \
+                const int row = idx / G::CR, cc = idx % G::CR;                                           \
+                const int n = min(max(pl.c0 + pl.cs * (j0_ + row), 0), L - 1);                           \
+                kreg[i] = *reinterpret_cast<const u32x4*>(kb + (int64_t)n * p.k_sl + cc * G::EPC);       \
+            }                                                                                            \
+        }                                                                                                \
+    }
+#define SPLAT_LSTORE(stage_)                                                                             \
+    {                                                                                                    \
+        char* ks_w = smem + (stage_) * G::STAGE;                                                         \
+        char* vs_w = ks_w + G::K_BYTES;                                                                  \
+        _Pragma("unroll") for (int i = 0; i < G::CPT; ++i) {                                             \
+            const int idx = tid + 256 * i;                                                               \
+            {                                                                                            \
+                const int row = idx / G::CR, cc = idx % G::CR;                                           \
+                *reinterpret_cast<u32x4*>(vs_w + row * G::V_ROW + cc * 16) = vreg[i];                    \
+            }                                                                                            \
+            if constexpr (KT) {                                                                          \
+                const int drow = idx / G::CRK, cc = idx % G::CRK;                                        \
+                *reinterpret_cast<u32x4*>(ks_w + drow * G::K_ROW + cc * 16) = kreg[i];                   \
+            } else {                                                                                     \
+                const int row = idx / G::CR, cc = idx % G::CR;                                           \
+                *reinterpret_cast<u32x4*>(ks_w + row * G::K_ROW + cc * 16) = kreg[i];                    \
+            }                                                                                            \
+        }                                                                                                \
+    }
+
+    // position of the tile being prefetched
+    int pf_seg = 0, pf_tile = 0;
+    auto pf_normalise = [&]() {
+        while (pf_seg < p.n_seg && pf_tile >= s_plan[pf_seg].n_tiles) {
+            ++pf_seg;
+            pf_tile = 0;
+        }
+    };
+    pf_normalise();
+    if (total_tiles > 0) {
+        SPLAT_GLOAD(pf_seg, pf_tile);
+        SPLAT_LSTORE(0);
+        ++pf_tile;
+        pf_normalise();
+    }
+    __syncthreads();
+
+    // per-lane row maps of the segment being computed
+    int cur_seg = -1, cur_tile = 0;
+    RowWin win[MT];
+    int w_lo_min = 0, w_lo_max = 0, w_hi_min = 0, w_hi_max = 0;
+    SegPlan cpl = {0, 1, 0, 1};
+
+    for (int it = 0; it < total_tiles; ++it) {
+        // advance the compute position; reload row maps on a segment change
+        if (cur_seg < 0 || cur_tile >= cpl.n_tiles) {
+            do {
+                ++cur_seg;
+            } while (s_plan[cur_seg].n_tiles == 0);
+            cur_tile = 0;
+            cpl = s_plan[cur_seg];
+            int lmin = 0x3fffffff, lmax = -0x3fffffff, hmin = 0x3fffffff, hmax = -0x3fffffff;
+            bool any_empty = false;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                RowMap m = {0, 1, 0};
+                if (my_row[mt] < L) m = load_row_map(s_seg[cur_seg], my_row[mt]);
+                win[mt] = make_row_win(m, cpl);
+                if (win[mt].cnt <= 0) {
+                    any_empty = true;
+                } else {
+                    lmin = min(lmin, win[mt].lo);
+                    lmax = max(lmax, win[mt].lo);
+                    hmin = min(hmin, win[mt].lo + win[mt].cnt);
+                    hmax = max(hmax, win[mt].lo + win[mt].cnt);
+                }
+            }
+            w_lo_min = wave_min_i(lmin);
+            w_lo_max = wave_max_i(lmax);
+            w_hi_min = wave_min_i(hmin);
+            w_hi_max = wave_max_i(hmax);
+            if (__any(any_empty) || !cpl.uniform) w_lo_max = 0x3fffffff;  // such a wave never drops the mask
+        }
+        const int j0 = cur_tile * kBN;
+        ++cur_tile;
+
+        const bool more = (it + 1 < total_tiles);
+        if (more) SPLAT_GLOAD(pf_seg, pf_tile);
+
+        const char* ks_l = smem + (it & 1) * G::STAGE;
+        const char* vs_l = ks_l + G::K_BYTES;
+
+        const bool skip = (j0 + kBN <= w_lo_min) || (j0 >= w_hi_max);
+        if (!skip) {
+            const bool full = (j0 >= w_lo_max) && (j0 + kBN <= w_hi_min);
+
+            // ---- S^T = K . Q^T ----
+            f32x16 s_acc[MT][NT];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) s_acc[mt][nt][j] = 0.f;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    Frag<T> kf;
+                    if constexpr (KT) {
+                        kf = lds_frag_cols<T>(ks_l, G::K_ROW, 16 * ks + 8 * g, 16 * ks + 8 * g + 4, 32 * nt, lane);
+                    } else {
+                        kf = lds_frag_rowmajor<T>(ks_l + (32 * nt + lm) * G::K_ROW + (16 * ks + 8 * g) * ES);
+                    }
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) mma32(s_acc[mt][nt], kf, qf[mt][ks]);
+                }
+            }
+
+            // ---- mask, online softmax ----
+            Frag<T> pf[MT][NT][2];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                float mx = kNegBigA;
+                if (full) {
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                        for (int j = 0; j < 16; ++j) mx = fmaxf(mx, s_acc[mt][nt][j]);
+                } else {
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                        for (int j = 0; j < 16; ++j) {
+                            const bool ok = win_live(win[mt], j0 + 32 * nt + acc_row(j, g));
+                            const float sv = ok ? s_acc[mt][nt][j] : kNegBigA;
+                            s_acc[mt][nt][j] = sv;
+                            mx = fmaxf(mx, sv);
+                        }
+                }
+                mx = fmaxf(mx, __shfl_xor(mx, 32));
+                const float m_new = fmaxf(m_run[mt], mx);
+                const float alpha = fast_exp2((m_run[mt] - m_new) * p.scale_log2e);
+                const float mb = m_new * p.scale_log2e;
+                m_run[mt] = m_new;
+                float rs = 0.f;
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) {
+                        float pv = fast_exp2(fmaf(s_acc[mt][nt][j], p.scale_log2e, -mb));
+                        if (!full) pv = (s_acc[mt][nt][j] > 0.5f * kNegBigA) ? pv : 0.f;
+                        rs += pv;
+                        pf[mt][nt][j >> 3].v[j & 7] = (T)pv;
+                    }
+                l_run[mt] = l_run[mt] * alpha + rs;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) o_acc[mt][dt][j] *= alpha;
+            }
+
+            // ---- O^T += V^T . P^T ----
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) {
+                        const int rbase = 32 * nt + 16 * t + 4 * g;
+                        Frag<T> vf = lds_frag_cols<T>(vs_l, G::V_ROW, rbase, rbase + 8, 32 * dt, lane);
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) mma32(o_acc[mt][dt], vf, pf[mt][nt][t]);
+                    }
+                }
+            }
+        }
+
+        if (more) {
+            SPLAT_LSTORE((it + 1) & 1);
+            ++pf_tile;
+            pf_normalise();
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue: O = O^T / l, one 4-element run per (row, register quad) ------------------------
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const float l_tot = l_run[mt] + __shfl_xor(l_run[mt], 32);
+        const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+        if (my_row[mt] < L) {
+            T* orow = ob + (int64_t)my_row[mt] * p.o_sl;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) {
+                    typedef T vec4 __attribute__((ext_vector_type(4)));
+                    vec4 o;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) o[i] = (T)(o_acc[mt][dt][4 * jj + i] * inv);
+                    *reinterpret_cast<vec4*>(orow + 32 * dt + 8 * jj + 4 * g) = o;
+                }
+        }
+    }
+}
+
+#undef SPLAT_GLOAD
+#undef SPLAT_LSTORE
+
+template <typename T, int D, int MT, bool KT>
+static int launch_attn(const AttnParams& p0, hipStream_t st) {
+    using G = TileGeom<T, D, KT>;
+    AttnParams p = p0;
+    constexpr int BM = 128 * MT;
+    p.n_row_blocks = (p.L + BM - 1) / BM;
+    p.total = p.B * p.H * p.n_row_blocks;
+    const int grid = ((p.total + 7) / 8) * 8;
+    const size_t lds = 2 * (size_t)G::STAGE;
+    auto kern = attn_fwd_kernel<T, D, MT, KT>;
+    static thread_local bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) {
+            set_error("splat_attention_fwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+            return (int)e;
+        }
+        attr_set = true;
+    }
+    kern<<<grid, 256, lds, st>>>(p);
+    return check_launch("splat_attention_fwd");
+}
+
+template <typename T>
+static int dispatch_attn(const AttnParams& p, int d, bool kt, hipStream_t st) {
+    // two 32-row tiles per wavefront when the problem has enough row blocks to fill the chip
+    if constexpr (sizeof(T) == 2) {
+        const bool big = (int64_t)p.B * p.H * ((p.L + 255) / 256) >= 512;
+        if (big) {
+            if (d == 64) return kt ? launch_attn<T, 64, 2, true>(p, st) : launch_attn<T, 64, 2, false>(p, st);
+            return kt ? launch_attn<T, 128, 2, true>(p, st) : launch_attn<T, 128, 2, false>(p, st);
+        }
+    }
+    if (d == 64) return kt ? launch_attn<T, 64, 1, true>(p, st) : launch_attn<T, 64, 1, false>(p, st);
+    return kt ? launch_attn<T, 128, 1, true>(p, st) : launch_attn<T, 128, 1, false>(p, st);
+}
+
+}  // namespace splat
+
+using namespace splat;
+
+extern "C" int splat_attention_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT, int64_t k_sb,
+                                   int64_t k_sh, int64_t k_sd, int64_t k_sl, const void* v, int64_t v_sb, int64_t v_sh,
+                                   int64_t v_sl, void* out, int64_t o_sb, int64_t o_sh, int64_t o_sl,
+                                   const splat_acsr_seg* segs, int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t d,
+                                   float scale, int32_t dtype, void* stream) {
+    if (!q || !kT || !v || !out || !segs) return fail(SPLAT_E_NULL, "splat_attention_fwd: null pointer argument");
+    if (B <= 0 || H <= 0 || L <= 0) return fail(SPLAT_E_SHAPE, "splat_attention_fwd: need B, H, L > 0 (got %d, %d, %d)", B, H, L);
+    if (L > (1 << 23)) return fail(SPLAT_E_SHAPE, "splat_attention_fwd: L is limited to 2^23 (got %d)", L);
+    if (d != 64 && d != 128) return fail(SPLAT_E_UNSUPPORTED, "splat_attention_fwd: head dim must be 64 or 128 (got %d)", d);
+    if (dtype != SPLAT_F32 && dtype != SPLAT_F16 && dtype != SPLAT_BF16)
+        return fail(SPLAT_E_DTYPE, "splat_attention_fwd: unknown dtype %d", dtype);
+    // the running max is taken over unscaled scores, which orders them correctly only for scale >= 0
+    if (!(scale >= 0.f)) return fail(SPLAT_E_UNSUPPORTED, "splat_attention_fwd: scale must be >= 0 (got %g)", (double)scale);
+    const int es = dtype == SPLAT_F32 ? 4 : 2;
+    const int epc = 16 / es;
+    bool kt;
+    if (k_sd == 1 && (k_sl % epc) == 0 && k_sl >= d)
+        kt = false;  // rows of K are contiguous: [.., L, d] memory viewed as [.., d, L]
+    else if (k_sl == 1)
+        kt = true;  // K^T contiguous: [.., d, L] memory
+    else
+        return fail(SPLAT_E_ALIGN, "splat_attention_fwd: kT needs unit stride along d (k_sd == 1) or along keys (k_sl == 1); got k_sd=%lld k_sl=%lld",
+                    (long long)k_sd, (long long)k_sl);
+    if (kt && ((L % epc) != 0 || (k_sd % epc) != 0 || L < epc))
+        return fail(SPLAT_E_ALIGN, "splat_attention_fwd: with K^T contiguous along keys, L and the d-stride must be multiples of %d (got L=%d, k_sd=%lld)",
+                    epc, L, (long long)k_sd);
+    auto mis = [&](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) != 0; };
+    auto bad = [&](int64_t s) { return (s % epc) != 0; };
+    if (mis(q) || mis(kT) || mis(v) || mis(out)) return fail(SPLAT_E_ALIGN, "splat_attention_fwd: q, kT, v and out must be 16-byte aligned");
+    if (bad(q_sb) || bad(q_sh) || bad(q_sl) || bad(k_sb) || bad(k_sh) || bad(v_sb) || bad(v_sh) || bad(v_sl) || bad(o_sb) || bad(o_sh) || bad(o_sl))
+        return fail(SPLAT_E_ALIGN, "splat_attention_fwd: every batch/head/row stride must be a multiple of %d elements (16 bytes)", epc);
+    if (q_sl < d || v_sl < d || o_sl < d) return fail(SPLAT_E_SHAPE, "splat_attention_fwd: row strides must be >= d");
+
+    AttnParams p;
+    p.q = q; p.k = kT; p.v = v; p.o = out;
+    p.q_sb = q_sb; p.q_sh = q_sh; p.q_sl = q_sl;
+    p.k_sb = k_sb; p.k_sh = k_sh; p.k_sd = k_sd; p.k_sl = k_sl;
+    p.v_sb = v_sb; p.v_sh = v_sh; p.v_sl = v_sl;
+    p.o_sb = o_sb; p.o_sh = o_sh; p.o_sl = o_sl;
+    p.B = B; p.H = H; p.L = L;
+    p.scale_log2e = scale * 1.4426950408889634f;
+    p.n_seg = n_seg;
+    if (int rc = fill_segs("splat_attention_fwd", segs, n_seg, p.seg, -1)) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case SPLAT_F32: return dispatch_attn<float>(p, d, kt, st);
+        case SPLAT_F16: return dispatch_attn<f16>(p, d, kt, st);
+        default: return dispatch_attn<bf16>(p, d, kt, st);
+    }
+}

@@ -1,0 +1,210 @@
+// Row softmax over the live slots of compressed [BH, L, T] score rows.
+//
+// One wavefront owns one row.  The row's live slots are read once with 16/32-byte loads (8 elements
+// per lane per step), kept in registers, reduced with wavefront shuffles (max, then sum of
+// exp2((x - max) * log2 e)) and written back once; dead slots (s >= nnz) are neither read as data nor
+// written.  HBM-bound: 2 * live slots * element size bytes per row.  Rows longer than 2048 slots, or
+// whose length is not a multiple of 8, take a three-pass kernel that re-reads the row from cache.
+#include "splat_common.hpp"
+
+namespace splat {
+
+struct SoftmaxSegs {
+    const float* nnz[SPLAT_MAX_SEGMENTS];
+    int off[SPLAT_MAX_SEGMENTS];
+    int n;
+};
+
+struct LiveRanges {
+    int lo[SPLAT_MAX_SEGMENTS], hi[SPLAT_MAX_SEGMENTS];
+    int n;
+    __device__ __forceinline__ void load(const SoftmaxSegs& s, int row, int T) {
+        n = s.n;
+#pragma unroll
+        for (int k = 0; k < SPLAT_MAX_SEGMENTS; ++k) {
+            lo[k] = hi[k] = 0;
+            if (k < s.n) {
+                lo[k] = s.off[k];
+                hi[k] = min(T, s.off[k] + (int)s.nnz[k][row]);
+            }
+        }
+    }
+    __device__ __forceinline__ bool live(int slot) const {
+        bool v = false;
+#pragma unroll
+        for (int k = 0; k < SPLAT_MAX_SEGMENTS; ++k) v |= (k < n) && slot >= lo[k] && slot < hi[k];
+        return v;
+    }
+    // 8-bit liveness of slots [s0, s0+8)
+    __device__ __forceinline__ uint32_t live8(int s0) const {
+        uint32_t m = 0;
+#pragma unroll
+        for (int k = 0; k < SPLAT_MAX_SEGMENTS; ++k) {
+            if (k < n) {
+                int a = max(lo[k], s0) - s0, b = min(hi[k], s0 + 8) - s0;
+                if (b > a) m |= ((1u << b) - 1u) & ~((1u << a) - 1u);
+            }
+        }
+        return m;
+    }
+};
+
+template <typename T>
+struct Vec8 {
+    typedef T type __attribute__((ext_vector_type(8)));
+};
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kNegBig = -1.0e30f;
+
+template <typename Tin, typename Tout, int NCH>
+__global__ __launch_bounds__(256) void softmax_rows_vec(const Tin* __restrict__ x, Tout* __restrict__ y, SoftmaxSegs segs,
+                                                        int64_t n_rows, int L, int T) {
+    typedef typename Vec8<Tin>::type vin;
+    typedef typename Vec8<Tout>::type vout;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= n_rows) return;
+    LiveRanges lr;
+    lr.load(segs, (int)(row % L), T);
+    const Tin* xr = x + row * (int64_t)T;
+    Tout* yr = y + row * (int64_t)T;
+    const int nchunk = T >> 3;
+
+    float v[NCH][8];
+    uint32_t live[NCH];
+    float mx = kNegBig;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int ch = lane + 64 * c;
+        live[c] = (ch < nchunk) ? lr.live8(ch << 3) : 0u;
+        if (live[c]) {
+            vin t = *reinterpret_cast<const vin*>(xr + (ch << 3));
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                v[c][e] = ((live[c] >> e) & 1u) ? (float)t[e] : kNegBig;
+                mx = fmaxf(mx, v[c][e]);
+            }
+        }
+    }
+    mx = wave_max(mx);
+    const float mb = mx * kLog2e;
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        if (live[c]) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float p = ((live[c] >> e) & 1u) ? fast_exp2(fmaf(v[c][e], kLog2e, -mb)) : 0.f;
+                v[c][e] = p;
+                sum += p;
+            }
+        }
+    }
+    sum = wave_sum(sum);
+    const float inv = sum > 0.f ? 1.0f / sum : 0.f;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        if (live[c]) {
+            const int ch = lane + 64 * c;
+            if (live[c] == 0xffu) {
+                vout o;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[e] = (Tout)(v[c][e] * inv);
+                *reinterpret_cast<vout*>(yr + (ch << 3)) = o;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if ((live[c] >> e) & 1u) yr[(ch << 3) + e] = (Tout)(v[c][e] * inv);
+            }
+        }
+    }
+}
+
+template <typename Tin, typename Tout>
+__global__ __launch_bounds__(256) void softmax_rows_any(const Tin* __restrict__ x, Tout* __restrict__ y, SoftmaxSegs segs,
+                                                        int64_t n_rows, int L, int T) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= n_rows) return;
+    LiveRanges lr;
+    lr.load(segs, (int)(row % L), T);
+    const Tin* xr = x + row * (int64_t)T;
+    Tout* yr = y + row * (int64_t)T;
+    float mx = kNegBig;
+    for (int s = lane; s < T; s += 64)
+        if (lr.live(s)) mx = fmaxf(mx, (float)xr[s]);
+    mx = wave_max(mx);
+    const float mb = mx * kLog2e;
+    float sum = 0.f;
+    for (int s = lane; s < T; s += 64)
+        if (lr.live(s)) sum += fast_exp2(fmaf((float)xr[s], kLog2e, -mb));
+    sum = wave_sum(sum);
+    const float inv = sum > 0.f ? 1.0f / sum : 0.f;
+    // in-place safe: every lane rewrites only the slots it reads in this loop
+    for (int s = lane; s < T; s += 64)
+        if (lr.live(s)) yr[s] = (Tout)(fast_exp2(fmaf((float)xr[s], kLog2e, -mb)) * inv);
+}
+
+template <typename Tin, typename Tout>
+static int launch_softmax(const void* x, void* y, const SoftmaxSegs& segs, int64_t n_rows, int L, int T, hipStream_t st) {
+    const unsigned grid = (unsigned)((n_rows + 3) / 4);
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 31) == 0;
+    const Tin* xi = (const Tin*)x;
+    Tout* yo = (Tout*)y;
+    if (aligned && (T & 7) == 0 && T <= 2048) {
+        const int nch = (T / 8 + 63) / 64;
+        if (nch <= 1)
+            softmax_rows_vec<Tin, Tout, 1><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+        else if (nch <= 2)
+            softmax_rows_vec<Tin, Tout, 2><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+        else
+            softmax_rows_vec<Tin, Tout, 4><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+    } else {
+        softmax_rows_any<Tin, Tout><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+    }
+    return check_launch("splat_softmax");
+}
+
+template <typename Tin>
+static int dispatch_out(const void* x, void* y, const SoftmaxSegs& segs, int64_t n_rows, int L, int T, int out_dtype, hipStream_t st) {
+    switch (out_dtype) {
+        case SPLAT_F32: return launch_softmax<Tin, float>(x, y, segs, n_rows, L, T, st);
+        case SPLAT_F16: return launch_softmax<Tin, f16>(x, y, segs, n_rows, L, T, st);
+        case SPLAT_BF16: return launch_softmax<Tin, bf16>(x, y, segs, n_rows, L, T, st);
+    }
+    return fail(SPLAT_E_DTYPE, "splat_softmax: unknown out_dtype %d", out_dtype);
+}
+
+}  // namespace splat
+
+using namespace splat;
+
+extern "C" int splat_softmax(const void* x, void* y, const splat_acsr_seg* segs, int32_t n_seg, int64_t BH, int32_t L,
+                             int32_t T, int32_t in_dtype, int32_t out_dtype, void* stream) {
+    if (!x || !y || !segs) return fail(SPLAT_E_NULL, "splat_softmax: null pointer argument");
+    if (n_seg < 1 || n_seg > SPLAT_MAX_SEGMENTS) return fail(SPLAT_E_SHAPE, "splat_softmax: n_seg must be 1..%d (got %d)", SPLAT_MAX_SEGMENTS, n_seg);
+    if (BH <= 0 || L <= 0 || T <= 0) return fail(SPLAT_E_SHAPE, "splat_softmax: need BH, L, T > 0 (got %lld, %d, %d)", (long long)BH, L, T);
+    if (BH * (int64_t)L > ((int64_t)1 << 33)) return fail(SPLAT_E_SHAPE, "splat_softmax: too many rows");
+    SoftmaxSegs s;
+    s.n = n_seg;
+    for (int k = 0; k < SPLAT_MAX_SEGMENTS; ++k) {
+        s.nnz[k] = nullptr;
+        s.off[k] = 0;
+    }
+    for (int k = 0; k < n_seg; ++k) {
+        if (!segs[k].nnz) return fail(SPLAT_E_NULL, "splat_softmax: segment %d has a null nnz array", k);
+        if (segs[k].slot_offset < 0 || segs[k].slot_offset >= T)
+            return fail(SPLAT_E_SHAPE, "splat_softmax: segment %d slot_offset %d outside [0, T=%d)", k, segs[k].slot_offset, T);
+        s.nnz[k] = segs[k].nnz;
+        s.off[k] = segs[k].slot_offset;
+    }
+    const int64_t n_rows = BH * L;
+    hipStream_t st = (hipStream_t)stream;
+    switch (in_dtype) {
+        case SPLAT_F32: return dispatch_out<float>(x, y, s, n_rows, L, T, out_dtype, st);
+        case SPLAT_F16: return dispatch_out<f16>(x, y, s, n_rows, L, T, out_dtype, st);
+        case SPLAT_BF16: return dispatch_out<bf16>(x, y, s, n_rows, L, T, out_dtype, st);
+    }
+    return fail(SPLAT_E_DTYPE, "splat_softmax: unknown in_dtype %d", in_dtype);
+}

@@ -1,0 +1,194 @@
+// SpMM on ACSR: out[bh, r, :] = sum over live slots s of p[bh, r, off + s] * V[bh, c(r, s), :].
+//
+// A workgroup of 4 wavefronts owns 128 consecutive rows of one (batch, head) and a chunk of up to 128
+// output columns; wavefront w owns rows 32w..32w+31.  Key positions are walked in tiles of 64 (see
+// acsr_plan.hpp).  The V tile is staged row-major in LDS and read as MFMA B operand with the transposing
+// LDS read; the A operand (probabilities) is read straight from the compressed rows: with a uniform
+// plan 8 consecutive positions of a row are 8 consecutive slots, one (possibly unaligned) 16-byte load.
+// Output orientation rows = queries, columns = output features, so stores are contiguous per row.
+// Bound by reading the compressed probabilities (HBM), not by MFMA.
+#include "acsr_plan.hpp"
+
+namespace splat {
+
+struct SpmmParams {
+    const void* p;
+    const void* v;
+    void* out;
+    int64_t v_sb, v_sh, v_sl;
+    int B, H, L, n_keys, n_out, T;
+    int out_dtype;
+    int n_seg;
+    SegPtrs seg[SPLAT_MAX_SEGMENTS];
+    int n_row_blocks, total, n_col_chunks;
+    int v_vec;
+};
+
+template <typename T, int DVT>
+__global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
+    constexpr int ES = sizeof(T);
+    constexpr int BM = 128;
+    constexpr int DVC = 32 * DVT;           // output columns per workgroup
+    constexpr int V_ROW = DVC * ES + 64;    // bytes per LDS row
+    constexpr int EPC = 16 / ES;
+    constexpr int CR = DVC * ES / 16;       // 16-byte chunks per LDS row
+    constexpr int NCHUNK = kBN * CR;        // chunks per tile
+
+    __shared__ __attribute__((aligned(16))) char s_v[V_ROW * kBN];
+    __shared__ SegPlan s_plan[SPLAT_MAX_SEGMENTS];
+    __shared__ SegPtrs s_seg[SPLAT_MAX_SEGMENTS];
+    __shared__ PlanScratch s_ps;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lm = lane & 31, g = lane >> 5;
+
+    const int logical = xcd_remap(blockIdx.x, gridDim.x);
+    if (logical >= p.total) return;
+    const int cchunk = logical % p.n_col_chunks;
+    const int rest = logical / p.n_col_chunks;
+    const int bh = rest / p.n_row_blocks;
+    const int rb = rest % p.n_row_blocks;
+    const int b = bh / p.H, h = bh % p.H;
+    const int r0 = rb * BM;
+    const int L = p.L;
+    const int col0 = cchunk * DVC;
+
+    const T* vb = (const T*)p.v + b * p.v_sb + h * p.v_sh;
+    const T* pb = (const T*)p.p + (int64_t)bh * L * p.T;
+
+    if (tid == 0) {
+#pragma unroll
+        for (int k = 0; k < SPLAT_MAX_SEGMENTS; ++k) s_seg[k] = p.seg[k];
+    }
+    __syncthreads();
+    plan_segments<BM>(s_seg, p.n_seg, r0, L, true, s_plan, &s_ps, tid);
+
+    const int my_row = r0 + 32 * wave + lm;  // A-operand row of this lane
+    const T* prow = pb + (int64_t)min(my_row, L - 1) * p.T;
+
+    f32x16 acc[DVT];
+#pragma unroll
+    for (int dt = 0; dt < DVT; ++dt)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[dt][j] = 0.f;
+
+    for (int sg = 0; sg < p.n_seg; ++sg) {
+        const SegPlan pl = s_plan[sg];
+        if (pl.n_tiles == 0) continue;
+        const int off = s_seg[sg].slot_offset;
+        RowMap m = {0, 1, 0};
+        if (my_row < L) m = load_row_map(s_seg[sg], my_row);
+        const RowWin win = make_row_win(m, pl);
+        int lmin = win.cnt > 0 ? win.lo : 0x3fffffff;
+        int hmax = win.cnt > 0 ? win.lo + win.cnt : -0x3fffffff;
+        lmin = wave_min_i(lmin);
+        hmax = wave_max_i(hmax);
+
+        for (int tile = 0; tile < pl.n_tiles; ++tile) {
+            const int j0 = tile * kBN;
+            __syncthreads();  // previous tile fully consumed
+            for (int idx = tid; idx < NCHUNK; idx += 256) {
+                const int row = idx / CR, cc = idx % CR;
+                const int n = min(max(pl.c0 + pl.cs * (j0 + row), 0), p.n_keys - 1);
+                const T* src = vb + (int64_t)n * p.v_sl;
+                const int c = col0 + cc * EPC;
+                u32x4 val = {0u, 0u, 0u, 0u};
+                if (p.v_vec && c + EPC <= p.n_out) {
+                    val = *reinterpret_cast<const u32x4*>(src + c);
+                } else {
+                    T tmp[EPC];
+#pragma unroll
+                    for (int e = 0; e < EPC; ++e) tmp[e] = (c + e < p.n_out) ? src[c + e] : (T)0.f;
+                    __builtin_memcpy(&val, tmp, 16);
+                }
+                *reinterpret_cast<u32x4*>(s_v + row * V_ROW + cc * 16) = val;
+            }
+            __syncthreads();
+            const bool skip = (j0 + kBN <= lmin) || (j0 >= hmax);  // wavefront-uniform
+            if (skip) continue;
+#pragma unroll
+            for (int t = 0; t < kBN / 16; ++t) {
+                // A fragment: positions jj..jj+7 of this lane's row
+                const int jj = j0 + 16 * t + 8 * g;
+                Frag<T> pf;
+                const int u = jj - win.lo;
+                if (win.lin == 1 && u >= 0 && u + 8 <= win.cnt) {
+                    __builtin_memcpy(&pf.v, prow + off + u, 8 * ES);  // any alignment
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) pf.v[e] = win_live(win, jj + e) ? prow[off + win_slot(win, jj + e)] : (T)0.f;
+                }
+#pragma unroll
+                for (int dt = 0; dt < DVT; ++dt) {
+                    Frag<T> vf = lds_frag_cols<T>(s_v, V_ROW, 16 * t + 8 * g, 16 * t + 8 * g + 4, 32 * dt, lane);
+                    mma32(acc[dt], pf, vf);
+                }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const int r = r0 + 32 * wave + acc_row(j, g);
+        if (r < L) {
+            const int64_t base = ((int64_t)bh * L + r) * p.n_out;
+#pragma unroll
+            for (int dt = 0; dt < DVT; ++dt) {
+                const int c = col0 + 32 * dt + lm;
+                if (c < p.n_out) store_as(p.out, base + c, acc[dt][j], p.out_dtype);
+            }
+        }
+    }
+}
+
+template <typename T>
+static int launch_spmm(SpmmParams p, hipStream_t st) {
+    p.n_row_blocks = (p.L + 127) / 128;
+    const int dvt = p.n_out > 64 ? 4 : (p.n_out > 32 ? 2 : 1);
+    p.n_col_chunks = (p.n_out + 32 * dvt - 1) / (32 * dvt);
+    const int64_t total = (int64_t)p.B * p.H * p.n_row_blocks * p.n_col_chunks;
+    if (total > 0x7ffffff0) return fail(SPLAT_E_SHAPE, "splat_spmm: problem too large for one launch");
+    p.total = (int)total;
+    const int grid = ((p.total + 7) / 8) * 8;
+    if (dvt == 4)
+        spmm_kernel<T, 4><<<grid, 256, 0, st>>>(p);
+    else if (dvt == 2)
+        spmm_kernel<T, 2><<<grid, 256, 0, st>>>(p);
+    else
+        spmm_kernel<T, 1><<<grid, 256, 0, st>>>(p);
+    return check_launch("splat_spmm");
+}
+
+}  // namespace splat
+
+using namespace splat;
+
+extern "C" int splat_spmm(const void* pp, const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sl, void* out,
+                          const splat_acsr_seg* segs, int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t n_keys,
+                          int32_t n_out, int32_t T, int32_t in_dtype, int32_t out_dtype, void* stream) {
+    if (!pp || !v || !out || !segs) return fail(SPLAT_E_NULL, "splat_spmm: null pointer argument");
+    if (B <= 0 || H <= 0 || L <= 0 || n_keys <= 0 || n_out <= 0 || T <= 0)
+        return fail(SPLAT_E_SHAPE, "splat_spmm: need B, H, L, n_keys, n_out, T > 0 (got %d, %d, %d, %d, %d, %d)", B, H, L, n_keys, n_out, T);
+    if (L > (1 << 23) || n_keys > (1 << 23)) return fail(SPLAT_E_SHAPE, "splat_spmm: L and n_keys are limited to 2^23");
+    if (out_dtype != SPLAT_F32 && out_dtype != SPLAT_F16 && out_dtype != SPLAT_BF16)
+        return fail(SPLAT_E_DTYPE, "splat_spmm: unknown out_dtype %d", out_dtype);
+    if (in_dtype != SPLAT_F32 && in_dtype != SPLAT_F16 && in_dtype != SPLAT_BF16)
+        return fail(SPLAT_E_DTYPE, "splat_spmm: unknown in_dtype %d", in_dtype);
+    if (v_sl < n_out) return fail(SPLAT_E_SHAPE, "splat_spmm: v row stride %lld < n_out %d", (long long)v_sl, n_out);
+    SpmmParams p;
+    p.p = pp; p.v = v; p.out = out;
+    p.v_sb = v_sb; p.v_sh = v_sh; p.v_sl = v_sl;
+    p.B = B; p.H = H; p.L = L; p.n_keys = n_keys; p.n_out = n_out; p.T = T;
+    p.out_dtype = out_dtype;
+    p.n_seg = n_seg;
+    if (int rc = fill_segs("splat_spmm", segs, n_seg, p.seg, T)) return rc;
+    const int es = in_dtype == SPLAT_F32 ? 4 : 2;
+    const int epc = 16 / es;
+    p.v_vec = ((reinterpret_cast<uintptr_t>(v) & 15) == 0 && v_sb % epc == 0 && v_sh % epc == 0 && v_sl % epc == 0) ? 1 : 0;
+    hipStream_t st = (hipStream_t)stream;
+    switch (in_dtype) {
+        case SPLAT_F32: return launch_spmm<float>(p, st);
+        case SPLAT_F16: return launch_spmm<f16>(p, st);
+        default: return launch_spmm<bf16>(p, st);
+    }
+}
