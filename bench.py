@@ -1,0 +1,219 @@
+#!/usr/bin/env python3
+"""Benchmark of the ACSR sparse-attention forward on one MI355X.
+
+A step is one fused forward (splat_attention_fwd) over BASELINE config 5: B=4, H=16, L=16384, d=128,
+bf16, causal window 512, scale 1/sqrt(d), seeded synthetic N(0,1) inputs already resident in HBM, K handed
+over as ``k.transpose(2, 3)`` (a view of row-major K; the K^T-contiguous layout is timed as an extra).
+Prints ONE JSON line.  `value` counts only nonzero (live) FLOPs: 4 * d * nnz * B * H.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "triton-fun_amd", "SPLAT")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16
+HBM_PEAK_GBPS = 8000.0
+# HBM bytes one fused launch moves at config 5, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
+# copy kernel of known size (see profiles/attention_fwd_cfg5_pmc.md); None until measured.
+FUSED_TRAFFIC_BYTES = None
+
+
+def causal_window_nnz(L: int, w: int) -> int:
+    return w * L - w * (w - 1) // 2
+
+
+def time_launches(fn, steps: int, warmup: int):
+    """Whole-region wall time (synchronise on both sides) and per-launch HIP-event durations on the
+    current stream, in ms."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    per = sorted(a.elapsed_time(b) for a, b in evs)
+    return wall_ms, per
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the host baseline")
+    ap.add_argument("--no-extras", action="store_true", help="skip the unfused kernels and the ACSR build")
+    ap.add_argument("--cpu-heads", type=int, default=16, help="(batch, head) pairs the host baseline computes")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 1 GiB device-to-device copy, the known-size kernel that HBM counters are scaled by")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the path shards over batch*heads with no exchange, and this build "
+              "has no multi-GPU launcher (--gpus must be 1)", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    import acsr_helpers as A
+    import r_softmax
+    import r_sddmm
+    import r_spmm
+    from r_attention import RegularAttention, attention_launcher
+    from oracle import splat_oracle as O  # cpu_baseline only
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a HIP device", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+
+    B, H, L, d, w = 4, 16, 16384, 128, 512
+    dtype = torch.bfloat16
+    scale = d ** -0.5
+    q, k, v = O.make_inputs(1005, B, H, L, d, dtype)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    kT_view = kd.transpose(2, 3)
+
+    t0 = time.perf_counter()
+    attn = RegularAttention(B, L, H, d, A.causal_windowed_pattern(L, w - 1), 16, 16, dev, dtype, scale=scale)
+    torch.cuda.synchronize()
+    setup_ms = (time.perf_counter() - t0) * 1e3
+
+    nnz = causal_window_nnz(L, w)
+    flops = 4.0 * d * nnz * B * H
+    io_bytes = 4.0 * B * H * L * d * 2
+
+    step = lambda: attn([qd, kT_view, vd])
+    wall_ms, per = time_launches(step, args.steps, args.warmup)
+    ms_per_step = wall_ms / args.steps
+    kern_ms = sum(per) / len(per)
+    tflops = flops / (ms_per_step * 1e-3) / 1e12
+    kern_tflops = flops / (kern_ms * 1e-3) / 1e12
+
+    out = {
+        "metric": "sparse-attn fwd ms + nnz-TFLOP/s (% MFMA peak) on 1 MI355X; softmax HBM GB/s",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s (nonzero FLOPs only, fused forward)",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic: seeded N(0,1) q/k/v (torch.Generator cpu seed 1005), resident in HBM",
+        "config": {"workload": "config 5: fused ACSR attention fwd, B=4 H=16 L=16384 d=128 bf16, causal window 512, "
+                               "scale 1/sqrt(d), K passed as k.transpose(2,3)",
+                   "B": B, "H": H, "L": L, "d": d, "window": w, "nnz_per_head": nnz},
+        "roofline": {"bound": "mfma", "achieved": round(kern_tflops, 2), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(kern_tflops / MFMA_PEAK_TFLOPS, 4), "traffic": FUSED_TRAFFIC_BYTES,
+                     "kernel": "attn_fwd_kernel<bf16,128,2,false>", "kernel_ms_avg": round(kern_ms, 4),
+                     "kernel_ms_min": round(per[0], 4), "algorithmic_flops": flops, "algorithmic_bytes": io_bytes,
+                     "hbm_frac_at_algorithmic_bytes": round(io_bytes / (kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
+        "fwd_ms": round(kern_ms, 4),
+        "pct_mfma_peak": round(100.0 * kern_tflops / MFMA_PEAK_TFLOPS, 2),
+        "acsr_setup_ms": round(setup_ms, 2),
+    }
+
+    extras = {}
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    if not args.no_extras:
+        # the literal reference layout: K^T contiguous [B, H, d, L]
+        kT_c = kT_view.contiguous()
+        _, per_c = time_launches(lambda: attn([qd, kT_c, vd]), max(5, args.steps // 2), 3)
+        ms_c = sum(per_c) / len(per_c)
+        extras["fused_kT_contiguous"] = {"ms": round(ms_c, 4), "tflops_nnz": round(flops / ms_c / 1e9, 2)}
+        del kT_c
+
+        # ACSR build on the config-5 mask (L*L bytes read once)
+        mask = A.causal_windowed_pattern(L, w - 1).device_mask(dev)
+
+        def build():
+            A._MASK_CACHE.clear()
+            A.create_acsr(mask, 16, dev)
+        _, per_b = time_launches(build, 10, 2)
+        ms_b = sum(per_b) / len(per_b)
+        extras["acsr_build_cfg5"] = {"ms_incl_readback": round(ms_b, 4), "mask_bytes": L * L,
+                                     "gbps": round(L * L / ms_b / 1e6, 1)}
+        del mask
+        A._MASK_CACHE.clear()
+
+        # unfused kernels at config 4 (dilated, B=2 H=32 L=8192 d=128 bf16, T=512): softmax GB/s is the metric's second half
+        B4, H4, L4, d4 = 2, 32, 8192, 128
+        q4, k4, v4 = O.make_inputs(1004, B4, H4, L4, d4, dtype)
+        q4, k4, v4 = q4.to(dev), k4.to(dev), v4.to(dev)
+        pat4 = A.dilated_pattern(L4, 512, 2)
+        acsr = A.create_acsr(pat4, 16, dev)
+        T4 = acsr[5]
+        nnz4 = float(acsr[4].sum().item())
+        s_buf = torch.empty(B4, H4, L4, T4, dtype=dtype, device=dev)
+        p_buf = torch.empty_like(s_buf)
+        o_buf = torch.empty(B4, H4, L4, d4, dtype=dtype, device=dev)
+        k4T = k4.transpose(2, 3)
+        run_sddmm = lambda: r_sddmm.rsddmm_launcher(q4, k4T, s_buf, acsr[0], acsr[1], acsr[2], acsr[3], T4, acsr[4], (1, 1),
+                                                    None, None, 16, 16, scale=d4 ** -0.5)
+        run_soft = lambda: r_softmax.rsoftmax_launcher(s_buf, p_buf, acsr[0], acsr[1], acsr[2], acsr[3], T4, 512, acsr[4],
+                                                       (1, 1), 16)
+        run_spmm = lambda: r_spmm.rspmm_launcher(p_buf, v4, o_buf, acsr[0], acsr[1], acsr[2], acsr[3], acsr[6], acsr[7],
+                                                 T4, acsr[4], (1, 1, 1), 16, 16)
+        for name, fn, byt, fl in (
+                ("sddmm_cfg4", run_sddmm, (2 * B4 * H4 * L4 * d4 + nnz4 * B4 * H4) * 2, 2 * d4 * nnz4 * B4 * H4),
+                ("softmax_cfg4", run_soft, 2 * nnz4 * B4 * H4 * 2, 0.0),
+                ("spmm_cfg4", run_spmm, (2 * B4 * H4 * L4 * d4 + nnz4 * B4 * H4) * 2, 2 * d4 * nnz4 * B4 * H4)):
+            _, pr = time_launches(fn, 20, 5)
+            ms = sum(pr) / len(pr)
+            extras[name] = {"ms": round(ms, 4), "gbps_algorithmic": round(byt / ms / 1e6, 1),
+                            "hbm_frac": round(byt / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+            if fl:
+                extras[name]["tflops_nnz"] = round(fl / ms / 1e9, 2)
+        out["softmax_gbps"] = extras["softmax_cfg4"]["gbps_algorithmic"]
+        del s_buf, p_buf, o_buf, q4, k4, v4
+    out["extras"] = extras
+
+    if not args.no_cpu:
+        # the reference's dense masked path (einsum of r_sddmm.py:186-188, masked softmax, matmul) in fp32 on the
+        # host cores, on `cpu_heads` (batch, head) pairs of the same workload; nonzero FLOPs counted as above
+        n = max(1, args.cpu_heads)
+        ii = np.arange(L)
+        mask_rows = lambda a, c: (ii[a:c, None] >= ii[None, :]) & (ii[a:c, None] - (w - 1) <= ii[None, :])
+        qs, ks, vs = q.reshape(B * H, 1, L, d)[:n], k.reshape(B * H, 1, L, d)[:n], v.reshape(B * H, 1, L, d)[:n]
+        t0 = time.perf_counter()
+        ref = O.dense_masked_attention_chunked(qs.transpose(0, 1), ks.transpose(0, 1).transpose(2, 3), vs.transpose(0, 1),
+                                               mask_rows, scale)
+        cpu_s = time.perf_counter() - t0
+        got = attn([qd, kT_view, vd]).float().reshape(B * H, L, d)[:n].cpu()
+        err = float((got - ref[0]).abs().max())
+        out["cpu_baseline"] = {"value": round(4.0 * d * nnz * n / cpu_s / 1e12, 5), "unit": out["unit"],
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"{n} of {B * H} (batch, head) pairs of config 5, dense fp32 masked attention "
+                                         f"in PyTorch on the host, {cpu_s:.1f} s",
+                               "max_abs_err_gpu_vs_cpu": round(err, 5)}
+
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

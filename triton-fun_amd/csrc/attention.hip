@@ -45,17 +45,76 @@ struct AttnParams {
 template <typename T, int D, bool KT>
 struct TileGeom {
     static constexpr int ES = sizeof(T);
-    static constexpr int K_ROW = KT ? (kBN * ES + 64) : (D * ES + 16);  // bytes per LDS row of the K tile
+    static constexpr int EPC = 16 / ES;                       // elements per 16-byte chunk
+    static constexpr int K_ROWB = KT ? kBN * ES : D * ES;     // bytes per LDS row of the K tile (no padding)
     static constexpr int K_ROWS = KT ? D : kBN;
-    static constexpr int K_BYTES = K_ROW * K_ROWS;
-    static constexpr int V_ROW = D * ES + 64;
-    static constexpr int V_BYTES = V_ROW * kBN;
+    static constexpr int V_ROWB = D * ES;
+    static constexpr int K_BYTES = K_ROWB * K_ROWS;
+    static constexpr int V_BYTES = V_ROWB * kBN;
     static constexpr int STAGE = K_BYTES + V_BYTES;
-    static constexpr int CPT = kBN * D * ES / 16 / 256;  // 16-byte chunks per thread per tile (K or V)
-    static constexpr int CR = D * ES / 16;               // chunks per row-major row
-    static constexpr int CRK = kBN * ES / 16;            // chunks per K^T row
-    static constexpr int EPC = 16 / ES;                  // elements per chunk
 };
+
+// XOR swizzle of the 16-byte chunk index of a row-major LDS tile with ROWB-byte rows, chosen so that 16
+// lanes reading the same logical chunk of 16 consecutive rows hit 16 different bank groups.
+template <int ROWB>
+__device__ __forceinline__ constexpr int swz(int row) {
+    constexpr int CPR = ROWB / 16;
+    constexpr int CH = CPR < 16 ? CPR : 16;
+    constexpr int RPB = ROWB >= 256 ? 1 : 256 / ROWB;
+    return (row / RPB) & (CH - 1);
+}
+template <int ROWB, bool SWZ>
+__device__ __forceinline__ int lds_off(int row, int byte_col) {
+    if constexpr (SWZ)
+        return row * ROWB + ((((byte_col >> 4) ^ swz<ROWB>(row)) << 4) | (byte_col & 15));
+    else
+        return row * ROWB + byte_col;
+}
+
+typedef __attribute__((address_space(1))) const void gptr_t;
+typedef __attribute__((address_space(3))) void lptr_t;
+
+// One wavefront-wide 1 KiB copy global -> LDS without passing through registers: lane i's 16 bytes land at
+// lds_block + 16*i (lds_block must be wavefront-uniform).
+__device__ __forceinline__ void dma16(const void* src, char* lds_block) {
+    __builtin_amdgcn_global_load_lds((gptr_t*)src, (lptr_t*)lds_block, 16, 0, 0);
+}
+__device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// Copy a ROWS x ROWB-byte tile into LDS; row r comes from row_ptr(r) (16-byte aligned, ROWB readable bytes).
+// Each wavefront issues ROWS*ROWB/4096 instructions of 1 KiB.
+template <typename T, int ROWB, int ROWS, bool SWZ, typename RowPtr>
+__device__ __forceinline__ void dma_tile(char* tile, int wave, int lane, RowPtr row_ptr) {
+    constexpr int NI = ROWS * ROWB / 1024;  // wavefront instructions per tile
+    constexpr int CPR = ROWB / 16;          // chunks per row
+    static_assert(NI % 4 == 0 && (1024 % ROWB == 0 || ROWB % 1024 == 0), "tile shape");
+#pragma unroll
+    for (int i = 0; i < NI / 4; ++i) {
+        const int q = wave + 4 * i;
+        const int flat = q * 64 + lane;  // chunk position in the tile
+        const int row = flat / CPR, pc = flat % CPR;
+        const int c = SWZ ? (pc ^ swz<ROWB>(row)) : pc;
+        dma16(reinterpret_cast<const char*>(row_ptr(row)) + c * 16, tile + q * 1024);
+    }
+}
+
+// K fragment (8 consecutive contraction values of row `row`) from a swizzled row-major tile.
+template <typename T, int ROWB>
+__device__ __forceinline__ Frag<T> lds_frag_row_swz(const char* tile, int row, int elem_col) {
+    Frag<T> f;
+    if constexpr (sizeof(T) == 2) {
+        u32x4 r = *reinterpret_cast<const u32x4*>(tile + lds_off<ROWB, true>(row, elem_col * 2));
+        f.v = __builtin_bit_cast(typename Frag<T>::vec, r);
+    } else {
+        u32x4 r0 = *reinterpret_cast<const u32x4*>(tile + lds_off<ROWB, true>(row, elem_col * 4));
+        u32x4 r1 = *reinterpret_cast<const u32x4*>(tile + lds_off<ROWB, true>(row, elem_col * 4 + 16));
+        u32x8 r = __builtin_shufflevector(r0, r1, 0, 1, 2, 3, 4, 5, 6, 7);
+        f.v = __builtin_bit_cast(typename Frag<T>::vec, r);
+    }
+    return f;
+}
+
+constexpr float kRescaleThreshold = 8.0f;  // in log2 units: exponentials stay below 2^8 before the reference moves
 
 template <typename T, int D, int MT, bool KT>
 __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
@@ -66,7 +125,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
     constexpr int DT = D / 32;  // 32-row tiles of O^T
     constexpr int NT = kBN / 32;
 
-    extern __shared__ __attribute__((aligned(16))) char smem[];
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
     __shared__ SegPlan s_plan[SPLAT_MAX_SEGMENTS];
     __shared__ SegPtrs s_seg[SPLAT_MAX_SEGMENTS];  // indexable copy of the segment pointers
     __shared__ PlanScratch s_ps;
@@ -99,6 +158,45 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
     int total_tiles = 0;
     for (int sg = 0; sg < p.n_seg; ++sg) total_tiles += s_plan[sg].n_tiles;
 
+    // ---- tile walker: asynchronous global -> LDS copies of tile (sg, tile) into a stage ----------
+    auto issue_tile = [&](int sg, int tile, int stage) {
+        const SegPlan pl = s_plan[sg];
+        const int j0 = tile * kBN;
+        char* ks_w = smem + stage * G::STAGE;
+        char* vs_w = ks_w + G::K_BYTES;
+        auto key_row = [&](int row) { return min(max(pl.c0 + pl.cs * (j0 + row), 0), L - 1); };
+        dma_tile<T, G::V_ROWB, kBN, false>(vs_w, wave, lane, [&](int row) { return vb + (int64_t)key_row(row) * p.v_sl; });
+        if constexpr (KT) {
+            // rows = contraction index, 64 consecutive keys per row (dense walk); a chunk that would run past
+            // the last key is replaced by the last whole chunk (those positions are never live)
+            constexpr int CPR = G::K_ROWB / 16;
+#pragma unroll
+            for (int i = 0; i < G::K_ROWS * G::K_ROWB / 4096; ++i) {
+                const int q = wave + 4 * i;
+                const int flat = q * 64 + lane;
+                const int row = flat / CPR, pc = flat % CPR;
+                const int c = min(pl.c0 + j0 + pc * G::EPC, L - G::EPC);
+                dma16(kb + (int64_t)row * p.k_sd + c, ks_w + q * 1024);
+            }
+        } else {
+            dma_tile<T, G::K_ROWB, kBN, true>(ks_w, wave, lane, [&](int row) { return kb + (int64_t)key_row(row) * p.k_sl; });
+        }
+    };
+
+    int pf_seg = 0, pf_tile = 0;  // position of the next tile to fetch
+    auto pf_normalise = [&]() {
+        while (pf_seg < p.n_seg && pf_tile >= s_plan[pf_seg].n_tiles) {
+            ++pf_seg;
+            pf_tile = 0;
+        }
+    };
+    pf_normalise();
+    if (total_tiles > 0) {
+        issue_tile(pf_seg, pf_tile, 0);
+        ++pf_tile;
+        pf_normalise();
+    }
+
     // ---- Q fragments (B operand of S^T), resident for the whole kernel --------------------------
     Frag<T> qf[MT][KS];
     int my_row[MT];
@@ -111,10 +209,10 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
     }
 
     f32x16 o_acc[MT][DT];
-    float m_run[MT], l_run[MT];
+    float m_ref[MT], l_run[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-        m_run[mt] = kNegBigA;
+        m_ref[mt] = kNegBigA;
         l_run[mt] = 0.f;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
@@ -122,66 +220,17 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
             for (int j = 0; j < 16; ++j) o_acc[mt][dt][j] = 0.f;
     }
 
-    // ---- tile walker -----------------------------------------------------------------------------
-    u32x4 kreg[G::CPT], vreg[G::CPT];
+    // lane-dependent parts of the LDS read addresses (stage base and tile constants are added per read)
+    int k_off[KS];  // row-major K: (row lm, logical chunk of step ks) after swizzling
+    if constexpr (!KT) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) k_off[ks] = lds_off<G::K_ROWB, true>(lm, (16 * ks + 8 * g) * ES);
+    }
+    // transposing reads: lane s of a 16-lane block addresses row s/4, 8 bytes at element column 16*(block%2) + 4*(s%4)
+    const int tr_row = (lane & 15) >> 2;
+    const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
-#define SPLAT_GLOAD(sg_, tile_)                                                                          \
-    {                                                                                                    \
-        const SegPlan pl = s_plan[sg_];                                                                  \
-        const int j0_ = (tile_) * kBN;                                                                   \
-        _Pragma("unroll") for (int i = 0; i < G::CPT; ++i) {                                             \
-            const int idx = tid + 256 * i;                                                               \
-            {                                                                                            \
-                const int row = idx / G::CR, cc = idx % G::CR;                                           \
-                const int n = min(max(pl.c0 + pl.cs * (j0_ + row), 0), L - 1);                           \
-                vreg[i] = *reinterpret_cast<const u32x4*>(vb + (int64_t)n * p.v_sl + cc * G::EPC);       \
-            }                                                                                            \
-            if constexpr (KT) {                                                                          \
-                const int drow = idx / G::CRK, cc = idx % G::CRK;                                        \
-                const int c = min(pl.c0 + j0_ + cc * G::EPC, L - G::EPC);                                \
-                kreg[i] = *reinterpret_cast<const u32x4*>(kb + (int64_t)drow * p.k_sd + c);              \
-            } else {                                                                                     \
-                const int row = idx / G::CR, cc = idx % G::CR;                                           \
-                const int n = min(max(pl.c0 + pl.cs * (j0_ + row), 0), L - 1);                           \
-                kreg[i] = *reinterpret_cast<const u32x4*>(kb + (int64_t)n * p.k_sl + cc * G::EPC);       \
-            }                                                                                            \
-        }                                                                                                \
-    }
-#define SPLAT_LSTORE(stage_)                                                                             \
-    {                                                                                                    \
-        char* ks_w = smem + (stage_) * G::STAGE;                                                         \
-        char* vs_w = ks_w + G::K_BYTES;                                                                  \
-        _Pragma("unroll") for (int i = 0; i < G::CPT; ++i) {                                             \
-            const int idx = tid + 256 * i;                                                               \
-            {                                                                                            \
-                const int row = idx / G::CR, cc = idx % G::CR;                                           \
-                *reinterpret_cast<u32x4*>(vs_w + row * G::V_ROW + cc * 16) = vreg[i];                    \
-            }                                                                                            \
-            if constexpr (KT) {                                                                          \
-                const int drow = idx / G::CRK, cc = idx % G::CRK;                                        \
-                *reinterpret_cast<u32x4*>(ks_w + drow * G::K_ROW + cc * 16) = kreg[i];                   \
-            } else {                                                                                     \
-                const int row = idx / G::CR, cc = idx % G::CR;                                           \
-                *reinterpret_cast<u32x4*>(ks_w + row * G::K_ROW + cc * 16) = kreg[i];                    \
-            }                                                                                            \
-        }                                                                                                \
-    }
-
-    // position of the tile being prefetched
-    int pf_seg = 0, pf_tile = 0;
-    auto pf_normalise = [&]() {
-        while (pf_seg < p.n_seg && pf_tile >= s_plan[pf_seg].n_tiles) {
-            ++pf_seg;
-            pf_tile = 0;
-        }
-    };
-    pf_normalise();
-    if (total_tiles > 0) {
-        SPLAT_GLOAD(pf_seg, pf_tile);
-        SPLAT_LSTORE(0);
-        ++pf_tile;
-        pf_normalise();
-    }
+    dma_wait_all();
     __syncthreads();
 
     // per-lane row maps of the segment being computed
@@ -189,6 +238,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
     RowWin win[MT];
     int w_lo_min = 0, w_lo_max = 0, w_hi_min = 0, w_hi_max = 0;
     SegPlan cpl = {0, 1, 0, 1};
+    const float c2 = p.scale_log2e;
 
     for (int it = 0; it < total_tiles; ++it) {
         // advance the compute position; reload row maps on a segment change
@@ -224,7 +274,11 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
         ++cur_tile;
 
         const bool more = (it + 1 < total_tiles);
-        if (more) SPLAT_GLOAD(pf_seg, pf_tile);
+        if (more) {
+            issue_tile(pf_seg, pf_tile, (it + 1) & 1);
+            ++pf_tile;
+            pf_normalise();
+        }
 
         const char* ks_l = smem + (it & 1) * G::STAGE;
         const char* vs_l = ks_l + G::K_BYTES;
@@ -242,61 +296,86 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
 #pragma unroll
                     for (int j = 0; j < 16; ++j) s_acc[mt][nt][j] = 0.f;
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
+            for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
+                for (int nt = 0; nt < NT; ++nt) {
                     Frag<T> kf;
                     if constexpr (KT) {
-                        kf = lds_frag_cols<T>(ks_l, G::K_ROW, 16 * ks + 8 * g, 16 * ks + 8 * g + 4, 32 * nt, lane);
+                        const int rr = 16 * ks + 8 * g + tr_row;
+                        if constexpr (sizeof(T) == 2) {
+                            const char* a0 = ks_l + rr * G::K_ROWB + (32 * nt + tr_col) * 2;
+                            kf = frag_from_tr<T>(lds_tr16(a0), lds_tr16(a0 + 4 * G::K_ROWB));
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 8; ++e)
+                                kf.v[e] = *reinterpret_cast<const float*>(ks_l + (16 * ks + 8 * g + e) * G::K_ROWB + (32 * nt + lm) * 4);
+                        }
                     } else {
-                        kf = lds_frag_rowmajor<T>(ks_l + (32 * nt + lm) * G::K_ROW + (16 * ks + 8 * g) * ES);
+                        if constexpr (sizeof(T) == 2) {
+                            u32x4 r = *reinterpret_cast<const u32x4*>(ks_l + k_off[ks] + 32 * nt * G::K_ROWB);
+                            kf.v = __builtin_bit_cast(typename Frag<T>::vec, r);
+                        } else {
+                            kf = lds_frag_row_swz<T, G::K_ROWB>(ks_l, 32 * nt + lm, 16 * ks + 8 * g);
+                        }
                     }
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt) mma32(s_acc[mt][nt], kf, qf[mt][ks]);
                 }
             }
 
-            // ---- mask, online softmax ----
+            // ---- mask, online softmax against a lazily updated reference ----
             Frag<T> pf[MT][NT][2];
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-                float mx = kNegBigA;
-                if (full) {
+                if (!full) {
+                    if (cpl.uniform) {  // live iff 0 <= position - lo < cnt
+                        const int base = j0 + 4 * g - win[mt].lo;
+                        const unsigned cnt = (unsigned)win[mt].cnt;
 #pragma unroll
-                    for (int nt = 0; nt < NT; ++nt)
+                        for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                        for (int j = 0; j < 16; ++j) mx = fmaxf(mx, s_acc[mt][nt][j]);
-                } else {
+                            for (int j = 0; j < 16; ++j) {
+                                const unsigned u = (unsigned)(base + 32 * nt + 8 * (j >> 2) + (j & 3));
+                                s_acc[mt][nt][j] = (u < cnt) ? s_acc[mt][nt][j] : kNegBigA;
+                            }
+                    } else {
 #pragma unroll
-                    for (int nt = 0; nt < NT; ++nt)
+                        for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                        for (int j = 0; j < 16; ++j) {
-                            const bool ok = win_live(win[mt], j0 + 32 * nt + acc_row(j, g));
-                            const float sv = ok ? s_acc[mt][nt][j] : kNegBigA;
-                            s_acc[mt][nt][j] = sv;
-                            mx = fmaxf(mx, sv);
-                        }
+                            for (int j = 0; j < 16; ++j)
+                                s_acc[mt][nt][j] = win_live(win[mt], j0 + 32 * nt + acc_row(j, g)) ? s_acc[mt][nt][j] : kNegBigA;
+                    }
                 }
-                mx = fmaxf(mx, __shfl_xor(mx, 32));
-                const float m_new = fmaxf(m_run[mt], mx);
-                const float alpha = fast_exp2((m_run[mt] - m_new) * p.scale_log2e);
-                const float mb = m_new * p.scale_log2e;
-                m_run[mt] = m_new;
+                float mx = s_acc[mt][0][0];
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) mx = fmaxf(mx, s_acc[mt][nt][j]);
+                mx = fmaxf(mx, __shfl_xor(mx, 32));  // the other half of the row lives in lane ^ 32
+                // move the reference only when some row's maximum has outrun it by the threshold (always on the
+                // first live tile); rows that do not move keep alpha = 1
+                if (__any((mx - m_ref[mt]) * c2 > kRescaleThreshold)) {
+                    const float m_new = ((mx - m_ref[mt]) * c2 > kRescaleThreshold) ? mx : m_ref[mt];
+                    const float alpha = fast_exp2((m_ref[mt] - m_new) * c2);
+                    m_ref[mt] = m_new;
+                    l_run[mt] *= alpha;
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                        for (int j = 0; j < 16; ++j) o_acc[mt][dt][j] *= alpha;
+                }
+                const float mb = m_ref[mt] * c2;
                 float rs = 0.f;
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                     for (int j = 0; j < 16; ++j) {
-                        float pv = fast_exp2(fmaf(s_acc[mt][nt][j], p.scale_log2e, -mb));
+                        float pv = fast_exp2(fmaf(s_acc[mt][nt][j], c2, -mb));
                         if (!full) pv = (s_acc[mt][nt][j] > 0.5f * kNegBigA) ? pv : 0.f;
                         rs += pv;
                         pf[mt][nt][j >> 3].v[j & 7] = (T)pv;
                     }
-                l_run[mt] = l_run[mt] * alpha + rs;
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int j = 0; j < 16; ++j) o_acc[mt][dt][j] *= alpha;
+                l_run[mt] += rs;
             }
 
             // ---- O^T += V^T . P^T ----
@@ -306,8 +385,18 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
                 for (int t = 0; t < 2; ++t) {
 #pragma unroll
                     for (int dt = 0; dt < DT; ++dt) {
+                        Frag<T> vf;
                         const int rbase = 32 * nt + 16 * t + 4 * g;
-                        Frag<T> vf = lds_frag_cols<T>(vs_l, G::V_ROW, rbase, rbase + 8, 32 * dt, lane);
+                        if constexpr (sizeof(T) == 2) {
+                            const char* a0 = vs_l + (rbase + tr_row) * G::V_ROWB + (32 * dt + tr_col) * 2;
+                            vf = frag_from_tr<T>(lds_tr16(a0), lds_tr16(a0 + 8 * G::V_ROWB));
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                vf.v[e] = *reinterpret_cast<const float*>(vs_l + (rbase + e) * G::V_ROWB + (32 * dt + lm) * 4);
+                                vf.v[4 + e] = *reinterpret_cast<const float*>(vs_l + (rbase + 8 + e) * G::V_ROWB + (32 * dt + lm) * 4);
+                            }
+                        }
 #pragma unroll
                         for (int mt = 0; mt < MT; ++mt) mma32(o_acc[mt][dt], vf, pf[mt][nt][t]);
                     }
@@ -315,12 +404,8 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
             }
         }
 
-        if (more) {
-            SPLAT_LSTORE((it + 1) & 1);
-            ++pf_tile;
-            pf_normalise();
-        }
-        __syncthreads();
+        dma_wait_all();   // the next tile has landed in LDS
+        __syncthreads();  // ... for every wavefront, and this tile's stage may be overwritten
     }
 
     // ---- epilogue: O = O^T / l, one 4-element run per (row, register quad) ------------------------
@@ -343,9 +428,6 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
         }
     }
 }
-
-#undef SPLAT_GLOAD
-#undef SPLAT_LSTORE
 
 template <typename T, int D, int MT, bool KT>
 static int launch_attn(const AttnParams& p0, hipStream_t st) {
