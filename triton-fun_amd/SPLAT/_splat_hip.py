@@ -12,7 +12,8 @@ from typing import Any, Sequence
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.normpath(os.path.join(_HERE, "..", "lib", "libsplat_hip.so"))
+# SPLAT_HIP_LIB selects another build of the same library (e.g. an instrumented one)
+LIB_PATH = os.environ.get("SPLAT_HIP_LIB") or os.path.normpath(os.path.join(_HERE, "..", "lib", "libsplat_hip.so"))
 
 SPLAT_F32, SPLAT_F16, SPLAT_BF16 = 0, 1, 2
 MAX_SEGMENTS = 4

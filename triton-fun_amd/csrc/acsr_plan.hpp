@@ -30,79 +30,116 @@ __device__ __forceinline__ RowMap load_row_map(const SegPtrs& s, int r) {
     return load_row_map(s.sTod_lin, s.sTod_trans, s.nnz, s.first_col, r);
 }
 
-// Scratch the planner needs in LDS.
+// LDS the planner needs: per-wavefront partial reductions, and the rows' integer maps for later reuse.
+template <int BM>
 struct PlanScratch {
-    int red[SPLAT_MAX_SEGMENTS][5];  // amin, cmax, linmin, linmax, nonuniform
+    int part[4][SPLAT_MAX_SEGMENTS][4];  // [wave][segment]: amin, cmax, linmin, linmax
+    int flag[4][SPLAT_MAX_SEGMENTS];     // [wave][segment]: some row breaks the common step / phase
+    int row_a[SPLAT_MAX_SEGMENTS][BM];
+    int row_lin[SPLAT_MAX_SEGMENTS][BM];
+    int row_cnt[SPLAT_MAX_SEGMENTS][BM];
 };
 
-// Fill plan[0..n_seg) for rows [r0, r0+BM) ∩ [0, n_rows).  All 256 threads of the workgroup call it; it
-// ends with a barrier.  `allow_gather` = false forces dense walks (column step 1).
+template <int BM>
+__device__ __forceinline__ RowMap cached_row_map(const PlanScratch<BM>* ps, int sg, int rr) {
+    RowMap m;
+    m.a = ps->row_a[sg][rr];
+    m.lin = ps->row_lin[sg][rr];
+    m.cnt = ps->row_cnt[sg][rr];
+    return m;
+}
+
+// Gather the maps of rows [r0, r0+BM) of every segment into LDS and reduce what the plans need.  Called by
+// all 256 threads of the workgroup (BM <= 256: one row per thread); contains two barriers.  Afterwards
+// segment_plan() may be evaluated by any thread.
+template <int BM>
+__device__ __forceinline__ void gather_row_maps(const SegPtrs* seg, int n_seg, int r0, int n_rows, PlanScratch<BM>* ps,
+                                                int tid) {
+    static_assert(BM <= 256, "one row per thread");
+    const int lane = tid & 63, wave = tid >> 6;
+    RowMap mine[SPLAT_MAX_SEGMENTS];
+#pragma unroll
+    for (int sg = 0; sg < SPLAT_MAX_SEGMENTS; ++sg) {
+        RowMap m = {0, 1, 0};
+        if (sg < n_seg && tid < BM && r0 + tid < n_rows) m = load_row_map(seg[sg], r0 + tid);
+        mine[sg] = m;
+        if (sg < n_seg) {
+            if (tid < BM) {
+                ps->row_a[sg][tid] = m.a;
+                ps->row_lin[sg][tid] = m.lin;
+                ps->row_cnt[sg][tid] = m.cnt;
+            }
+            const int amin = wave_min_i(m.cnt > 0 ? m.a : 0x7fffffff);
+            const int cmax = wave_max_i(m.cnt > 0 ? m.a + m.lin * (m.cnt - 1) : -1);
+            const int linmin = wave_min_i(m.cnt > 1 ? m.lin : 0x7fffffff);
+            const int linmax = wave_max_i(m.cnt > 1 ? m.lin : 0);
+            if (lane == 0) {
+                ps->part[wave][sg][0] = amin;
+                ps->part[wave][sg][1] = cmax;
+                ps->part[wave][sg][2] = linmin;
+                ps->part[wave][sg][3] = linmax;
+            }
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int sg = 0; sg < SPLAT_MAX_SEGMENTS; ++sg) {
+        if (sg < n_seg) {
+            int amin = 0x7fffffff, linmin = 0x7fffffff, linmax = 0;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                amin = min(amin, ps->part[w][sg][0]);
+                linmin = min(linmin, ps->part[w][sg][2]);
+                linmax = max(linmax, ps->part[w][sg][3]);
+            }
+            bool bad = (linmax != 0 && linmin != linmax);
+            const int step = (linmax == 0) ? 1 : linmin;  // no row with 2+ columns: any step fits
+            if (!bad && step > 1) bad = mine[sg].cnt > 0 && ((mine[sg].a - amin) % step) != 0;
+            const int any_bad = __any(bad) ? 1 : 0;
+            if (lane == 0) ps->flag[wave][sg] = any_bad;
+        }
+    }
+    __syncthreads();
+}
+
+// The workgroup's plan for segment sg (valid after gather_row_maps).  `allow_gather` = false forces dense walks.
+template <int BM>
+__device__ __forceinline__ SegPlan segment_plan(const PlanScratch<BM>* ps, int sg, bool allow_gather) {
+    int amin = 0x7fffffff, cmax = -1, linmin = 0x7fffffff, linmax = 0, bad = 0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        amin = min(amin, ps->part[w][sg][0]);
+        cmax = max(cmax, ps->part[w][sg][1]);
+        linmin = min(linmin, ps->part[w][sg][2]);
+        linmax = max(linmax, ps->part[w][sg][3]);
+        bad |= ps->flag[w][sg];
+    }
+    SegPlan pl;
+    if (cmax < 0) {
+        pl.c0 = 0;
+        pl.cs = 1;
+        pl.n_tiles = 0;
+        pl.uniform = 1;
+        return pl;
+    }
+    const int step = (linmax == 0) ? 1 : linmin;
+    const bool uni = (bad == 0) && (allow_gather || step == 1);
+    pl.uniform = uni ? 1 : 0;
+    pl.cs = uni ? step : 1;
+    // dense walks start on a tile boundary (keeps 16-byte K^T loads aligned and lets neighbouring row blocks
+    // share cache lines); gathered walks start at the first live column
+    pl.c0 = (pl.cs == 1) ? (amin & ~(kBN - 1)) : amin;
+    const int n_pos = (cmax - pl.c0) / pl.cs + 1;
+    pl.n_tiles = (n_pos + kBN - 1) / kBN;
+    return pl;
+}
+
+// gather_row_maps + one SegPlan per segment in LDS (plan[0..n_seg)); ends with a barrier.
 template <int BM>
 __device__ __forceinline__ void plan_segments(const SegPtrs* seg, int n_seg, int r0, int n_rows, bool allow_gather,
-                                              SegPlan* plan, PlanScratch* ps, int tid) {
-    if (tid < SPLAT_MAX_SEGMENTS) {
-        ps->red[tid][0] = 0x7fffffff;
-        ps->red[tid][1] = -1;
-        ps->red[tid][2] = 0x7fffffff;
-        ps->red[tid][3] = 0;
-        ps->red[tid][4] = 0;
-    }
-    __syncthreads();
-    for (int sg = 0; sg < n_seg; ++sg) {
-        for (int rr = tid; rr < BM; rr += 256) {
-            const int r = r0 + rr;
-            if (r < n_rows) {
-                RowMap m = load_row_map(seg[sg], r);
-                if (m.cnt > 0) {
-                    atomicMin(&ps->red[sg][0], m.a);
-                    atomicMax(&ps->red[sg][1], m.a + m.lin * (m.cnt - 1));
-                    if (m.cnt > 1) {
-                        atomicMin(&ps->red[sg][2], m.lin);
-                        atomicMax(&ps->red[sg][3], m.lin);
-                    }
-                }
-            }
-        }
-    }
-    __syncthreads();
-    for (int sg = 0; sg < n_seg; ++sg) {
-        const int amin = ps->red[sg][0], linmin = ps->red[sg][2], linmax = ps->red[sg][3];
-        const int step = (linmax == 0) ? 1 : linmin;  // no row with 2+ columns: any step fits
-        if (linmax != 0 && linmin != linmax) {
-            if (tid == 0) ps->red[sg][4] = 1;
-        } else if (step > 1) {
-            for (int rr = tid; rr < BM; rr += 256) {
-                const int r = r0 + rr;
-                if (r < n_rows) {
-                    RowMap m = load_row_map(seg[sg], r);
-                    if (m.cnt > 0 && ((m.a - amin) % step) != 0) atomicOr(&ps->red[sg][4], 1);
-                }
-            }
-        }
-    }
-    __syncthreads();
-    if (tid < n_seg) {
-        const int sg = tid;
-        SegPlan pl;
-        const int amin = ps->red[sg][0], cmax = ps->red[sg][1], linmin = ps->red[sg][2], linmax = ps->red[sg][3];
-        if (cmax < 0) {
-            pl.c0 = 0;
-            pl.cs = 1;
-            pl.n_tiles = 0;
-            pl.uniform = 1;
-        } else {
-            const int step = (linmax == 0) ? 1 : linmin;
-            const bool uni = (ps->red[sg][4] == 0) && (allow_gather || step == 1);
-            pl.uniform = uni ? 1 : 0;
-            pl.cs = uni ? step : 1;
-            // dense walks start on a tile boundary (keeps 16-byte K^T loads aligned and lets neighbouring row
-            // blocks share cache lines); gathered walks start at the first live column
-            pl.c0 = (pl.cs == 1) ? (amin & ~(kBN - 1)) : amin;
-            const int n_pos = (cmax - pl.c0) / pl.cs + 1;
-            pl.n_tiles = (n_pos + kBN - 1) / kBN;
-        }
-        plan[sg] = pl;
-    }
+                                              SegPlan* plan, PlanScratch<BM>* ps, int tid) {
+    gather_row_maps<BM>(seg, n_seg, r0, n_rows, ps, tid);
+    if (tid < n_seg) plan[tid] = segment_plan<BM>(ps, tid, allow_gather);
     __syncthreads();
 }
 

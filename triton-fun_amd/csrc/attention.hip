@@ -114,10 +114,13 @@ __device__ __forceinline__ Frag<T> lds_frag_row_swz(const char* tile, int row, i
     return f;
 }
 
+#ifndef SPLAT_EXP
+#define SPLAT_EXP 0
+#endif
 constexpr float kRescaleThreshold = 8.0f;  // in log2 units: exponentials stay below 2^8 before the reference moves
 
 template <typename T, int D, int MT, bool KT>
-__global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
+__global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn_fwd_kernel(const AttnParams p) {
     using G = TileGeom<T, D, KT>;
     constexpr int ES = G::ES;
     constexpr int BM = 128 * MT;
@@ -127,8 +130,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
 
     extern __shared__ __attribute__((aligned(1024))) char smem[];
     __shared__ SegPlan s_plan[SPLAT_MAX_SEGMENTS];
-    __shared__ SegPtrs s_seg[SPLAT_MAX_SEGMENTS];  // indexable copy of the segment pointers
-    __shared__ PlanScratch s_ps;
+    __shared__ PlanScratch<BM> s_ps;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lm = lane & 31, g = lane >> 5;
@@ -148,13 +150,9 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
     T* ob = (T*)p.o + b * p.o_sb + h * p.o_sh;
 
     // ---- plan: per segment, the column range and step of this row block ------------------------
-    if (tid == 0) {
-#pragma unroll
-        for (int k = 0; k < SPLAT_MAX_SEGMENTS; ++k) s_seg[k] = p.seg[k];
-    }
-    __syncthreads();
-    plan_segments<BM>(s_seg, p.n_seg, r0, L, !KT, s_plan, &s_ps, tid);
+    plan_segments<BM>(p.seg, p.n_seg, r0, L, !KT, s_plan, &s_ps, tid);
 
+    if (SPLAT_EXP & 128) return;
     int total_tiles = 0;
     for (int sg = 0; sg < p.n_seg; ++sg) total_tiles += s_plan[sg].n_tiles;
 
@@ -232,6 +230,10 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
 
     dma_wait_all();
     __syncthreads();
+    if (SPLAT_EXP & 256) {
+        if (qf[0][0].v[0] == (T)12345.f) ob[0] = (T)0.f;
+        return;
+    }
 
     // per-lane row maps of the segment being computed
     int cur_seg = -1, cur_tile = 0;
@@ -252,9 +254,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
             bool any_empty = false;
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-                RowMap m = {0, 1, 0};
-                if (my_row[mt] < L) m = load_row_map(s_seg[cur_seg], my_row[mt]);
-                win[mt] = make_row_win(m, cpl);
+                win[mt] = make_row_win(cached_row_map<BM>(&s_ps, cur_seg, (wave * MT + mt) * 32 + lm), cpl);
                 if (win[mt].cnt <= 0) {
                     any_empty = true;
                 } else {
@@ -274,7 +274,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
         ++cur_tile;
 
         const bool more = (it + 1 < total_tiles);
-        if (more) {
+        if (more && !(SPLAT_EXP & 32)) {
             issue_tile(pf_seg, pf_tile, (it + 1) & 1);
             ++pf_tile;
             pf_normalise();
@@ -283,9 +283,9 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
         const char* ks_l = smem + (it & 1) * G::STAGE;
         const char* vs_l = ks_l + G::K_BYTES;
 
-        const bool skip = (j0 + kBN <= w_lo_min) || (j0 >= w_hi_max);
+        const bool skip = ((SPLAT_EXP & 1) != 0) || (j0 + kBN <= w_lo_min) || (j0 >= w_hi_max);
         if (!skip) {
-            const bool full = (j0 >= w_lo_max) && (j0 + kBN <= w_hi_min);
+            const bool full = ((SPLAT_EXP & 2) != 0) || ((j0 >= w_lo_max) && (j0 + kBN <= w_hi_min));
 
             // ---- S^T = K . Q^T ----
             f32x16 s_acc[MT][NT];
@@ -354,7 +354,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
                 mx = fmaxf(mx, __shfl_xor(mx, 32));  // the other half of the row lives in lane ^ 32
                 // move the reference only when some row's maximum has outrun it by the threshold (always on the
                 // first live tile); rows that do not move keep alpha = 1
-                if (__any((mx - m_ref[mt]) * c2 > kRescaleThreshold)) {
+                if (!(SPLAT_EXP & 4) && __any((mx - m_ref[mt]) * c2 > kRescaleThreshold)) {
                     const float m_new = ((mx - m_ref[mt]) * c2 > kRescaleThreshold) ? mx : m_ref[mt];
                     const float alpha = fast_exp2((m_ref[mt] - m_new) * c2);
                     m_ref[mt] = m_new;
@@ -370,7 +370,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
                 for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                     for (int j = 0; j < 16; ++j) {
-                        float pv = fast_exp2(fmaf(s_acc[mt][nt][j], c2, -mb));
+                        float pv = (SPLAT_EXP & 8) ? s_acc[mt][nt][j] : fast_exp2(fmaf(s_acc[mt][nt][j], c2, -mb));
                         if (!full) pv = (s_acc[mt][nt][j] > 0.5f * kNegBigA) ? pv : 0.f;
                         rs += pv;
                         pf[mt][nt][j >> 3].v[j & 7] = (T)pv;
@@ -404,17 +404,19 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
             }
         }
 
-        dma_wait_all();   // the next tile has landed in LDS
+        if (!(SPLAT_EXP & 16)) dma_wait_all();   // the next tile has landed in LDS
         __syncthreads();  // ... for every wavefront, and this tile's stage may be overwritten
     }
 
-    // ---- epilogue: O = O^T / l, one 4-element run per (row, register quad) ------------------------
+    // ---- epilogue: O = O^T / l, transposed through LDS so that every global store is a contiguous run --------
+    // (all wavefronts left the loop through its final barrier; each one now uses a private region of the stages)
+    {
+        constexpr int OROW = D * ES + 16;  // padded row of the staging tile
+        char* stg = smem + wave * (32 * OROW);
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        const float l_tot = l_run[mt] + __shfl_xor(l_run[mt], 32);
-        const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-        if (my_row[mt] < L) {
-            T* orow = ob + (int64_t)my_row[mt] * p.o_sl;
+        for (int mt = 0; mt < MT; ++mt) {
+            const float l_tot = l_run[mt] + __shfl_xor(l_run[mt], 32);
+            const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -423,8 +425,21 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnParams p) {
                     vec4 o;
 #pragma unroll
                     for (int i = 0; i < 4; ++i) o[i] = (T)(o_acc[mt][dt][4 * jj + i] * inv);
-                    *reinterpret_cast<vec4*>(orow + 32 * dt + 8 * jj + 4 * g) = o;
+                    *reinterpret_cast<vec4*>(stg + lm * OROW + (32 * dt + 8 * jj + 4 * g) * ES) = o;
                 }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wavefront's LDS writes are visible to its own reads
+            constexpr int CPR = D * ES / 16;                    // 16-byte chunks per output row
+            if (!(SPLAT_EXP & 512)) {
+#pragma unroll
+                for (int i = 0; i < 32 * CPR / 64; ++i) {
+                    const int flat = i * 64 + lane;
+                    const int row = flat / CPR, c = flat % CPR;
+                    const int r = r0 + (wave * MT + mt) * 32 + row;
+                    const u32x4 val = *reinterpret_cast<const u32x4*>(stg + row * OROW + c * 16);
+                    if (r < L) *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(ob + (int64_t)r * p.o_sl) + c * 16) = val;
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // reads done before the next m-tile reuses the region
         }
     }
 }
@@ -454,14 +469,9 @@ static int launch_attn(const AttnParams& p0, hipStream_t st) {
 
 template <typename T>
 static int dispatch_attn(const AttnParams& p, int d, bool kt, hipStream_t st) {
-    // two 32-row tiles per wavefront when the problem has enough row blocks to fill the chip
-    if constexpr (sizeof(T) == 2) {
-        const bool big = (int64_t)p.B * p.H * ((p.L + 255) / 256) >= 512;
-        if (big) {
-            if (d == 64) return kt ? launch_attn<T, 64, 2, true>(p, st) : launch_attn<T, 64, 2, false>(p, st);
-            return kt ? launch_attn<T, 128, 2, true>(p, st) : launch_attn<T, 128, 2, false>(p, st);
-        }
-    }
+    // One 32-row tile per wavefront (BM = 128): 16-bit kernels then fit two workgroups per CU, whose
+    // wavefronts hide each other's LDS, barrier and prologue latency.  Two tiles per wavefront (MT = 2) halve
+    // the LDS traffic per MFMA but need all 512 registers of a SIMD lane and measured slower.
     if (d == 64) return kt ? launch_attn<T, 64, 1, true>(p, st) : launch_attn<T, 64, 1, false>(p, st);
     return kt ? launch_attn<T, 128, 1, true>(p, st) : launch_attn<T, 128, 1, false>(p, st);
 }

@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256) void sddmm_kernel(const SddmmParams p) {
     __shared__ __attribute__((aligned(16))) char s_k[K_ROW * K_ROWS];
     __shared__ SegPlan s_plan[SPLAT_MAX_SEGMENTS];
     __shared__ SegPtrs s_seg[SPLAT_MAX_SEGMENTS];
-    __shared__ PlanScratch s_ps;
+    __shared__ PlanScratch<BM> s_ps;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lm = lane & 31, g = lane >> 5;
@@ -75,8 +75,7 @@ __global__ __launch_bounds__(256) void sddmm_kernel(const SddmmParams p) {
 #pragma unroll
         for (int k = 0; k < SPLAT_MAX_SEGMENTS; ++k) s_seg[k] = p.seg[k];
     }
-    __syncthreads();
-    plan_segments<BM>(s_seg, p.n_seg, r0, L, !KT, s_plan, &s_ps, tid);
+    plan_segments<BM>(p.seg, p.n_seg, r0, L, !KT, s_plan, &s_ps, tid);
 
     // A-operand rows of this lane: query row 32*wave + lm of the block
     const int q_row = min(r0 + 32 * wave + lm, L - 1);
@@ -97,10 +96,7 @@ __global__ __launch_bounds__(256) void sddmm_kernel(const SddmmParams p) {
         int lmin = 0x3fffffff, hmax = -0x3fffffff;
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
-            const int r = r0 + 32 * wave + acc_row(j, g);
-            RowMap m = {0, 1, 0};
-            if (r < L) m = load_row_map(s_seg[sg], r);
-            win[j] = make_row_win(m, pl);
+            win[j] = make_row_win(cached_row_map<BM>(&s_ps, sg, 32 * wave + acc_row(j, g)), pl);
             if (win[j].cnt > 0) {
                 lmin = min(lmin, win[j].lo);
                 hmax = max(hmax, win[j].lo + win[j].cnt);

@@ -37,7 +37,7 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
     __shared__ __attribute__((aligned(16))) char s_v[V_ROW * kBN];
     __shared__ SegPlan s_plan[SPLAT_MAX_SEGMENTS];
     __shared__ SegPtrs s_seg[SPLAT_MAX_SEGMENTS];
-    __shared__ PlanScratch s_ps;
+    __shared__ PlanScratch<BM> s_ps;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lm = lane & 31, g = lane >> 5;
@@ -60,8 +60,7 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
 #pragma unroll
         for (int k = 0; k < SPLAT_MAX_SEGMENTS; ++k) s_seg[k] = p.seg[k];
     }
-    __syncthreads();
-    plan_segments<BM>(s_seg, p.n_seg, r0, L, true, s_plan, &s_ps, tid);
+    plan_segments<BM>(p.seg, p.n_seg, r0, L, true, s_plan, &s_ps, tid);
 
     const int my_row = r0 + 32 * wave + lm;  // A-operand row of this lane
     const T* prow = pb + (int64_t)min(my_row, L - 1) * p.T;
@@ -76,9 +75,7 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
         const SegPlan pl = s_plan[sg];
         if (pl.n_tiles == 0) continue;
         const int off = s_seg[sg].slot_offset;
-        RowMap m = {0, 1, 0};
-        if (my_row < L) m = load_row_map(s_seg[sg], my_row);
-        const RowWin win = make_row_win(m, pl);
+        const RowWin win = make_row_win(cached_row_map<BM>(&s_ps, sg, 32 * wave + lm), pl);
         int lmin = win.cnt > 0 ? win.lo : 0x3fffffff;
         int hmax = win.cnt > 0 ? win.lo + win.cnt : -0x3fffffff;
         lmin = wave_min_i(lmin);
