@@ -71,6 +71,22 @@ __device__ __forceinline__ int lds_off(int row, int byte_col) {
         return row * ROWB + byte_col;
 }
 
+// Swizzle of the 64-byte block index for tiles read with the transposing read, whose 64 lanes touch 8
+// consecutive rows x 64 bytes: 4 consecutive rows must fall into the 4 different 64-byte quadrants of the
+// 256-byte bank space (what a row pitch of 256+64 bytes would give, which the 1 KiB LDS-DMA blocks rule out).
+template <int ROWB>
+__device__ __forceinline__ constexpr int swz64(int row) {
+    return ROWB >= 256 ? (row & 3) : ((row >> 1) & 1);
+}
+// logical 16-byte chunk held at physical chunk position pc of `row`; MODE 0: none, 1: chunk XOR (b128 row reads),
+// 2: 64-byte block XOR (transposing reads)
+template <int ROWB, int MODE>
+__device__ __forceinline__ int logical_chunk(int row, int pc) {
+    if constexpr (MODE == 1) return pc ^ swz<ROWB>(row);
+    if constexpr (MODE == 2) return (((pc >> 2) ^ swz64<ROWB>(row)) << 2) | (pc & 3);
+    return pc;
+}
+
 typedef __attribute__((address_space(1))) const void gptr_t;
 typedef __attribute__((address_space(3))) void lptr_t;
 
@@ -83,7 +99,7 @@ __device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0
 
 // Copy a ROWS x ROWB-byte tile into LDS; row r comes from row_ptr(r) (16-byte aligned, ROWB readable bytes).
 // Each wavefront issues ROWS*ROWB/4096 instructions of 1 KiB.
-template <typename T, int ROWB, int ROWS, bool SWZ, typename RowPtr>
+template <typename T, int ROWB, int ROWS, int SWZ, typename RowPtr>
 __device__ __forceinline__ void dma_tile(char* tile, int wave, int lane, RowPtr row_ptr) {
     constexpr int NI = ROWS * ROWB / 1024;  // wavefront instructions per tile
     constexpr int CPR = ROWB / 16;          // chunks per row
@@ -93,7 +109,7 @@ __device__ __forceinline__ void dma_tile(char* tile, int wave, int lane, RowPtr 
         const int q = wave + 4 * i;
         const int flat = q * 64 + lane;  // chunk position in the tile
         const int row = flat / CPR, pc = flat % CPR;
-        const int c = SWZ ? (pc ^ swz<ROWB>(row)) : pc;
+        const int c = logical_chunk<ROWB, SWZ>(row, pc);
         dma16(reinterpret_cast<const char*>(row_ptr(row)) + c * 16, tile + q * 1024);
     }
 }
@@ -119,6 +135,70 @@ __device__ __forceinline__ Frag<T> lds_frag_row_swz(const char* tile, int row, i
 #endif
 constexpr float kRescaleThreshold = 8.0f;  // in log2 units: exponentials stay below 2^8 before the reference moves
 
+typedef __attribute__((address_space(3))) const u32x4 lds_u32x4;
+typedef __attribute__((address_space(3))) const float lds_f32;
+
+__device__ __forceinline__ u32x4 lds_load128(uint32_t addr) { return *reinterpret_cast<lds_u32x4*>((uintptr_t)addr); }
+__device__ __forceinline__ s16x4 lds_load_tr16(uint32_t addr) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_s16x4*>((uintptr_t)addr));
+}
+__device__ __forceinline__ float lds_load_f32(uint32_t addr) { return *reinterpret_cast<lds_f32*>((uintptr_t)addr); }
+
+// Mask (unless FULL), fold one 64-key tile of scores of one 32-row tile into the running softmax state and
+// emit the exponentials as MFMA B fragments.  One lane owns one query row (half of its 64 positions).
+template <bool FULL, typename T, int DT>
+__device__ __forceinline__ void softmax_tile(f32x16 (&s)[2], Frag<T> (&pf)[2][2], float& m_ref, float& l_run,
+                                             f32x16 (&o)[DT], const RowWin& win, bool uniform, int j0, int g, float c2) {
+    if constexpr (!FULL) {
+        if (uniform) {  // live iff 0 <= position - lo < cnt
+            const int base = j0 + 4 * g - win.lo;
+            const unsigned cnt = (unsigned)win.cnt;
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    const unsigned u = (unsigned)(base + 32 * nt + 8 * (j >> 2) + (j & 3));
+                    s[nt][j] = (u < cnt) ? s[nt][j] : kNegBigA;
+                }
+        } else {
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) s[nt][j] = win_live(win, j0 + 32 * nt + acc_row(j, g)) ? s[nt][j] : kNegBigA;
+        }
+    }
+    float mx = s[0][0];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) mx = fmaxf(mx, s[nt][j]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32));  // the other half of the row lives in lane ^ 32
+    // move the reference only when some row's maximum has outrun it by the threshold (always on the first
+    // live tile); rows that do not move keep alpha = 1
+    if (!(SPLAT_EXP & 4) && __any((mx - m_ref) * c2 > kRescaleThreshold)) {
+        const float m_new = ((mx - m_ref) * c2 > kRescaleThreshold) ? mx : m_ref;
+        const float alpha = fast_exp2((m_ref - m_new) * c2);
+        m_ref = m_new;
+        l_run *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) o[dt][j] *= alpha;
+    }
+    const float mb = m_ref * c2;
+    float rs = 0.f;
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            float pv = fast_exp2(fmaf(s[nt][j], c2, -mb));
+            if constexpr (!FULL) pv = (s[nt][j] > 0.5f * kNegBigA) ? pv : 0.f;
+            rs += pv;
+            pf[nt][j >> 3].v[j & 7] = (T)pv;
+        }
+    l_run += rs;
+}
+
 template <typename T, int D, int MT, bool KT>
 __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn_fwd_kernel(const AttnParams p) {
     using G = TileGeom<T, D, KT>;
@@ -127,12 +207,16 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
     constexpr int KS = D / 16;  // contraction steps of the score product
     constexpr int DT = D / 32;  // 32-row tiles of O^T
     constexpr int NT = kBN / 32;
+    static_assert(NT == 2, "softmax_tile assumes two 32-key tiles");
+    static_assert((G::STAGE & (G::STAGE - 1)) == 0, "the stage toggle is an XOR");
+    constexpr bool FAST_DMA = (ES == 2);  // lane offsets of the LDS-DMA do not depend on the instruction index
 
     extern __shared__ __attribute__((aligned(1024))) char smem[];
     __shared__ SegPlan s_plan[SPLAT_MAX_SEGMENTS];
     __shared__ PlanScratch<BM> s_ps;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lm = lane & 31, g = lane >> 5;
 
     const int logical = xcd_remap(blockIdx.x, gridDim.x);
@@ -157,40 +241,96 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
     for (int sg = 0; sg < p.n_seg; ++sg) total_tiles += s_plan[sg].n_tiles;
 
     // ---- tile walker: asynchronous global -> LDS copies of tile (sg, tile) into a stage ----------
-    auto issue_tile = [&](int sg, int tile, int stage) {
-        const SegPlan pl = s_plan[sg];
+    // A tile is copied as 1 KiB blocks, one wavefront instruction each; block q holds tile rows q*RPI.. and
+    // wavefront w issues blocks w, w+4, ...  Lane i of a block supplies physical chunk i, i.e. (row i / CPR,
+    // chunk position i % CPR), and loads the logical chunk the tile's swizzle assigns to that position.  For
+    // 16-bit types that assignment does not depend on the block, so a lane's source offset within a block is
+    // a per-segment constant and the block's base is wavefront-uniform.
+    constexpr int V_CPR = G::V_ROWB / 16, V_RPI = 1024 / G::V_ROWB;
+    constexpr int K_CPR = G::K_ROWB / 16, K_RPI = 1024 / G::K_ROWB;
+    constexpr int V_NI = kBN * G::V_ROWB / 4096, K_NI = G::K_ROWS * G::K_ROWB / 4096;  // blocks per wavefront
+    auto issue_tile_general = [&](const SegPlan& pl, int tile, int stage) {
         const int j0 = tile * kBN;
         char* ks_w = smem + stage * G::STAGE;
         char* vs_w = ks_w + G::K_BYTES;
         auto key_row = [&](int row) { return min(max(pl.c0 + pl.cs * (j0 + row), 0), L - 1); };
-        dma_tile<T, G::V_ROWB, kBN, false>(vs_w, wave, lane, [&](int row) { return vb + (int64_t)key_row(row) * p.v_sl; });
+        dma_tile<T, G::V_ROWB, kBN, (ES == 2 ? 2 : 0)>(vs_w, wave, lane, [&](int row) { return vb + (int64_t)key_row(row) * p.v_sl; });
         if constexpr (KT) {
             // rows = contraction index, 64 consecutive keys per row (dense walk); a chunk that would run past
             // the last key is replaced by the last whole chunk (those positions are never live)
-            constexpr int CPR = G::K_ROWB / 16;
 #pragma unroll
-            for (int i = 0; i < G::K_ROWS * G::K_ROWB / 4096; ++i) {
+            for (int i = 0; i < K_NI; ++i) {
                 const int q = wave + 4 * i;
                 const int flat = q * 64 + lane;
-                const int row = flat / CPR, pc = flat % CPR;
-                const int c = min(pl.c0 + j0 + pc * G::EPC, L - G::EPC);
+                const int row = flat / K_CPR, pc = flat % K_CPR;
+                const int lc = logical_chunk<G::K_ROWB, (ES == 2 ? 2 : 0)>(row, pc);
+                const int c = min(pl.c0 + j0 + lc * G::EPC, L - G::EPC);
                 dma16(kb + (int64_t)row * p.k_sd + c, ks_w + q * 1024);
             }
         } else {
-            dma_tile<T, G::K_ROWB, kBN, true>(ks_w, wave, lane, [&](int row) { return kb + (int64_t)key_row(row) * p.k_sl; });
+            dma_tile<T, G::K_ROWB, kBN, 1>(ks_w, wave, lane, [&](int row) { return kb + (int64_t)key_row(row) * p.k_sl; });
+        }
+    };
+    // per-lane byte offsets inside a block for the segment being fetched (FAST_DMA only)
+    uint32_t v_lane_off = 0, k_lane_off = 0;
+    auto set_lane_offsets = [&](const SegPlan& pl) {
+        if constexpr (FAST_DMA) {
+            const int vr = lane / V_CPR, vpc = lane % V_CPR;
+            v_lane_off = (uint32_t)((int64_t)pl.cs * vr * p.v_sl * ES) + logical_chunk<G::V_ROWB, 2>(vr, vpc) * 16;
+            const int kr = lane / K_CPR, kpc = lane % K_CPR;
+            if constexpr (KT)
+                k_lane_off = (uint32_t)((int64_t)kr * p.k_sd * ES) + logical_chunk<G::K_ROWB, 2>(kr, kpc) * 16;
+            else
+                k_lane_off = (uint32_t)((int64_t)pl.cs * kr * p.k_sl * ES) +
+                             logical_chunk<G::K_ROWB, 1>(wave * K_RPI + kr, kpc) * 16;
+        }
+    };
+    auto issue_tile = [&](const SegPlan& pl, int tile, int stage) {
+        const int j0 = tile * kBN;
+        const int key_first = pl.c0 + pl.cs * j0, key_last = pl.c0 + pl.cs * (j0 + kBN - 1);
+        bool fast = FAST_DMA && key_last < L;
+        if constexpr (KT) fast = fast && (key_first + kBN <= L);
+        if (!fast) {
+            issue_tile_general(pl, tile, stage);
+            return;
+        }
+        char* ks_w = smem + stage * G::STAGE;
+        char* vs_w = ks_w + G::K_BYTES;
+#pragma unroll
+        for (int i = 0; i < V_NI; ++i) {
+            const int q = wave + 4 * i;
+            const char* base = reinterpret_cast<const char*>(vb + (int64_t)(key_first + pl.cs * q * V_RPI) * p.v_sl);
+            dma16(base + v_lane_off, vs_w + q * 1024);
+        }
+#pragma unroll
+        for (int i = 0; i < K_NI; ++i) {
+            const int q = wave + 4 * i;
+            const char* base;
+            if constexpr (KT)
+                base = reinterpret_cast<const char*>(kb + (int64_t)(q * K_RPI) * p.k_sd + key_first);
+            else
+                base = reinterpret_cast<const char*>(kb + (int64_t)(key_first + pl.cs * q * K_RPI) * p.k_sl);
+            dma16(base + k_lane_off, ks_w + q * 1024);
         }
     };
 
     int pf_seg = 0, pf_tile = 0;  // position of the next tile to fetch
+    SegPlan ppl = {0, 1, 0, 1};
     auto pf_normalise = [&]() {
+        bool moved = (pf_seg == 0 && pf_tile == 0);
         while (pf_seg < p.n_seg && pf_tile >= s_plan[pf_seg].n_tiles) {
             ++pf_seg;
             pf_tile = 0;
+            moved = true;
+        }
+        if (moved && pf_seg < p.n_seg) {
+            ppl = s_plan[pf_seg];
+            set_lane_offsets(ppl);
         }
     };
     pf_normalise();
     if (total_tiles > 0) {
-        issue_tile(pf_seg, pf_tile, 0);
+        issue_tile(ppl, pf_tile, 0);
         ++pf_tile;
         pf_normalise();
     }
@@ -218,15 +358,33 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
             for (int j = 0; j < 16; ++j) o_acc[mt][dt][j] = 0.f;
     }
 
-    // lane-dependent parts of the LDS read addresses (stage base and tile constants are added per read)
-    int k_off[KS];  // row-major K: (row lm, logical chunk of step ks) after swizzling
-    if constexpr (!KT) {
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) k_off[ks] = lds_off<G::K_ROWB, true>(lm, (16 * ks + 8 * g) * ES);
-    }
+    // ---- LDS read addresses: lane-dependent part + current stage; tile constants go into the instruction's
+    // immediate offset; the stage is toggled by XOR once per tile -----------------------------------------
+    const uint32_t smem_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
     // transposing reads: lane s of a 16-lane block addresses row s/4, 8 bytes at element column 16*(block%2) + 4*(s%4)
     const int tr_row = (lane & 15) >> 2;
     const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    uint32_t k_addr[KT ? NT : KS];  // K tile: row-major: (row lm, swizzled chunk of step ks); K^T: (row 8g + tr_row, block nt)
+    uint32_t v_addr[DT];            // V tile: (row 4g + tr_row, swizzled 64-byte block dt, column tr_col)
+    if constexpr (ES == 2) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+            v_addr[dt] = smem_base + G::K_BYTES + (4 * g + tr_row) * G::V_ROWB +
+                         ((dt ^ swz64<G::V_ROWB>(4 * g + tr_row)) * 64) + tr_col * 2;
+        if constexpr (KT) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+                k_addr[nt] = smem_base + (8 * g + tr_row) * G::K_ROWB + ((nt ^ swz64<G::K_ROWB>(8 * g + tr_row)) * 64) + tr_col * 2;
+        } else {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) k_addr[ks] = smem_base + lds_off<G::K_ROWB, true>(lm, (16 * ks + 8 * g) * ES);
+        }
+    } else {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) v_addr[dt] = smem_base + G::K_BYTES + (32 * dt + lm) * 4;
+#pragma unroll
+        for (int i = 0; i < (KT ? NT : KS); ++i) k_addr[i] = smem_base;
+    }
 
     dma_wait_all();
     __syncthreads();
@@ -275,13 +433,10 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
 
         const bool more = (it + 1 < total_tiles);
         if (more && !(SPLAT_EXP & 32)) {
-            issue_tile(pf_seg, pf_tile, (it + 1) & 1);
+            issue_tile(ppl, pf_tile, (it + 1) & 1);
             ++pf_tile;
             pf_normalise();
         }
-
-        const char* ks_l = smem + (it & 1) * G::STAGE;
-        const char* vs_l = ks_l + G::K_BYTES;
 
         const bool skip = ((SPLAT_EXP & 1) != 0) || (j0 + kBN <= w_lo_min) || (j0 >= w_hi_max);
         if (!skip) {
@@ -300,20 +455,20 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
                     Frag<T> kf;
-                    if constexpr (KT) {
-                        const int rr = 16 * ks + 8 * g + tr_row;
-                        if constexpr (sizeof(T) == 2) {
-                            const char* a0 = ks_l + rr * G::K_ROWB + (32 * nt + tr_col) * 2;
-                            kf = frag_from_tr<T>(lds_tr16(a0), lds_tr16(a0 + 4 * G::K_ROWB));
+                    if constexpr (ES == 2) {
+                        if constexpr (KT) {
+                            // rows 16ks + 8g + {0..3} and +4: multiples of 4 rows leave the lane's swizzle term alone
+                            const uint32_t a0 = k_addr[nt] + 16 * ks * G::K_ROWB;
+                            kf = frag_from_tr<T>(lds_load_tr16(a0), lds_load_tr16(a0 + 4 * G::K_ROWB));
                         } else {
+                            kf.v = __builtin_bit_cast(typename Frag<T>::vec, lds_load128(k_addr[ks] + 32 * nt * G::K_ROWB));
+                        }
+                    } else {
+                        const char* ks_l = smem + (it & 1) * G::STAGE;
+                        if constexpr (KT) {
 #pragma unroll
                             for (int e = 0; e < 8; ++e)
                                 kf.v[e] = *reinterpret_cast<const float*>(ks_l + (16 * ks + 8 * g + e) * G::K_ROWB + (32 * nt + lm) * 4);
-                        }
-                    } else {
-                        if constexpr (sizeof(T) == 2) {
-                            u32x4 r = *reinterpret_cast<const u32x4*>(ks_l + k_off[ks] + 32 * nt * G::K_ROWB);
-                            kf.v = __builtin_bit_cast(typename Frag<T>::vec, r);
                         } else {
                             kf = lds_frag_row_swz<T, G::K_ROWB>(ks_l, 32 * nt + lm, 16 * ks + 8 * g);
                         }
@@ -325,57 +480,14 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
 
             // ---- mask, online softmax against a lazily updated reference ----
             Frag<T> pf[MT][NT][2];
+            if (full) {
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                if (!full) {
-                    if (cpl.uniform) {  // live iff 0 <= position - lo < cnt
-                        const int base = j0 + 4 * g - win[mt].lo;
-                        const unsigned cnt = (unsigned)win[mt].cnt;
+                for (int mt = 0; mt < MT; ++mt)
+                    softmax_tile<true, T, DT>(s_acc[mt], pf[mt], m_ref[mt], l_run[mt], o_acc[mt], win[mt], true, j0, g, c2);
+            } else {
 #pragma unroll
-                        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                            for (int j = 0; j < 16; ++j) {
-                                const unsigned u = (unsigned)(base + 32 * nt + 8 * (j >> 2) + (j & 3));
-                                s_acc[mt][nt][j] = (u < cnt) ? s_acc[mt][nt][j] : kNegBigA;
-                            }
-                    } else {
-#pragma unroll
-                        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                            for (int j = 0; j < 16; ++j)
-                                s_acc[mt][nt][j] = win_live(win[mt], j0 + 32 * nt + acc_row(j, g)) ? s_acc[mt][nt][j] : kNegBigA;
-                    }
-                }
-                float mx = s_acc[mt][0][0];
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                    for (int j = 0; j < 16; ++j) mx = fmaxf(mx, s_acc[mt][nt][j]);
-                mx = fmaxf(mx, __shfl_xor(mx, 32));  // the other half of the row lives in lane ^ 32
-                // move the reference only when some row's maximum has outrun it by the threshold (always on the
-                // first live tile); rows that do not move keep alpha = 1
-                if (!(SPLAT_EXP & 4) && __any((mx - m_ref[mt]) * c2 > kRescaleThreshold)) {
-                    const float m_new = ((mx - m_ref[mt]) * c2 > kRescaleThreshold) ? mx : m_ref[mt];
-                    const float alpha = fast_exp2((m_ref[mt] - m_new) * c2);
-                    m_ref[mt] = m_new;
-                    l_run[mt] *= alpha;
-#pragma unroll
-                    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                        for (int j = 0; j < 16; ++j) o_acc[mt][dt][j] *= alpha;
-                }
-                const float mb = m_ref[mt] * c2;
-                float rs = 0.f;
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                    for (int j = 0; j < 16; ++j) {
-                        float pv = (SPLAT_EXP & 8) ? s_acc[mt][nt][j] : fast_exp2(fmaf(s_acc[mt][nt][j], c2, -mb));
-                        if (!full) pv = (s_acc[mt][nt][j] > 0.5f * kNegBigA) ? pv : 0.f;
-                        rs += pv;
-                        pf[mt][nt][j >> 3].v[j & 7] = (T)pv;
-                    }
-                l_run[mt] += rs;
+                for (int mt = 0; mt < MT; ++mt)
+                    softmax_tile<false, T, DT>(s_acc[mt], pf[mt], m_ref[mt], l_run[mt], o_acc[mt], win[mt], cpl.uniform != 0, j0, g, c2);
             }
 
             // ---- O^T += V^T . P^T ----
@@ -386,15 +498,15 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
 #pragma unroll
                     for (int dt = 0; dt < DT; ++dt) {
                         Frag<T> vf;
-                        const int rbase = 32 * nt + 16 * t + 4 * g;
-                        if constexpr (sizeof(T) == 2) {
-                            const char* a0 = vs_l + (rbase + tr_row) * G::V_ROWB + (32 * dt + tr_col) * 2;
-                            vf = frag_from_tr<T>(lds_tr16(a0), lds_tr16(a0 + 8 * G::V_ROWB));
+                        if constexpr (ES == 2) {
+                            const uint32_t a0 = v_addr[dt] + (32 * nt + 16 * t) * G::V_ROWB;
+                            vf = frag_from_tr<T>(lds_load_tr16(a0), lds_load_tr16(a0 + 8 * G::V_ROWB));
                         } else {
+                            const int rbase = 32 * nt + 16 * t + 4 * g;
 #pragma unroll
                             for (int e = 0; e < 4; ++e) {
-                                vf.v[e] = *reinterpret_cast<const float*>(vs_l + (rbase + e) * G::V_ROWB + (32 * dt + lm) * 4);
-                                vf.v[4 + e] = *reinterpret_cast<const float*>(vs_l + (rbase + 8 + e) * G::V_ROWB + (32 * dt + lm) * 4);
+                                vf.v[e] = lds_load_f32(v_addr[dt] + (rbase + e) * G::V_ROWB);
+                                vf.v[4 + e] = lds_load_f32(v_addr[dt] + (rbase + 8 + e) * G::V_ROWB);
                             }
                         }
 #pragma unroll
@@ -403,6 +515,12 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
                 }
             }
         }
+
+        // the other stage becomes current
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) v_addr[dt] ^= G::STAGE;
+#pragma unroll
+        for (int i = 0; i < (KT ? NT : KS); ++i) k_addr[i] ^= G::STAGE;
 
         if (!(SPLAT_EXP & 16)) dma_wait_all();   // the next tile has landed in LDS
         __syncthreads();  // ... for every wavefront, and this tile's stage may be overwritten
