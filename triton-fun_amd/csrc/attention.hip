@@ -178,21 +178,26 @@ __device__ __forceinline__ void softmax_tile(f32x16 (&s)[2], Frag<T> (&pf)[2][2]
     if (!(SPLAT_EXP & 4) && __any((mx - m_ref) * c2 > kRescaleThreshold)) {
         const float m_new = ((mx - m_ref) * c2 > kRescaleThreshold) ? mx : m_ref;
         const float alpha = fast_exp2((m_ref - m_new) * c2);
+        const bool had_data = __any(m_ref > 0.5f * kNegBigA);  // otherwise O and l are still all zero
         m_ref = m_new;
-        l_run *= alpha;
+        if (had_data) {
+            l_run *= alpha;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
+            for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-            for (int j = 0; j < 16; ++j) o[dt][j] *= alpha;
+                for (int j = 0; j < 16; ++j) o[dt][j] *= alpha;
+        }
     }
-    const float mb = m_ref * c2;
+    // Masked scores are -1e30: their exponential underflows to exactly 0 as long as the reference is a real
+    // score.  A row that has seen no live score yet keeps the -1e30 reference; give it offset 0 so that its
+    // (all masked) entries still map to 0 instead of exp2(0).
+    const float mb = (FULL || m_ref > 0.5f * kNegBigA) ? m_ref * c2 : 0.f;
     float rs = 0.f;
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
-            float pv = fast_exp2(fmaf(s[nt][j], c2, -mb));
-            if constexpr (!FULL) pv = (s[nt][j] > 0.5f * kNegBigA) ? pv : 0.f;
+            const float pv = fast_exp2(fmaf(s[nt][j], c2, -mb));
             rs += pv;
             pf[nt][j >> 3].v[j & 7] = (T)pv;
         }
@@ -239,6 +244,7 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
     if (SPLAT_EXP & 128) return;
     int total_tiles = 0;
     for (int sg = 0; sg < p.n_seg; ++sg) total_tiles += s_plan[sg].n_tiles;
+    total_tiles = __builtin_amdgcn_readfirstlane(total_tiles);
 
     // ---- tile walker: asynchronous global -> LDS copies of tile (sg, tile) into a stage ----------
     // A tile is copied as 1 KiB blocks, one wavefront instruction each; block q holds tile rows q*RPI.. and
@@ -271,20 +277,32 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
             dma_tile<T, G::K_ROWB, kBN, 1>(ks_w, wave, lane, [&](int row) { return kb + (int64_t)key_row(row) * p.k_sl; });
         }
     };
-    // per-lane byte offsets inside a block for the segment being fetched (FAST_DMA only)
+    // FAST_DMA state for the segment being fetched: per-lane byte offsets inside a block, wavefront-uniform
+    // running pointers to block `wave` of the next tile, and the byte distance between tile positions.
     uint32_t v_lane_off = 0, k_lane_off = 0;
+    const char* v_next = nullptr;
+    const char* k_next = nullptr;
+    int64_t v_key = 0, k_key = 0;  // bytes from one tile position to the next (K^T layout: from one d row to the next)
     auto set_lane_offsets = [&](const SegPlan& pl) {
         if constexpr (FAST_DMA) {
             const int vr = lane / V_CPR, vpc = lane % V_CPR;
             v_lane_off = (uint32_t)((int64_t)pl.cs * vr * p.v_sl * ES) + logical_chunk<G::V_ROWB, 2>(vr, vpc) * 16;
+            v_key = (int64_t)p.v_sl * ES * pl.cs;
+            v_next = reinterpret_cast<const char*>(vb) + (int64_t)pl.c0 * p.v_sl * ES + (int64_t)wave * V_RPI * v_key;
             const int kr = lane / K_CPR, kpc = lane % K_CPR;
-            if constexpr (KT)
+            if constexpr (KT) {
                 k_lane_off = (uint32_t)((int64_t)kr * p.k_sd * ES) + logical_chunk<G::K_ROWB, 2>(kr, kpc) * 16;
-            else
+                k_key = (int64_t)p.k_sd * ES;
+                k_next = reinterpret_cast<const char*>(kb) + (int64_t)pl.c0 * ES + (int64_t)wave * K_RPI * k_key;
+            } else {
                 k_lane_off = (uint32_t)((int64_t)pl.cs * kr * p.k_sl * ES) +
                              logical_chunk<G::K_ROWB, 1>(wave * K_RPI + kr, kpc) * 16;
+                k_key = (int64_t)p.k_sl * ES * pl.cs;
+                k_next = reinterpret_cast<const char*>(kb) + (int64_t)pl.c0 * p.k_sl * ES + (int64_t)wave * K_RPI * k_key;
+            }
         }
     };
+    // Tiles of a segment are issued in order, so the running pointers simply advance by one tile per call.
     auto issue_tile = [&](const SegPlan& pl, int tile, int stage) {
         const int j0 = tile * kBN;
         const int key_first = pl.c0 + pl.cs * j0, key_last = pl.c0 + pl.cs * (j0 + kBN - 1);
@@ -292,26 +310,24 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
         if constexpr (KT) fast = fast && (key_first + kBN <= L);
         if (!fast) {
             issue_tile_general(pl, tile, stage);
-            return;
-        }
-        char* ks_w = smem + stage * G::STAGE;
-        char* vs_w = ks_w + G::K_BYTES;
+        } else {
+            char* ks_w = smem + stage * G::STAGE;
+            char* vs_w = ks_w + G::K_BYTES;
+            const char* vbase = v_next;
+            const char* kbase = k_next;
 #pragma unroll
-        for (int i = 0; i < V_NI; ++i) {
-            const int q = wave + 4 * i;
-            const char* base = reinterpret_cast<const char*>(vb + (int64_t)(key_first + pl.cs * q * V_RPI) * p.v_sl);
-            dma16(base + v_lane_off, vs_w + q * 1024);
-        }
+            for (int i = 0; i < V_NI; ++i) {
+                dma16(vbase + v_lane_off, vs_w + (wave + 4 * i) * 1024);
+                vbase += 4 * V_RPI * v_key;
+            }
 #pragma unroll
-        for (int i = 0; i < K_NI; ++i) {
-            const int q = wave + 4 * i;
-            const char* base;
-            if constexpr (KT)
-                base = reinterpret_cast<const char*>(kb + (int64_t)(q * K_RPI) * p.k_sd + key_first);
-            else
-                base = reinterpret_cast<const char*>(kb + (int64_t)(key_first + pl.cs * q * K_RPI) * p.k_sl);
-            dma16(base + k_lane_off, ks_w + q * 1024);
+            for (int i = 0; i < K_NI; ++i) {
+                dma16(kbase + k_lane_off, ks_w + (wave + 4 * i) * 1024);
+                kbase += 4 * K_RPI * k_key;
+            }
         }
+        v_next += kBN * v_key;
+        k_next += KT ? (int64_t)(kBN * ES) : kBN * k_key;
     };
 
     int pf_seg = 0, pf_tile = 0;  // position of the next tile to fetch
@@ -324,7 +340,11 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
             moved = true;
         }
         if (moved && pf_seg < p.n_seg) {
-            ppl = s_plan[pf_seg];
+            const SegPlan t = s_plan[pf_seg];  // the same for every lane: keep it in scalar registers
+            ppl.c0 = __builtin_amdgcn_readfirstlane(t.c0);
+            ppl.cs = __builtin_amdgcn_readfirstlane(t.cs);
+            ppl.n_tiles = __builtin_amdgcn_readfirstlane(t.n_tiles);
+            ppl.uniform = __builtin_amdgcn_readfirstlane(t.uniform);
             set_lane_offsets(ppl);
         }
     };
@@ -393,6 +413,9 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
         return;
     }
 
+    if ((SPLAT_EXP & 32768) && (blockIdx.x & 8)) {
+        for (int z = 0; z < 10; ++z) __builtin_amdgcn_s_sleep(127);
+    }
     // per-lane row maps of the segment being computed
     int cur_seg = -1, cur_tile = 0;
     RowWin win[MT];
@@ -400,14 +423,28 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
     SegPlan cpl = {0, 1, 0, 1};
     const float c2 = p.scale_log2e;
 
+#if SPLAT_EXP & 65536
+    unsigned long long tl[16][8];
+    const bool tl_on = (blockIdx.x == 4001 || blockIdx.x == 4009);
+#define TL(i_) if (tl_on && it < 16) tl[it][i_] = __builtin_readcyclecounter();
+#else
+#define TL(i_)
+#endif
     for (int it = 0; it < total_tiles; ++it) {
+        TL(0)
         // advance the compute position; reload row maps on a segment change
         if (cur_seg < 0 || cur_tile >= cpl.n_tiles) {
             do {
                 ++cur_seg;
             } while (s_plan[cur_seg].n_tiles == 0);
             cur_tile = 0;
-            cpl = s_plan[cur_seg];
+            {
+                const SegPlan t = s_plan[cur_seg];
+                cpl.c0 = __builtin_amdgcn_readfirstlane(t.c0);
+                cpl.cs = __builtin_amdgcn_readfirstlane(t.cs);
+                cpl.n_tiles = __builtin_amdgcn_readfirstlane(t.n_tiles);
+                cpl.uniform = __builtin_amdgcn_readfirstlane(t.uniform);
+            }
             int lmin = 0x3fffffff, lmax = -0x3fffffff, hmin = 0x3fffffff, hmax = -0x3fffffff;
             bool any_empty = false;
 #pragma unroll
@@ -438,11 +475,14 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
             pf_normalise();
         }
 
+        TL(1)
         const bool skip = ((SPLAT_EXP & 1) != 0) || (j0 + kBN <= w_lo_min) || (j0 >= w_hi_max);
         if (!skip) {
             const bool full = ((SPLAT_EXP & 2) != 0) || ((j0 >= w_lo_max) && (j0 + kBN <= w_hi_min));
 
             // ---- S^T = K . Q^T ----
+            // All K fragments of a 32-key tile are requested from LDS before the first MFMA that needs them, so
+            // that the reads of tile nt+1 are in flight while the matrix unit works on tile nt.
             f32x16 s_acc[MT][NT];
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
@@ -450,11 +490,12 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
                 for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                     for (int j = 0; j < 16; ++j) s_acc[mt][nt][j] = 0.f;
+            Frag<T> kfr[NT][KS];
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
+            for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
-                    Frag<T> kf;
+                for (int ks = 0; ks < KS; ++ks) {
+                    Frag<T>& kf = kfr[nt][ks];
                     if constexpr (ES == 2) {
                         if constexpr (KT) {
                             // rows 16ks + 8g + {0..3} and +4: multiples of 4 rows leave the lane's swizzle term alone
@@ -473,14 +514,31 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
                             kf = lds_frag_row_swz<T, G::K_ROWB>(ks_l, 32 * nt + lm, 16 * ks + 8 * g);
                         }
                     }
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt) mma32(s_acc[mt][nt], kf, qf[mt][ks]);
                 }
             }
+            __builtin_amdgcn_sched_barrier(0);  // keep the requests above the matrix work
+            if (SPLAT_EXP & 16384) __builtin_amdgcn_s_setprio(1);
+            if (!(SPLAT_EXP & 1024)) {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) mma32(s_acc[mt][nt], kfr[nt][ks], qf[mt][ks]);
+            }
 
+            TL(2)
+            if (SPLAT_EXP & 16384) __builtin_amdgcn_s_setprio(0);
             // ---- mask, online softmax against a lazily updated reference ----
             Frag<T> pf[MT][NT][2];
-            if (full) {
+            if (SPLAT_EXP & 4096) {
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                        for (int j = 0; j < 16; ++j) pf[mt][nt][j >> 3].v[j & 7] = (T)s_acc[mt][nt][j];
+            } else if (full) {
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
                     softmax_tile<true, T, DT>(s_acc[mt], pf[mt], m_ref[mt], l_run[mt], o_acc[mt], win[mt], true, j0, g, c2);
@@ -490,32 +548,47 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
                     softmax_tile<false, T, DT>(s_acc[mt], pf[mt], m_ref[mt], l_run[mt], o_acc[mt], win[mt], cpl.uniform != 0, j0, g, c2);
             }
 
+            TL(3)
             // ---- O^T += V^T . P^T ----
+            // V fragments are requested one 16-key step (DT fragments) ahead of the MFMAs that consume them.
+            auto load_v = [&](int nt, int t, int dt) {
+                Frag<T> vf;
+                if constexpr (ES == 2) {
+                    const uint32_t a0 = v_addr[dt] + (32 * nt + 16 * t) * G::V_ROWB;
+                    vf = frag_from_tr<T>(lds_load_tr16(a0), lds_load_tr16(a0 + 8 * G::V_ROWB));
+                } else {
+                    const int rbase = 32 * nt + 16 * t + 4 * g;
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-#pragma unroll
-                for (int t = 0; t < 2; ++t) {
-#pragma unroll
-                    for (int dt = 0; dt < DT; ++dt) {
-                        Frag<T> vf;
-                        if constexpr (ES == 2) {
-                            const uint32_t a0 = v_addr[dt] + (32 * nt + 16 * t) * G::V_ROWB;
-                            vf = frag_from_tr<T>(lds_load_tr16(a0), lds_load_tr16(a0 + 8 * G::V_ROWB));
-                        } else {
-                            const int rbase = 32 * nt + 16 * t + 4 * g;
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) {
-                                vf.v[e] = lds_load_f32(v_addr[dt] + (rbase + e) * G::V_ROWB);
-                                vf.v[4 + e] = lds_load_f32(v_addr[dt] + (rbase + 8 + e) * G::V_ROWB);
-                            }
-                        }
-#pragma unroll
-                        for (int mt = 0; mt < MT; ++mt) mma32(o_acc[mt][dt], vf, pf[mt][nt][t]);
+                    for (int e = 0; e < 4; ++e) {
+                        vf.v[e] = lds_load_f32(v_addr[dt] + (rbase + e) * G::V_ROWB);
+                        vf.v[4 + e] = lds_load_f32(v_addr[dt] + (rbase + 8 + e) * G::V_ROWB);
                     }
+                }
+                return vf;
+            };
+            Frag<T> vfr[2][DT];
+            if (SPLAT_EXP & 16384) __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) vfr[0][dt] = load_v(0, 0, dt);
+#pragma unroll
+            for (int step = 0; step < 2 * NT; ++step) {
+                const int nt = step >> 1, t = step & 1;
+                if (step + 1 < 2 * NT) {
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) vfr[(step + 1) & 1][dt] = load_v((step + 1) >> 1, (step + 1) & 1, dt);
+                }
+                __builtin_amdgcn_sched_barrier(0);  // keep the requests above the matrix work
+                if (!(SPLAT_EXP & 2048)) {
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) mma32(o_acc[mt][dt], vfr[step & 1][dt], pf[mt][nt][t]);
                 }
             }
         }
 
+        TL(4)
+        if (SPLAT_EXP & 16384) __builtin_amdgcn_s_setprio(0);
         // the other stage becomes current
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) v_addr[dt] ^= G::STAGE;
@@ -523,8 +596,18 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
         for (int i = 0; i < (KT ? NT : KS); ++i) k_addr[i] ^= G::STAGE;
 
         if (!(SPLAT_EXP & 16)) dma_wait_all();   // the next tile has landed in LDS
-        __syncthreads();  // ... for every wavefront, and this tile's stage may be overwritten
+        TL(5)
+        if (!(SPLAT_EXP & 8192)) __syncthreads();  // ... for every wavefront, and this tile's stage may be overwritten
+        TL(6)
     }
+#if SPLAT_EXP & 65536
+    if (tl_on && lane == 0) {
+        unsigned long long* dbg = reinterpret_cast<unsigned long long*>(const_cast<void*>(p.q)) + ((blockIdx.x == 4009) ? 4096 : 0) + wave * 128;
+        for (int a = 0; a < 16; ++a)
+            for (int c = 0; c < 7; ++c) dbg[a * 8 + c] = (a < total_tiles) ? tl[a][c] : 0ull;
+        dbg[7] = (unsigned long long)total_tiles;
+    }
+#endif
 
     // ---- epilogue: O = O^T / l, transposed through LDS so that every global store is a contiguous run --------
     // (all wavefronts left the loop through its final barrier; each one now uses a private region of the stages)
@@ -609,8 +692,9 @@ extern "C" int splat_attention_fwd(const void* q, int64_t q_sb, int64_t q_sh, in
     if (d != 64 && d != 128) return fail(SPLAT_E_UNSUPPORTED, "splat_attention_fwd: head dim must be 64 or 128 (got %d)", d);
     if (dtype != SPLAT_F32 && dtype != SPLAT_F16 && dtype != SPLAT_BF16)
         return fail(SPLAT_E_DTYPE, "splat_attention_fwd: unknown dtype %d", dtype);
-    // the running max is taken over unscaled scores, which orders them correctly only for scale >= 0
-    if (!(scale >= 0.f)) return fail(SPLAT_E_UNSUPPORTED, "splat_attention_fwd: scale must be >= 0 (got %g)", (double)scale);
+    // the running max is taken over unscaled scores (needs scale >= 0) and masked scores are zeroed through
+    // the underflow of exp2(-1e30 * scale) (needs scale > 0)
+    if (!(scale > 0.f)) return fail(SPLAT_E_UNSUPPORTED, "splat_attention_fwd: scale must be > 0 (got %g)", (double)scale);
     const int es = dtype == SPLAT_F32 ? 4 : 2;
     const int epc = 16 / es;
     bool kt;
