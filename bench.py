@@ -24,8 +24,8 @@ for _p in (ROOT, os.path.join(ROOT, "triton-fun_amd", "SPLAT")):
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes one fused launch moves at config 5, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
-# copy kernel of known size (see profiles/attention_fwd_cfg5_pmc.md); None until measured.
-FUSED_TRAFFIC_BYTES = None
+# copy kernel of known size (profiles/attn_fwd_kernel_cfg5_hbm_traffic.md).
+FUSED_TRAFFIC_BYTES = 1.503e9
 
 
 def causal_window_nnz(L: int, w: int) -> int:
@@ -124,7 +124,7 @@ def main() -> int:
                    "B": B, "H": H, "L": L, "d": d, "window": w, "nnz_per_head": nnz},
         "roofline": {"bound": "mfma", "achieved": round(kern_tflops, 2), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(kern_tflops / MFMA_PEAK_TFLOPS, 4), "traffic": FUSED_TRAFFIC_BYTES,
-                     "kernel": "attn_fwd_kernel<bf16,128,2,false>", "kernel_ms_avg": round(kern_ms, 4),
+                     "kernel": "attn_fwd_kernel<bf16,128,1,false>", "kernel_ms_avg": round(kern_ms, 4),
                      "kernel_ms_min": round(per[0], 4), "algorithmic_flops": flops, "algorithmic_bytes": io_bytes,
                      "hbm_frac_at_algorithmic_bytes": round(io_bytes / (kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
         "fwd_ms": round(kern_ms, 4),
