@@ -71,7 +71,9 @@ typedef struct splat_acsr_seg {
                                  row.  Used for rows with exactly one live column, whose stored
                                  translation acsr_helpers.py:126-130 hard-codes to 0.   */
     int32_t slot_offset;     /* first compressed slot of this segment (0 for one segment) */
-    int32_t reserved;
+    int32_t row_stride_hint; /* 0 or 1: none.  n > 1: every row's column step is n and its first column is
+                                congruent to the row index modulo n (splat_acsr_build reports this in
+                                summary[2..4]); kernels then group rows by phase.  Only affects speed. */
 } splat_acsr_seg;
 
 int splat_version(void);
@@ -87,7 +89,10 @@ const char* splat_last_error(void);
  *                      splat_acsr_seg.first_col are derived from them
  *   summary            [8] int32 output: [0] T = max row sum (acsr_helpers.py:153), [1] number of
  *                      rows that trip the reference's "Incorrect unpacking of affine-indices."
- *                      assertion (nnz > 1 but fewer than two entries equal to 1), [2..7] reserved.
+ *                      assertion (nnz > 1 but fewer than two entries equal to 1), [2] / [3] smallest / largest column
+ *                      step over rows with nnz > 1 (INT32_MAX / 0 when there is none), [4] number of rows with
+ *                      nnz > 1 whose first column is not congruent to the row index modulo the row's step,
+ *                      [5..7] reserved.
  * Reads rows*ld bytes once; the caller reads `summary` back after synchronising the stream. */
 int splat_acsr_build(const uint8_t* mask, int64_t rows, int64_t cols, int64_t ld,
                      int32_t block_height, float* dTos_lin, float* dTos_trans, float* sTod_lin,

@@ -29,7 +29,7 @@ class SplatError(RuntimeError):
 class AcsrSeg(ctypes.Structure):
     _fields_ = [("dTos_lin", ctypes.c_void_p), ("dTos_trans", ctypes.c_void_p), ("sTod_lin", ctypes.c_void_p),
                 ("sTod_trans", ctypes.c_void_p), ("nnz", ctypes.c_void_p), ("first_col", ctypes.c_void_p),
-                ("slot_offset", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+                ("slot_offset", ctypes.c_int32), ("row_stride_hint", ctypes.c_int32)]
 
 
 _lib = None
@@ -104,7 +104,8 @@ def require_device_tensor(t: torch.Tensor, name: str) -> None:
 
 
 def seg_array(segments: Sequence[tuple]) -> Any:
-    """segments: (dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnzs, first_col | None, slot_offset)."""
+    """segments: (dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnzs, first_col | None, slot_offset); the row-stride
+    hint is read from the attribute ``splat_row_stride`` of sTod_trans when the builder attached one."""
     if not 1 <= len(segments) <= MAX_SEGMENTS:
         raise SplatError(f"between 1 and {MAX_SEGMENTS} ACSR segments are supported (got {len(segments)})")
     arr = (AcsrSeg * len(segments))()
@@ -117,5 +118,5 @@ def seg_array(segments: Sequence[tuple]) -> Any:
         arr[i].sTod_lin, arr[i].sTod_trans, arr[i].nnz = c.data_ptr(), d.data_ptr(), n.data_ptr()
         arr[i].first_col = fc.data_ptr() if fc is not None else None
         arr[i].slot_offset = int(off)
-        arr[i].reserved = 0
+        arr[i].row_stride_hint = int(getattr(d, "splat_row_stride", 1))
     return arr

@@ -207,7 +207,7 @@ def mask_shape(mask) -> tuple[int, int]:
 class AcsrBuild:
     """Everything one ``splat_acsr_build`` call produced for (mask, BLOCK_HEIGHT)."""
     __slots__ = ("dTos_lin", "dTos_trans", "sTod_lin", "sTod_trans", "nnz", "T", "span_start", "span_end",
-                 "row_first", "row_last")
+                 "row_first", "row_last", "row_stride")
 
 
 def build_acsr(mask, BLOCK_HEIGHT: int, dev: torch.device) -> AcsrBuild:
@@ -236,6 +236,8 @@ def build_acsr(mask, BLOCK_HEIGHT: int, dev: torch.device) -> AcsrBuild:
     host = summary.cpu()  # the one synchronisation: T is returned as a Python int, like the reference
     assert int(host[1]) == 0, "Incorrect unpacking of affine-indices."
     b.T = int(host[0])
+    # rows whose columns step by n and start in phase with the row index (dilated windows): kernels group them by phase
+    b.row_stride = int(host[2]) if (int(host[2]) == int(host[3]) and int(host[3]) > 1 and int(host[4]) == 0) else 1
     entry.builds[BLOCK_HEIGHT] = b
     return b
 
@@ -257,10 +259,12 @@ def create_acsr(mask, BLOCK_HEIGHT: int, GPU_ID: Any):
 
     The returned ``sTod_translations`` tensor carries an attribute ``splat_first_col`` (int32 tensor, first
     live column per row) that the launchers pick up: rows with a single live column store translation 0
-    whatever that column is, so the column itself has to travel separately."""
+    whatever that column is, so the column itself has to travel separately.  ``splat_row_stride`` (int) is a speed
+    hint for patterns whose rows alternate column phase."""
     dev = _hip.resolve_device(GPU_ID)
     b = build_acsr(mask, BLOCK_HEIGHT, dev)
     b.sTod_trans.splat_first_col = b.row_first
+    b.sTod_trans.splat_row_stride = b.row_stride
     return (b.dTos_lin, b.dTos_trans, b.sTod_lin, b.sTod_trans, b.nnz, b.T, b.span_start, b.span_end)
 
 

@@ -1,6 +1,7 @@
 // ACSR builder and mask generators.
 //
-// splat_acsr_build: one wavefront per mask row streams the row once (16-byte loads), reducing the
+// splat_acsr_build: one wavefront (short rows) or one workgroup (rows >= 4 KiB) per mask row streams the row once
+// (16-byte loads), reducing the
 // byte sum (nnz), the first two columns whose byte equals 1 (the affine map's anchors a < b) and the
 // first/last nonzero column.  Lane 0 then evaluates the 2x2 solve of acsr_helpers.py:122 in closed
 // form in double precision and rounds to float32, which is what the reference's
@@ -76,54 +77,14 @@ struct RowScan {
 };
 
 __global__ void acsr_init_summary(int32_t* summary) {
-    if (threadIdx.x < 8) summary[threadIdx.x] = 0;
+    if (threadIdx.x < 8) summary[threadIdx.x] = (threadIdx.x == 2) ? 0x7fffffff : 0;
 }
 
-__global__ __launch_bounds__(256) void acsr_rows_kernel(const uint8_t* __restrict__ mask, int rows, int cols,
-                                                        int64_t ld, int vec_ok, float* __restrict__ dTos_lin,
-                                                        float* __restrict__ dTos_trans, float* __restrict__ sTod_lin,
-                                                        float* __restrict__ sTod_trans, float* __restrict__ nnz_out,
-                                                        int32_t* __restrict__ row_first,
-                                                        int32_t* __restrict__ row_last, int32_t* __restrict__ summary) {
-    const int lane = threadIdx.x & 63;
-    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= rows) return;
-    const uint8_t* p = mask + (int64_t)row * ld;
-    RowScan s;
-    s.init();
-    int done = 0;
-    if (vec_ok) {
-        const int nvec = cols >> 4;
-        const uint4* pv = reinterpret_cast<const uint4*>(p);
-        int i = lane;
-        // four independent 16-byte loads in flight per lane
-        for (; i + 192 < nvec; i += 256) {
-            uint4 x0 = pv[i], x1 = pv[i + 64], x2 = pv[i + 128], x3 = pv[i + 192];
-            const uint4 xs[4] = {x0, x1, x2, x3};
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                int c = (i + 64 * u) << 4;
-                if ((xs[u].x | xs[u].y | xs[u].z | xs[u].w) == 0) continue;
-                s.dword(xs[u].x, c);
-                s.dword(xs[u].y, c + 4);
-                s.dword(xs[u].z, c + 8);
-                s.dword(xs[u].w, c + 12);
-            }
-        }
-        for (; i < nvec; i += 64) {
-            uint4 x = pv[i];
-            int c = i << 4;
-            s.dword(x.x, c);
-            s.dword(x.y, c + 4);
-            s.dword(x.z, c + 8);
-            s.dword(x.w, c + 12);
-        }
-        done = nvec << 4;
-    }
-    for (int c = done + lane; c < cols; c += 64) s.byte(p[c], c);
-    s.wave_reduce();
-    if (lane != 0) return;
-
+// What one row contributes once its scan is reduced: the closed-form 2x2 solve.  (The summary extrema are
+// reduced by the span kernel: per-row atomics on one address cost more than streaming the whole mask.)
+__device__ __forceinline__ void finish_row(const RowScan& s, int row, int cols, float* dTos_lin, float* dTos_trans,
+                                           float* sTod_lin, float* sTod_trans, float* nnz_out, int32_t* row_first,
+                                           int32_t* row_last, int32_t* summary) {
     const int nnz = (int)s.sum;
     double x0 = 1.0, x1 = 0.0;
     int step = 1;
@@ -144,29 +105,144 @@ __global__ __launch_bounds__(256) void acsr_rows_kernel(const uint8_t* __restric
     nnz_out[row] = (float)nnz;
     if (row_first) row_first[row] = (s.first == kInf) ? cols : s.first;
     if (row_last) row_last[row] = s.last;
-    atomicMax(&summary[0], nnz);
+}
+
+__device__ __forceinline__ void scan_chunk(RowScan& s, const u32x4& x, int c) {
+    if ((x.x | x.y | x.z | x.w) == 0) return;
+    s.dword(x.x, c);
+    s.dword(x.y, c + 4);
+    s.dword(x.z, c + 8);
+    s.dword(x.w, c + 12);
+}
+
+// Short rows: one wavefront per row, four rows per workgroup.
+__global__ __launch_bounds__(256) void acsr_rows_kernel(const uint8_t* __restrict__ mask, int rows, int cols,
+                                                        int64_t ld, int vec_ok, float* __restrict__ dTos_lin,
+                                                        float* __restrict__ dTos_trans, float* __restrict__ sTod_lin,
+                                                        float* __restrict__ sTod_trans, float* __restrict__ nnz_out,
+                                                        int32_t* __restrict__ row_first,
+                                                        int32_t* __restrict__ row_last, int32_t* __restrict__ summary) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const uint8_t* p = mask + (int64_t)row * ld;
+    RowScan s;
+    s.init();
+    int done = 0;
+    if (vec_ok) {
+        const int nvec = cols >> 4;
+        const u32x4* pv = reinterpret_cast<const u32x4*>(p);
+        for (int i = lane; i < nvec; i += 64) scan_chunk(s, pv[i], i << 4);
+        done = nvec << 4;
+    }
+    for (int c = done + lane; c < cols; c += 64) s.byte(p[c], c);
+    s.wave_reduce();
+    if (lane == 0) finish_row(s, row, cols, dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnz_out, row_first, row_last, summary);
+}
+
+// Long rows (>= 4 KiB, 16-byte aligned): one workgroup per row, so that the memory system sees a few thousand
+// sequential 4 KiB-wide streams instead of tens of thousands of 1 KiB-wide ones; up to 8 loads in flight per lane.
+__global__ __launch_bounds__(256) void acsr_rows_wide_kernel(const uint8_t* __restrict__ mask, int rows, int cols,
+                                                             int64_t ld, float* __restrict__ dTos_lin,
+                                                             float* __restrict__ dTos_trans, float* __restrict__ sTod_lin,
+                                                             float* __restrict__ sTod_trans, float* __restrict__ nnz_out,
+                                                             int32_t* __restrict__ row_first,
+                                                             int32_t* __restrict__ row_last, int32_t* __restrict__ summary) {
+    __shared__ uint32_t s_sum[4];
+    __shared__ int s_m1[4], s_m2[4], s_first[4], s_last[4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int row = blockIdx.x;
+    const uint8_t* p = mask + (int64_t)row * ld;
+    RowScan s;
+    s.init();
+    const int nvec = cols >> 4;
+    const u32x4* pv = reinterpret_cast<const u32x4*>(p);
+    int i = tid;
+    for (; i + 7 * 256 < nvec; i += 8 * 256) {
+        u32x4 xs[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) xs[u] = __builtin_nontemporal_load(pv + i + 256 * u);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) scan_chunk(s, xs[u], (i + 256 * u) << 4);
+    }
+    for (; i + 3 * 256 < nvec; i += 4 * 256) {
+        u32x4 xs[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) xs[u] = __builtin_nontemporal_load(pv + i + 256 * u);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) scan_chunk(s, xs[u], (i + 256 * u) << 4);
+    }
+    for (; i < nvec; i += 256) scan_chunk(s, pv[i], i << 4);
+    for (int c = (nvec << 4) + tid; c < cols; c += 256) s.byte(p[c], c);
+    s.wave_reduce();
+    if (lane == 0) {
+        s_sum[wave] = s.sum;
+        s_m1[wave] = s.m1;
+        s_m2[wave] = s.m2;
+        s_first[wave] = s.first;
+        s_last[wave] = s.last;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        RowScan t;
+        t.init();
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            t.sum += s_sum[w];
+            const int n1 = min(t.m1, s_m1[w]);
+            const int n2 = min(max(t.m1, s_m1[w]), min(t.m2, s_m2[w]));
+            t.m1 = n1;
+            t.m2 = n2;
+            t.first = min(t.first, s_first[w]);
+            t.last = max(t.last, s_last[w]);
+        }
+        finish_row(t, row, cols, dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnz_out, row_first, row_last, summary);
+    }
 }
 
 // One thread per row block: span_start = min(cols, min_r trans_r), span_end = max(-1, max_r nnz_r*lin_r + trans_r)
-// evaluated in double from the exact integers (a, lin, nnz) and rounded once to float32.
-__global__ void acsr_spans_kernel(const float* __restrict__ sTod_lin, const float* __restrict__ sTod_trans,
-                                  const float* __restrict__ nnz, int rows, int cols, int block_height,
-                                  float* __restrict__ span_start, float* __restrict__ span_end) {
+// evaluated in double from the exact integers (a, lin, nnz) and rounded once to float32.  The same pass reduces
+// the summary: T = max nnz, smallest / largest column step over rows with nnz > 1, and how many rows with
+// nnz > 1 have a first column that is not congruent to the row index modulo their step.
+__global__ __launch_bounds__(256) void acsr_spans_kernel(const float* __restrict__ sTod_lin,
+                                                         const float* __restrict__ sTod_trans,
+                                                         const float* __restrict__ nnz, int rows, int cols,
+                                                         int block_height, float* __restrict__ span_start,
+                                                         float* __restrict__ span_end, int32_t* __restrict__ summary) {
     const int g = blockIdx.x * blockDim.x + threadIdx.x;
     const int n_blocks = (rows + block_height - 1) / block_height;
-    if (g >= n_blocks) return;
-    double lo = (double)cols, hi = -1.0;
-    const int r1 = min(rows, (g + 1) * block_height);
-    for (int r = g * block_height; r < r1; ++r) {
-        const float linf = sTod_lin[r];
-        const int lin = (int)linf;
-        const int a = (int)rintf(linf * sTod_trans[r]);
-        const double t = (double)a / (double)lin;
-        lo = fmin(lo, t);
-        hi = fmax(hi, (double)((int64_t)nnz[r] * lin) + t);
+    int t_max = 0, step_min = 0x7fffffff, step_max = 0, off_phase = 0;
+    if (g < n_blocks) {
+        double lo = (double)cols, hi = -1.0;
+        const int r1 = min(rows, (g + 1) * block_height);
+        for (int r = g * block_height; r < r1; ++r) {
+            const float linf = sTod_lin[r];
+            const int lin = (int)linf;
+            const int a = (int)rintf(linf * sTod_trans[r]);
+            const int cnt = (int)nnz[r];
+            const double t = (double)a / (double)lin;
+            lo = fmin(lo, t);
+            hi = fmax(hi, (double)((int64_t)cnt * lin) + t);
+            t_max = max(t_max, cnt);
+            if (cnt > 1) {
+                step_min = min(step_min, lin);
+                step_max = max(step_max, lin);
+                off_phase += ((a - r) % lin) != 0;
+            }
+        }
+        span_start[g] = (float)lo;
+        span_end[g] = (float)hi;
     }
-    span_start[g] = (float)lo;
-    span_end[g] = (float)hi;
+    t_max = wave_max_i(t_max);
+    step_min = wave_min_i(step_min);
+    step_max = wave_max_i(step_max);
+    off_phase = (int)wave_sum((float)off_phase);  // at most 64 * block_height per wavefront: exact in float
+    if ((threadIdx.x & 63) == 0) {
+        atomicMax(&summary[0], t_max);
+        atomicMin(&summary[2], step_min);
+        atomicMax(&summary[3], step_max);
+        if (off_phase) atomicAdd(&summary[4], off_phase);
+    }
 }
 
 __device__ __forceinline__ bool mask_pred(int pattern, int64_t i, int64_t j, int64_t p0, int64_t p1) {
@@ -233,11 +309,15 @@ extern "C" int splat_acsr_build(const uint8_t* mask, int64_t rows, int64_t cols,
     hipStream_t st = (hipStream_t)stream;
     const int vec_ok = ((reinterpret_cast<uintptr_t>(mask) & 15) == 0 && (ld & 15) == 0) ? 1 : 0;
     acsr_init_summary<<<1, 64, 0, st>>>(summary);
-    acsr_rows_kernel<<<(unsigned)((rows + 3) / 4), 256, 0, st>>>(mask, (int)rows, (int)cols, ld, vec_ok, dTos_lin, dTos_trans,
-                                                                 sTod_lin, sTod_trans, nnz, row_first, row_last, summary);
+    if (vec_ok && cols >= 4096)
+        acsr_rows_wide_kernel<<<(unsigned)rows, 256, 0, st>>>(mask, (int)rows, (int)cols, ld, dTos_lin, dTos_trans, sTod_lin,
+                                                              sTod_trans, nnz, row_first, row_last, summary);
+    else
+        acsr_rows_kernel<<<(unsigned)((rows + 3) / 4), 256, 0, st>>>(mask, (int)rows, (int)cols, ld, vec_ok, dTos_lin, dTos_trans,
+                                                                     sTod_lin, sTod_trans, nnz, row_first, row_last, summary);
     const int n_blocks = (int)((rows + block_height - 1) / block_height);
     acsr_spans_kernel<<<(n_blocks + 255) / 256, 256, 0, st>>>(sTod_lin, sTod_trans, nnz, (int)rows, (int)cols, block_height,
-                                                               span_start, span_end);
+                                                               span_start, span_end, summary);
     return check_launch("splat_acsr_build");
 }
 

@@ -49,19 +49,19 @@ __device__ __forceinline__ RowMap cached_row_map(const PlanScratch<BM>* ps, int 
     return m;
 }
 
-// Gather the maps of rows [r0, r0+BM) of every segment into LDS and reduce what the plans need.  Called by
+// Gather the maps of rows r0 + rs*k, k in [0, BM), of every segment into LDS and reduce what the plans need.  Called by
 // all 256 threads of the workgroup (BM <= 256: one row per thread); contains two barriers.  Afterwards
 // segment_plan() may be evaluated by any thread.
 template <int BM>
-__device__ __forceinline__ void gather_row_maps(const SegPtrs* seg, int n_seg, int r0, int n_rows, PlanScratch<BM>* ps,
-                                                int tid) {
+__device__ __forceinline__ void gather_row_maps(const SegPtrs* seg, int n_seg, int r0, int rs, int n_rows,
+                                                PlanScratch<BM>* ps, int tid) {
     static_assert(BM <= 256, "one row per thread");
     const int lane = tid & 63, wave = tid >> 6;
     RowMap mine[SPLAT_MAX_SEGMENTS];
 #pragma unroll
     for (int sg = 0; sg < SPLAT_MAX_SEGMENTS; ++sg) {
         RowMap m = {0, 1, 0};
-        if (sg < n_seg && tid < BM && r0 + tid < n_rows) m = load_row_map(seg[sg], r0 + tid);
+        if (sg < n_seg && tid < BM && r0 + rs * tid < n_rows) m = load_row_map(seg[sg], r0 + rs * tid);
         mine[sg] = m;
         if (sg < n_seg) {
             if (tid < BM) {
@@ -136,11 +136,24 @@ __device__ __forceinline__ SegPlan segment_plan(const PlanScratch<BM>* ps, int s
 
 // gather_row_maps + one SegPlan per segment in LDS (plan[0..n_seg)); ends with a barrier.
 template <int BM>
-__device__ __forceinline__ void plan_segments(const SegPtrs* seg, int n_seg, int r0, int n_rows, bool allow_gather,
-                                              SegPlan* plan, PlanScratch<BM>* ps, int tid) {
-    gather_row_maps<BM>(seg, n_seg, r0, n_rows, ps, tid);
+__device__ __forceinline__ void plan_segments(const SegPtrs* seg, int n_seg, int r0, int rs, int n_rows,
+                                              bool allow_gather, SegPlan* plan, PlanScratch<BM>* ps, int tid) {
+    gather_row_maps<BM>(seg, n_seg, r0, rs, n_rows, ps, tid);
     if (tid < n_seg) plan[tid] = segment_plan<BM>(ps, tid, allow_gather);
     __syncthreads();
+}
+
+// Row blocks.  With row stride rs a workgroup owns the BM rows first + rs*k: the rows of one column phase out
+// of BM*rs consecutive ones (rs = 1: BM consecutive rows).  Patterns whose rows alternate phase (dilated
+// windows) then get uniform plans.  Block index -> first row.
+__device__ __forceinline__ int block_first_row(int block, int BM, int rs) { return (block / rs) * BM * rs + (block % rs); }
+inline int count_row_blocks(int n_rows, int BM, int rs) { return ((n_rows + BM * rs - 1) / (BM * rs)) * rs; }
+// The row stride the segments agree on (their hints are equal and > 1), else 1.
+inline int common_row_stride(const splat_acsr_seg* segs, int n_seg) {
+    int rs = segs[0].row_stride_hint;
+    for (int k = 1; k < n_seg; ++k)
+        if (segs[k].row_stride_hint != rs) return 1;
+    return (rs > 1 && rs <= 64) ? rs : 1;
 }
 
 // How one row tests a tile position j (relative to the plan's c0/cs).

@@ -40,6 +40,7 @@ struct AttnParams {
     SegPtrs seg[SPLAT_MAX_SEGMENTS];
     int n_row_blocks;
     int total;
+    int row_stride;
 };
 
 template <typename T, int D, bool KT>
@@ -230,7 +231,8 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
     // later row blocks of causal patterns carry the most keys: hand them out first
     const int rb = p.n_row_blocks - 1 - (logical % p.n_row_blocks);
     const int b = bh / p.H, h = bh % p.H;
-    const int r0 = rb * BM;
+    const int rs = p.row_stride;
+    const int r0 = block_first_row(rb, BM, rs);
     const int L = p.L;
 
     const T* qb = (const T*)p.q + b * p.q_sb + h * p.q_sh;
@@ -239,7 +241,7 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
     T* ob = (T*)p.o + b * p.o_sb + h * p.o_sh;
 
     // ---- plan: per segment, the column range and step of this row block ------------------------
-    plan_segments<BM>(p.seg, p.n_seg, r0, L, !KT, s_plan, &s_ps, tid);
+    plan_segments<BM>(p.seg, p.n_seg, r0, rs, L, !KT, s_plan, &s_ps, tid);
 
     if (SPLAT_EXP & 128) return;
     int total_tiles = 0;
@@ -360,7 +362,7 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
     int my_row[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-        my_row[mt] = r0 + (wave * MT + mt) * 32 + lm;
+        my_row[mt] = r0 + rs * ((wave * MT + mt) * 32 + lm);
         const T* qr = qb + (int64_t)min(my_row[mt], L - 1) * p.q_sl;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) qf[mt][ks] = global_frag<T>(qr + 16 * ks + 8 * g);
@@ -635,7 +637,7 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
                 for (int i = 0; i < 32 * CPR / 64; ++i) {
                     const int flat = i * 64 + lane;
                     const int row = flat / CPR, c = flat % CPR;
-                    const int r = r0 + (wave * MT + mt) * 32 + row;
+                    const int r = r0 + rs * ((wave * MT + mt) * 32 + row);
                     const u32x4 val = *reinterpret_cast<const u32x4*>(stg + row * OROW + c * 16);
                     if (r < L) *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(ob + (int64_t)r * p.o_sl) + c * 16) = val;
                 }
@@ -650,7 +652,7 @@ static int launch_attn(const AttnParams& p0, hipStream_t st) {
     using G = TileGeom<T, D, KT>;
     AttnParams p = p0;
     constexpr int BM = 128 * MT;
-    p.n_row_blocks = (p.L + BM - 1) / BM;
+    p.n_row_blocks = count_row_blocks(p.L, BM, p.row_stride);
     p.total = p.B * p.H * p.n_row_blocks;
     const int grid = ((p.total + 7) / 8) * 8;
     const size_t lds = 2 * (size_t)G::STAGE;
@@ -725,6 +727,7 @@ extern "C" int splat_attention_fwd(const void* q, int64_t q_sb, int64_t q_sh, in
     p.scale_log2e = scale * 1.4426950408889634f;
     p.n_seg = n_seg;
     if (int rc = fill_segs("splat_attention_fwd", segs, n_seg, p.seg, -1)) return rc;
+    p.row_stride = common_row_stride(segs, n_seg);
     hipStream_t st = (hipStream_t)stream;
     switch (dtype) {
         case SPLAT_F32: return dispatch_attn<float>(p, d, kt, st);

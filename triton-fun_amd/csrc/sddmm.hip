@@ -27,6 +27,7 @@ struct SddmmParams {
     SegPtrs seg[SPLAT_MAX_SEGMENTS];
     int n_row_blocks, total;
     int q_vec, k_vec;  // 16-byte loads are legal for q / k
+    int row_stride;
 };
 
 // 8 consecutive contraction values of one row from global memory, zero beyond `d`.
@@ -65,7 +66,8 @@ __global__ __launch_bounds__(256) void sddmm_kernel(const SddmmParams p) {
     const int bh = logical / p.n_row_blocks;
     const int rb = logical % p.n_row_blocks;
     const int b = bh / p.H, h = bh % p.H;
-    const int r0 = rb * BM;
+    const int rs = p.row_stride;
+    const int r0 = block_first_row(rb, BM, rs);
     const int L = p.L, d = p.d;
 
     const T* qb = (const T*)p.q + b * p.q_sb + h * p.q_sh;
@@ -75,10 +77,10 @@ __global__ __launch_bounds__(256) void sddmm_kernel(const SddmmParams p) {
 #pragma unroll
         for (int k = 0; k < SPLAT_MAX_SEGMENTS; ++k) s_seg[k] = p.seg[k];
     }
-    plan_segments<BM>(p.seg, p.n_seg, r0, L, !KT, s_plan, &s_ps, tid);
+    plan_segments<BM>(p.seg, p.n_seg, r0, rs, L, !KT, s_plan, &s_ps, tid);
 
     // A-operand rows of this lane: query row 32*wave + lm of the block
-    const int q_row = min(r0 + 32 * wave + lm, L - 1);
+    const int q_row = min(r0 + rs * (32 * wave + lm), L - 1);
     const T* qr = qb + (int64_t)q_row * p.q_sl;
     Frag<T> qf[QF];
     if constexpr (QREG) {
@@ -181,7 +183,7 @@ __global__ __launch_bounds__(256) void sddmm_kernel(const SddmmParams p) {
             // ---- scatter the live positions to their compressed slots ----
 #pragma unroll
             for (int j = 0; j < 16; ++j) {
-                const int r = r0 + 32 * wave + acc_row(j, g);
+                const int r = r0 + rs * (32 * wave + acc_row(j, g));
                 const int64_t row_base = ((int64_t)bh * L + r) * p.T + off;
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
@@ -195,7 +197,7 @@ __global__ __launch_bounds__(256) void sddmm_kernel(const SddmmParams p) {
 
 template <typename T>
 static int launch_sddmm(SddmmParams p, bool kt, hipStream_t st) {
-    p.n_row_blocks = (p.L + 127) / 128;
+    p.n_row_blocks = count_row_blocks(p.L, 128, p.row_stride);
     p.total = p.B * p.H * p.n_row_blocks;
     const int grid = ((p.total + 7) / 8) * 8;
     const bool qreg = p.d <= 128;
@@ -241,6 +243,7 @@ extern "C" int splat_sddmm(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_
     p.out_dtype = out_dtype;
     p.n_seg = n_seg;
     if (int rc = fill_segs("splat_sddmm", segs, n_seg, p.seg, T)) return rc;
+    p.row_stride = common_row_stride(segs, n_seg);
     const int es = in_dtype == SPLAT_F32 ? 4 : 2;
     const int epc = 16 / es;
     auto al = [&](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };

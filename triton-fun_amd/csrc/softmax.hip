@@ -66,7 +66,6 @@ __global__ __launch_bounds__(256) void softmax_rows_vec(const Tin* __restrict__ 
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= n_rows) return;
     LiveRanges lr;
-    lr.load(segs, (int)(row % L), T);
     const Tin* xr = x + row * (int64_t)T;
     Tout* yr = y + row * (int64_t)T;
     const int nchunk = T >> 3;
@@ -74,12 +73,21 @@ __global__ __launch_bounds__(256) void softmax_rows_vec(const Tin* __restrict__ 
     float v[NCH][8];
     uint32_t live[NCH];
     float mx = kNegBig;
+    // the loads do not wait for the row's live counts: a chunk inside the row is fetched whole and the dead
+    // slots in it are discarded afterwards
+    vin raw[NCH];
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int ch = lane + 64 * c;
+        if (ch < nchunk) raw[c] = __builtin_nontemporal_load(reinterpret_cast<const vin*>(xr + (ch << 3)));
+    }
+    lr.load(segs, (int)(row % L), T);
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
         const int ch = lane + 64 * c;
         live[c] = (ch < nchunk) ? lr.live8(ch << 3) : 0u;
         if (live[c]) {
-            vin t = *reinterpret_cast<const vin*>(xr + (ch << 3));
+            const vin t = raw[c];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 v[c][e] = ((live[c] >> e) & 1u) ? (float)t[e] : kNegBig;

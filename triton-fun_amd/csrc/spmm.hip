@@ -22,6 +22,7 @@ struct SpmmParams {
     SegPtrs seg[SPLAT_MAX_SEGMENTS];
     int n_row_blocks, total, n_col_chunks;
     int v_vec;
+    int row_stride;
 };
 
 template <typename T, int DVT>
@@ -49,7 +50,8 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
     const int bh = rest / p.n_row_blocks;
     const int rb = rest % p.n_row_blocks;
     const int b = bh / p.H, h = bh % p.H;
-    const int r0 = rb * BM;
+    const int rs = p.row_stride;
+    const int r0 = block_first_row(rb, BM, rs);
     const int L = p.L;
     const int col0 = cchunk * DVC;
 
@@ -60,9 +62,9 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
 #pragma unroll
         for (int k = 0; k < SPLAT_MAX_SEGMENTS; ++k) s_seg[k] = p.seg[k];
     }
-    plan_segments<BM>(p.seg, p.n_seg, r0, L, true, s_plan, &s_ps, tid);
+    plan_segments<BM>(p.seg, p.n_seg, r0, rs, L, true, s_plan, &s_ps, tid);
 
-    const int my_row = r0 + 32 * wave + lm;  // A-operand row of this lane
+    const int my_row = r0 + rs * (32 * wave + lm);  // A-operand row of this lane
     const T* prow = pb + (int64_t)min(my_row, L - 1) * p.T;
 
     f32x16 acc[DVT];
@@ -126,7 +128,7 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
 
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
-        const int r = r0 + 32 * wave + acc_row(j, g);
+        const int r = r0 + rs * (32 * wave + acc_row(j, g));
         if (r < L) {
             const int64_t base = ((int64_t)bh * L + r) * p.n_out;
 #pragma unroll
@@ -140,7 +142,7 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
 
 template <typename T>
 static int launch_spmm(SpmmParams p, hipStream_t st) {
-    p.n_row_blocks = (p.L + 127) / 128;
+    p.n_row_blocks = count_row_blocks(p.L, 128, p.row_stride);
     const int dvt = p.n_out > 64 ? 4 : (p.n_out > 32 ? 2 : 1);
     p.n_col_chunks = (p.n_out + 32 * dvt - 1) / (32 * dvt);
     const int64_t total = (int64_t)p.B * p.H * p.n_row_blocks * p.n_col_chunks;
@@ -179,6 +181,7 @@ extern "C" int splat_spmm(const void* pp, const void* v, int64_t v_sb, int64_t v
     p.out_dtype = out_dtype;
     p.n_seg = n_seg;
     if (int rc = fill_segs("splat_spmm", segs, n_seg, p.seg, T)) return rc;
+    p.row_stride = common_row_stride(segs, n_seg);
     const int es = in_dtype == SPLAT_F32 ? 4 : 2;
     const int epc = 16 / es;
     p.v_vec = ((reinterpret_cast<uintptr_t>(v) & 15) == 0 && v_sb % epc == 0 && v_sh % epc == 0 && v_sl % epc == 0) ? 1 : 0;
