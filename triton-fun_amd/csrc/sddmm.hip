@@ -1,18 +1,18 @@
 // SDDMM on ACSR: out[bh, r, off + s] = scale * <q[bh, r, :], K[bh, c(r, s), :]> for the live slots only.
 //
-// A workgroup of 4 wavefronts owns 128 consecutive rows of one (batch, head); wavefront w owns rows
-// 32w..32w+31.  The key positions its rows' spans cover are walked in tiles of 64 (see acsr_plan.hpp);
-// K is staged through LDS in chunks of 64 contraction values, Q fragments stay in registers when the
-// head dimension is <= 128 and are re-read from cache otherwise.  Scores are produced with 32x32x16
-// MFMA in the orientation rows = queries, columns = keys, so that the 32 lanes of a half-wavefront hold
-// 32 consecutive key positions of one row: with a uniform plan these are consecutive compressed slots
-// and every store instruction writes two contiguous runs.  Dead positions are never stored.
-// The kernel is bound by the compressed output (HBM), not by MFMA: 2*d flops per 2-4 output bytes.
+// A workgroup of 4 wavefronts owns 128 rows of one (batch, head) (rows first + rs*k, see acsr_plan.hpp);
+// wavefront w owns rows 32w..32w+31 of the block.  The key positions its rows' spans cover are walked in tiles
+// of 64.  Per tile the K rows are staged in LDS in chunks of DC contraction values (128 for 16-bit types, 64 for
+// fp32; the copy of the next chunk is issued to registers before the math of the current one); Q fragments
+// stay in registers when d <= DC and are re-read from cache otherwise.  Scores are produced transposed (rows =
+// keys, columns = queries, 32x32x16 MFMA) so that one lane owns one query row; each 32-key half tile is then
+// turned around in a per-wavefront LDS staging area so that a lane writes 8 consecutive positions of one row:
+// with a uniform plan these are 8 consecutive compressed slots, one 16-byte store (any alignment).  Dead
+// positions are never stored.  The kernel is bound by the compressed output (HBM), not by MFMA: 2*d flops per
+// 2-4 output bytes.
 #include "acsr_plan.hpp"
 
 namespace splat {
-
-constexpr int kDC = 64;  // contraction values per LDS chunk
 
 struct SddmmParams {
     const void* q;
@@ -30,6 +30,11 @@ struct SddmmParams {
     int row_stride;
 };
 
+template <typename T>
+struct SddmmGeom {
+    static constexpr int DC = sizeof(T) == 2 ? 128 : 64;  // contraction values per LDS chunk
+};
+
 // 8 consecutive contraction values of one row from global memory, zero beyond `d`.
 template <typename T>
 __device__ __forceinline__ Frag<T> load_q_frag(const T* row, int k0, int d, bool vec) {
@@ -41,21 +46,23 @@ __device__ __forceinline__ Frag<T> load_q_frag(const T* row, int k0, int d, bool
 }
 
 template <typename T, bool KT, bool QREG>
-__global__ __launch_bounds__(256) void sddmm_kernel(const SddmmParams p) {
+__global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
     constexpr int ES = sizeof(T);
     constexpr int BM = 128;
     constexpr int NT = kBN / 32;
-    constexpr int KSC = kDC / 16;                                       // MFMA steps per chunk
-    constexpr int K_ROW = KT ? (kBN * ES + 64) : (kDC * ES + 16);       // bytes per LDS row
-    constexpr int K_ROWS = KT ? kDC : kBN;
+    constexpr int DC = SddmmGeom<T>::DC;
+    constexpr int KSC = DC / 16;                                  // MFMA steps per chunk
+    constexpr int K_ROW = KT ? (kBN * ES + 64) : (DC * ES + 16);  // bytes per LDS row
+    constexpr int K_ROWS = KT ? DC : kBN;
     constexpr int EPC = 16 / ES;
-    constexpr int CPT = kBN * kDC * ES / 16 / 256;                      // 16-byte chunks per thread
-    constexpr int CR = KT ? (kBN * ES / 16) : (kDC * ES / 16);          // chunks per LDS row
-    constexpr int QF = QREG ? 8 : 1;
+    constexpr int CPT = kBN * DC * ES / 16 / 256;                 // 16-byte chunks per thread
+    constexpr int CR = KT ? (kBN * ES / 16) : (DC * ES / 16);     // chunks per LDS row
+    constexpr int S_ROW = 32 * 4 + 16;                            // staging row: 32 floats + pad
 
     __shared__ __attribute__((aligned(16))) char s_k[K_ROW * K_ROWS];
+    __shared__ __attribute__((aligned(16))) char s_stage[4][32 * S_ROW];
     __shared__ SegPlan s_plan[SPLAT_MAX_SEGMENTS];
-    __shared__ SegPtrs s_seg[SPLAT_MAX_SEGMENTS];
+    __shared__ int s_off[SPLAT_MAX_SEGMENTS];
     __shared__ PlanScratch<BM> s_ps;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -75,37 +82,84 @@ __global__ __launch_bounds__(256) void sddmm_kernel(const SddmmParams p) {
 
     if (tid == 0) {
 #pragma unroll
-        for (int k = 0; k < SPLAT_MAX_SEGMENTS; ++k) s_seg[k] = p.seg[k];
+        for (int k = 0; k < SPLAT_MAX_SEGMENTS; ++k) s_off[k] = p.seg[k].slot_offset;
     }
     plan_segments<BM>(p.seg, p.n_seg, r0, rs, L, !KT, s_plan, &s_ps, tid);
 
-    // A-operand rows of this lane: query row 32*wave + lm of the block
+    // B-operand row of this lane: query row 32*wave + lm of the block
     const int q_row = min(r0 + rs * (32 * wave + lm), L - 1);
     const T* qr = qb + (int64_t)q_row * p.q_sl;
-    Frag<T> qf[QF];
+    Frag<T> qf[KSC];
     if constexpr (QREG) {
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) qf[ks] = load_q_frag<T>(qr, 16 * ks + 8 * g, d, p.q_vec != 0);
+        for (int ks = 0; ks < KSC; ++ks) qf[ks] = load_q_frag<T>(qr, 16 * ks + 8 * g, d, p.q_vec != 0);
     }
-    const int n_chunks = (d + kDC - 1) / kDC;
+    const int n_chunks = QREG ? 1 : (d + DC - 1) / DC;
+    const int ks_used = QREG ? (d + 15) / 16 : KSC;  // MFMA steps that hold data when d <= DC
+
+    // one 16-byte piece of the K chunk (positions j0.., contraction values kd0..) for this thread's slot i
+    auto load_piece = [&](const SegPlan& pl, int j0, int kd0, int i) {
+        const int idx = tid + 256 * i;
+        const int row = idx / CR, cc = idx % CR;
+        u32x4 val = {0u, 0u, 0u, 0u};
+        if constexpr (KT) {
+            // LDS row = contraction index, columns = key positions (dense walk, cs == 1)
+            const int kd = kd0 + row;
+            const int c = pl.c0 + j0 + cc * EPC;
+            if (kd < d) {
+                const T* src = kb + (int64_t)kd * p.k_sd;
+                if (p.k_vec && c + EPC <= p.n_keys) {
+                    val = *reinterpret_cast<const u32x4*>(src + c);
+                } else {
+                    T tmp[EPC];
+#pragma unroll
+                    for (int e = 0; e < EPC; ++e) tmp[e] = (c + e < p.n_keys) ? src[(int64_t)(c + e) * p.k_sl] : (T)0.f;
+                    __builtin_memcpy(&val, tmp, 16);
+                }
+            }
+        } else {
+            const int n = min(max(pl.c0 + pl.cs * (j0 + row), 0), p.n_keys - 1);
+            const T* src = kb + (int64_t)n * p.k_sl;
+            const int kd = kd0 + cc * EPC;
+            if (p.k_vec && kd + EPC <= d) {
+                val = *reinterpret_cast<const u32x4*>(src + kd);
+            } else if (kd < d) {
+                T tmp[EPC];
+#pragma unroll
+                for (int e = 0; e < EPC; ++e) tmp[e] = (kd + e < d) ? src[(int64_t)(kd + e) * p.k_sd] : (T)0.f;
+                __builtin_memcpy(&val, tmp, 16);
+            }
+        }
+        return val;
+    };
+
+    char* stg = s_stage[wave];
+    const int64_t out_bh = (int64_t)bh * L * p.T;
 
     for (int sg = 0; sg < p.n_seg; ++sg) {
         const SegPlan pl = s_plan[sg];
         if (pl.n_tiles == 0) continue;
-        const int off = s_seg[sg].slot_offset;
-        // the 16 output rows this lane holds (acc_row(j, g)), and the wavefront's span in positions
-        RowWin win[16];
-        int lmin = 0x3fffffff, hmax = -0x3fffffff;
-#pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            win[j] = make_row_win(cached_row_map<BM>(&s_ps, sg, 32 * wave + acc_row(j, g)), pl);
-            if (win[j].cnt > 0) {
-                lmin = min(lmin, win[j].lo);
-                hmax = max(hmax, win[j].lo + win[j].cnt);
-            }
-        }
+        const int off = s_off[sg];
+        // this lane's own row (source of the wavefront's span) and the 2 block rows it writes out
+        const RowWin mine = make_row_win(cached_row_map<BM>(&s_ps, sg, 32 * wave + lm), pl);
+        int lmin = mine.cnt > 0 ? mine.lo : 0x3fffffff;
+        int hmax = mine.cnt > 0 ? mine.lo + mine.cnt : -0x3fffffff;
         lmin = wave_min_i(lmin);
         hmax = wave_max_i(hmax);
+        RowWin wr[2];
+        int64_t wbase[2];
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const int rr = 32 * wave + 16 * c + (lane >> 2);
+            wr[c] = make_row_win(cached_row_map<BM>(&s_ps, sg, rr), pl);
+            const int r = r0 + rs * rr;
+            if (r >= L) wr[c].cnt = 0;
+            wbase[c] = out_bh + (int64_t)r * p.T + off;
+        }
+
+        u32x4 kreg[CPT];
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) kreg[i] = load_piece(pl, 0, 0, i);
 
         for (int tile = 0; tile < pl.n_tiles; ++tile) {
             const int j0 = tile * kBN;
@@ -116,58 +170,34 @@ __global__ __launch_bounds__(256) void sddmm_kernel(const SddmmParams p) {
 #pragma unroll
                 for (int j = 0; j < 16; ++j) acc[nt][j] = 0.f;
 
-            // with Q in registers (d <= 128) the chunk loop has at most 2 trips and is fully unrolled, so that
-            // the register array qf is only ever indexed by constants
-#pragma unroll
-            for (int ch = 0; ch < (QREG ? 2 : n_chunks); ++ch) {
-                if (QREG && ch >= n_chunks) break;
-                const int kd0 = ch * kDC;
+            for (int ch = 0; ch < n_chunks; ++ch) {
+                const int kd0 = ch * DC;
                 __syncthreads();  // previous chunk fully consumed
-                // ---- stage the K chunk: positions j0..j0+63, contraction values kd0..kd0+63 ----
 #pragma unroll
                 for (int i = 0; i < CPT; ++i) {
                     const int idx = tid + 256 * i;
-                    const int row = idx / CR, cc = idx % CR;
-                    u32x4 val = {0u, 0u, 0u, 0u};
-                    if constexpr (KT) {
-                        // LDS row = contraction index, columns = key positions (dense walk, cs == 1)
-                        const int kd = kd0 + row;
-                        const int c = pl.c0 + j0 + cc * EPC;
-                        if (kd < d) {
-                            const T* src = kb + (int64_t)kd * p.k_sd;
-                            if (p.k_vec && c + EPC <= p.n_keys) {
-                                val = *reinterpret_cast<const u32x4*>(src + c);
-                            } else {
-                                T tmp[EPC];
+                    *reinterpret_cast<u32x4*>(s_k + (idx / CR) * K_ROW + (idx % CR) * 16) = kreg[i];
+                }
+                // request the next chunk (of the next tile when this was the last chunk) while this one is used
+                {
+                    const bool last_ch = (ch + 1 == n_chunks);
+                    const int nj0 = last_ch ? j0 + kBN : j0;
+                    const int nkd0 = last_ch ? 0 : kd0 + DC;
+                    if (!(last_ch && tile + 1 == pl.n_tiles)) {
 #pragma unroll
-                                for (int e = 0; e < EPC; ++e) tmp[e] = (c + e < p.n_keys) ? src[(int64_t)(c + e) * p.k_sl] : (T)0.f;
-                                __builtin_memcpy(&val, tmp, 16);
-                            }
-                        }
-                    } else {
-                        const int n = min(max(pl.c0 + pl.cs * (j0 + row), 0), p.n_keys - 1);
-                        const T* src = kb + (int64_t)n * p.k_sl;
-                        const int kd = kd0 + cc * EPC;
-                        if (p.k_vec && kd + EPC <= d) {
-                            val = *reinterpret_cast<const u32x4*>(src + kd);
-                        } else {
-                            T tmp[EPC];
-#pragma unroll
-                            for (int e = 0; e < EPC; ++e) tmp[e] = (kd + e < d) ? src[(int64_t)(kd + e) * p.k_sd] : (T)0.f;
-                            __builtin_memcpy(&val, tmp, 16);
-                        }
+                        for (int i = 0; i < CPT; ++i) kreg[i] = load_piece(pl, nj0, nkd0, i);
                     }
-                    *reinterpret_cast<u32x4*>(s_k + row * K_ROW + cc * 16) = val;
                 }
                 __syncthreads();
                 if (skip) continue;
 #pragma unroll
                 for (int ks = 0; ks < KSC; ++ks) {
-                    Frag<T> a;
+                    if (QREG && ks >= ks_used) break;
+                    Frag<T> qv;
                     if constexpr (QREG)
-                        a = qf[(ch * KSC + ks) & 7];
+                        qv = qf[ks];
                     else
-                        a = load_q_frag<T>(qr, kd0 + 16 * ks + 8 * g, d, p.q_vec != 0);
+                        qv = load_q_frag<T>(qr, kd0 + 16 * ks + 8 * g, d, p.q_vec != 0);
 #pragma unroll
                     for (int nt = 0; nt < NT; ++nt) {
                         Frag<T> kf;
@@ -175,21 +205,56 @@ __global__ __launch_bounds__(256) void sddmm_kernel(const SddmmParams p) {
                             kf = lds_frag_cols<T>(s_k, K_ROW, 16 * ks + 8 * g, 16 * ks + 8 * g + 4, 32 * nt, lane);
                         else
                             kf = lds_frag_rowmajor<T>(s_k + (32 * nt + lm) * K_ROW + (16 * ks + 8 * g) * ES);
-                        mma32(acc[nt], a, kf);
+                        mma32(acc[nt], kf, qv);  // rows = keys, columns = queries
                     }
                 }
             }
             if (skip) continue;
-            // ---- scatter the live positions to their compressed slots ----
+
 #pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                const int r = r0 + rs * (32 * wave + acc_row(j, g));
-                const int64_t row_base = ((int64_t)bh * L + r) * p.T + off;
+            for (int nt = 0; nt < NT; ++nt) {
+                // ---- turn the half tile around: lane (query lm, half g) holds positions 8jq + 4g + {0..3} ----
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
-                    const int jj = j0 + 32 * nt + lm;
-                    if (win_live(win[j], jj)) store_as(p.out, row_base + win_slot(win[j], jj), acc[nt][j] * p.scale, p.out_dtype);
+                for (int jq = 0; jq < 4; ++jq) {
+                    f32x4 v4 = {acc[nt][4 * jq] * p.scale, acc[nt][4 * jq + 1] * p.scale, acc[nt][4 * jq + 2] * p.scale,
+                                acc[nt][4 * jq + 3] * p.scale};
+                    *reinterpret_cast<f32x4*>(stg + lm * S_ROW + (8 * jq + 4 * g) * 4) = v4;
                 }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wavefront's LDS writes are visible to its own reads
+                // ---- lane writes positions 8*(lane%4) .. +7 of block rows 32w + 16c + lane/4 ----
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    const char* src = stg + (16 * c + (lane >> 2)) * S_ROW + (lane & 3) * 32;
+                    const f32x4 a0 = *reinterpret_cast<const f32x4*>(src);
+                    const f32x4 a1 = *reinterpret_cast<const f32x4*>(src + 16);
+                    const float v[8] = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+                    const RowWin& w = wr[c];
+                    const int jj = j0 + 32 * nt + 8 * (lane & 3);
+                    const int u = jj - w.lo;
+                    if (w.lin == 1 && u >= 0 && u + 8 <= w.cnt) {
+                        const int64_t o = wbase[c] + u;
+                        if (p.out_dtype == SPLAT_BF16) {
+                            typedef bf16 v8 __attribute__((ext_vector_type(8)));
+                            v8 t;
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) t[e] = (bf16)v[e];
+                            __builtin_memcpy((bf16*)p.out + o, &t, 16);
+                        } else if (p.out_dtype == SPLAT_F16) {
+                            typedef f16 v8 __attribute__((ext_vector_type(8)));
+                            v8 t;
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) t[e] = (f16)v[e];
+                            __builtin_memcpy((f16*)p.out + o, &t, 16);
+                        } else {
+                            __builtin_memcpy((float*)p.out + o, v, 32);
+                        }
+                    } else if (w.cnt > 0) {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (win_live(w, jj + e)) store_as(p.out, wbase[c] + win_slot(w, jj + e), v[e], p.out_dtype);
+                    }
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // staging reads done before it is overwritten
             }
         }
     }
@@ -200,7 +265,7 @@ static int launch_sddmm(SddmmParams p, bool kt, hipStream_t st) {
     p.n_row_blocks = count_row_blocks(p.L, 128, p.row_stride);
     p.total = p.B * p.H * p.n_row_blocks;
     const int grid = ((p.total + 7) / 8) * 8;
-    const bool qreg = p.d <= 128;
+    const bool qreg = p.d <= SddmmGeom<T>::DC;
     if (kt) {
         if (qreg)
             sddmm_kernel<T, true, true><<<grid, 256, 0, st>>>(p);

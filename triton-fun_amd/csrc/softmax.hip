@@ -57,14 +57,18 @@ struct Vec8 {
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kNegBig = -1.0e30f;
 
-template <typename Tin, typename Tout, int NCH>
+// LPR lanes share one row (64 / LPR rows per wavefront): rows shorter than 512 slots still fill every lane.
+template <typename Tin, typename Tout, int NCH, int LPR>
 __global__ __launch_bounds__(256) void softmax_rows_vec(const Tin* __restrict__ x, Tout* __restrict__ y, SoftmaxSegs segs,
                                                         int64_t n_rows, int L, int T) {
     typedef typename Vec8<Tin>::type vin;
     typedef typename Vec8<Tout>::type vout;
-    const int lane = threadIdx.x & 63;
-    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= n_rows) return;
+    constexpr int RPW = 64 / LPR;  // rows per wavefront
+    const int lane = threadIdx.x & (LPR - 1);
+    const int64_t row_raw = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW + ((threadIdx.x & 63) / LPR);
+    const bool row_ok = row_raw < n_rows;
+    if (RPW == 1 && !row_ok) return;
+    const int64_t row = row_ok ? row_raw : n_rows - 1;  // surplus lane groups shadow the last row and store nothing
     LiveRanges lr;
     const Tin* xr = x + row * (int64_t)T;
     Tout* yr = y + row * (int64_t)T;
@@ -78,13 +82,13 @@ __global__ __launch_bounds__(256) void softmax_rows_vec(const Tin* __restrict__ 
     vin raw[NCH];
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
-        const int ch = lane + 64 * c;
+        const int ch = lane + LPR * c;
         if (ch < nchunk) raw[c] = __builtin_nontemporal_load(reinterpret_cast<const vin*>(xr + (ch << 3)));
     }
     lr.load(segs, (int)(row % L), T);
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
-        const int ch = lane + 64 * c;
+        const int ch = lane + LPR * c;
         live[c] = (ch < nchunk) ? lr.live8(ch << 3) : 0u;
         if (live[c]) {
             const vin t = raw[c];
@@ -95,7 +99,8 @@ __global__ __launch_bounds__(256) void softmax_rows_vec(const Tin* __restrict__ 
             }
         }
     }
-    mx = wave_max(mx);
+#pragma unroll
+    for (int o = LPR / 2; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
     const float mb = mx * kLog2e;
     float sum = 0.f;
 #pragma unroll
@@ -109,12 +114,13 @@ __global__ __launch_bounds__(256) void softmax_rows_vec(const Tin* __restrict__ 
             }
         }
     }
-    sum = wave_sum(sum);
+#pragma unroll
+    for (int o = LPR / 2; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
     const float inv = sum > 0.f ? 1.0f / sum : 0.f;
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
-        if (live[c]) {
-            const int ch = lane + 64 * c;
+        if (live[c] && row_ok) {
+            const int ch = lane + LPR * c;
             if (live[c] == 0xffu) {
                 vout o;
 #pragma unroll
@@ -156,18 +162,24 @@ __global__ __launch_bounds__(256) void softmax_rows_any(const Tin* __restrict__ 
 
 template <typename Tin, typename Tout>
 static int launch_softmax(const void* x, void* y, const SoftmaxSegs& segs, int64_t n_rows, int L, int T, hipStream_t st) {
-    const unsigned grid = (unsigned)((n_rows + 3) / 4);
+    unsigned grid = (unsigned)((n_rows + 3) / 4);
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 31) == 0;
     const Tin* xi = (const Tin*)x;
     Tout* yo = (Tout*)y;
     if (aligned && (T & 7) == 0 && T <= 2048) {
         const int nch = (T / 8 + 63) / 64;
-        if (nch <= 1)
-            softmax_rows_vec<Tin, Tout, 1><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+        if (T <= 128) {
+            grid = (unsigned)((n_rows + 15) / 16);
+            softmax_rows_vec<Tin, Tout, 1, 16><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+        } else if (T <= 256) {
+            grid = (unsigned)((n_rows + 7) / 8);
+            softmax_rows_vec<Tin, Tout, 1, 32><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+        } else if (nch <= 1)
+            softmax_rows_vec<Tin, Tout, 1, 64><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
         else if (nch <= 2)
-            softmax_rows_vec<Tin, Tout, 2><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+            softmax_rows_vec<Tin, Tout, 2, 64><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
         else
-            softmax_rows_vec<Tin, Tout, 4><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+            softmax_rows_vec<Tin, Tout, 4, 64><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
     } else {
         softmax_rows_any<Tin, Tout><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
     }

@@ -26,7 +26,7 @@ struct SpmmParams {
 };
 
 template <typename T, int DVT>
-__global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
+__global__ __launch_bounds__(256, 2) void spmm_kernel(const SpmmParams p) {
     constexpr int ES = sizeof(T);
     constexpr int BM = 128;
     constexpr int DVC = 32 * DVT;           // output columns per workgroup
@@ -35,7 +35,9 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
     constexpr int CR = DVC * ES / 16;       // 16-byte chunks per LDS row
     constexpr int NCHUNK = kBN * CR;        // chunks per tile
 
+    constexpr int P_ROW = kBN * ES + 16;    // bytes per row of the probability staging tile
     __shared__ __attribute__((aligned(16))) char s_v[V_ROW * kBN];
+    __shared__ __attribute__((aligned(16))) char s_p[4][32 * P_ROW];
     __shared__ SegPlan s_plan[SPLAT_MAX_SEGMENTS];
     __shared__ SegPtrs s_seg[SPLAT_MAX_SEGMENTS];
     __shared__ PlanScratch<BM> s_ps;
@@ -77,50 +79,101 @@ __global__ __launch_bounds__(256) void spmm_kernel(const SpmmParams p) {
         const SegPlan pl = s_plan[sg];
         if (pl.n_tiles == 0) continue;
         const int off = s_seg[sg].slot_offset;
+
         const RowWin win = make_row_win(cached_row_map<BM>(&s_ps, sg, 32 * wave + lm), pl);
+        RowWin wr[4];
+        const T* wrow[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int rr = 32 * wave + 8 * c + (lane >> 3);
+            wr[c] = make_row_win(cached_row_map<BM>(&s_ps, sg, rr), pl);
+            const int r = r0 + rs * rr;
+            if (r >= L) wr[c].cnt = 0;
+            wrow[c] = pb + (int64_t)min(r, L - 1) * p.T + off;
+        }
         int lmin = win.cnt > 0 ? win.lo : 0x3fffffff;
         int hmax = win.cnt > 0 ? win.lo + win.cnt : -0x3fffffff;
         lmin = wave_min_i(lmin);
         hmax = wave_max_i(hmax);
 
+        // one 16-byte piece of the V tile at positions j0.. for this thread's slot i
+        auto load_piece = [&](int j0, int i) {
+            const int idx = tid + 256 * i;
+            const int row = idx / CR, cc = idx % CR;
+            const int n = min(max(pl.c0 + pl.cs * (j0 + row), 0), p.n_keys - 1);
+            const T* src = vb + (int64_t)n * p.v_sl;
+            const int c = col0 + cc * EPC;
+            u32x4 val = {0u, 0u, 0u, 0u};
+            if (p.v_vec && c + EPC <= p.n_out) {
+                val = *reinterpret_cast<const u32x4*>(src + c);
+            } else if (c < p.n_out) {
+                T tmp[EPC];
+#pragma unroll
+                for (int e = 0; e < EPC; ++e) tmp[e] = (c + e < p.n_out) ? src[c + e] : (T)0.f;
+                __builtin_memcpy(&val, tmp, 16);
+            }
+            return val;
+        };
+        constexpr int CPT = NCHUNK / 256;
+        static_assert(NCHUNK % 256 == 0, "tile shape");
+        u32x4 vreg[CPT];
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) vreg[i] = load_piece(0, i);
+        // A tile's probabilities: lane (row 8c + lane/8 of the wavefront's 32, piece lane%8) fetches 8 consecutive
+        // positions, so one instruction reads 8 rows x 64 consecutive slots; the pieces are turned into A fragments
+        // (lane = row) through a per-wavefront staging tile.  Requested one tile ahead, like V.
+        typedef T vec8 __attribute__((ext_vector_type(8)));
+        auto load_probs = [&](int j0, int c) {
+            vec8 v;
+            const RowWin& w = wr[c];
+            const int jj = j0 + 8 * (lane & 7);
+            const int u = jj - w.lo;
+            if (w.lin == 1 && u >= 0 && u + 8 <= w.cnt) {
+                __builtin_memcpy(&v, wrow[c] + u, 8 * ES);  // any alignment
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] = win_live(w, jj + e) ? wrow[c][win_slot(w, jj + e)] : (T)0.f;
+            }
+            return v;
+        };
+        vec8 praw[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) praw[c] = load_probs(0, c);
+
         for (int tile = 0; tile < pl.n_tiles; ++tile) {
             const int j0 = tile * kBN;
+            const bool skip = (j0 + kBN <= lmin) || (j0 >= hmax);  // wavefront-uniform
             __syncthreads();  // previous tile fully consumed
-            for (int idx = tid; idx < NCHUNK; idx += 256) {
-                const int row = idx / CR, cc = idx % CR;
-                const int n = min(max(pl.c0 + pl.cs * (j0 + row), 0), p.n_keys - 1);
-                const T* src = vb + (int64_t)n * p.v_sl;
-                const int c = col0 + cc * EPC;
-                u32x4 val = {0u, 0u, 0u, 0u};
-                if (p.v_vec && c + EPC <= p.n_out) {
-                    val = *reinterpret_cast<const u32x4*>(src + c);
-                } else {
-                    T tmp[EPC];
 #pragma unroll
-                    for (int e = 0; e < EPC; ++e) tmp[e] = (c + e < p.n_out) ? src[c + e] : (T)0.f;
-                    __builtin_memcpy(&val, tmp, 16);
-                }
-                *reinterpret_cast<u32x4*>(s_v + row * V_ROW + cc * 16) = val;
+            for (int i = 0; i < CPT; ++i) {
+                const int idx = tid + 256 * i;
+                *reinterpret_cast<u32x4*>(s_v + (idx / CR) * V_ROW + (idx % CR) * 16) = vreg[i];
+            }
+            // while the tile settles in LDS: request the next V tile and this tile's probability fragments
+            if (tile + 1 < pl.n_tiles) {
+#pragma unroll
+                for (int i = 0; i < CPT; ++i) vreg[i] = load_piece(j0 + kBN, i);
+            }
+            char* stg = s_p[wave];
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                *reinterpret_cast<vec8*>(stg + (8 * c + (lane >> 3)) * P_ROW + (lane & 7) * 8 * ES) = praw[c];
+            if (tile + 1 < pl.n_tiles) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) praw[c] = load_probs(j0 + kBN, c);
             }
             __syncthreads();
-            const bool skip = (j0 + kBN <= lmin) || (j0 >= hmax);  // wavefront-uniform
             if (skip) continue;
+            Frag<T> pf[kBN / 16];
+#pragma unroll
+            for (int t = 0; t < kBN / 16; ++t) pf[t] = lds_frag_rowmajor<T>(stg + lm * P_ROW + (16 * t + 8 * g) * ES);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // fragments read before the next tile overwrites the staging
 #pragma unroll
             for (int t = 0; t < kBN / 16; ++t) {
-                // A fragment: positions jj..jj+7 of this lane's row
-                const int jj = j0 + 16 * t + 8 * g;
-                Frag<T> pf;
-                const int u = jj - win.lo;
-                if (win.lin == 1 && u >= 0 && u + 8 <= win.cnt) {
-                    __builtin_memcpy(&pf.v, prow + off + u, 8 * ES);  // any alignment
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) pf.v[e] = win_live(win, jj + e) ? prow[off + win_slot(win, jj + e)] : (T)0.f;
-                }
 #pragma unroll
                 for (int dt = 0; dt < DVT; ++dt) {
                     Frag<T> vf = lds_frag_cols<T>(s_v, V_ROW, 16 * t + 8 * g, 16 * t + 8 * g + 4, 32 * dt, lane);
-                    mma32(acc[dt], pf, vf);
+                    mma32(acc[dt], pf[t], vf);
                 }
             }
         }
