@@ -131,9 +131,6 @@ __device__ __forceinline__ Frag<T> lds_frag_row_swz(const char* tile, int row, i
     return f;
 }
 
-#ifndef SPLAT_EXP
-#define SPLAT_EXP 0
-#endif
 constexpr float kRescaleThreshold = 8.0f;  // in log2 units: exponentials stay below 2^8 before the reference moves
 
 typedef __attribute__((address_space(3))) const u32x4 lds_u32x4;
@@ -176,7 +173,7 @@ __device__ __forceinline__ void softmax_tile(f32x16 (&s)[2], Frag<T> (&pf)[2][2]
     mx = fmaxf(mx, __shfl_xor(mx, 32));  // the other half of the row lives in lane ^ 32
     // move the reference only when some row's maximum has outrun it by the threshold (always on the first
     // live tile); rows that do not move keep alpha = 1
-    if (!(SPLAT_EXP & 4) && __any((mx - m_ref) * c2 > kRescaleThreshold)) {
+    if (__any((mx - m_ref) * c2 > kRescaleThreshold)) {
         const float m_new = ((mx - m_ref) * c2 > kRescaleThreshold) ? mx : m_ref;
         const float alpha = fast_exp2((m_ref - m_new) * c2);
         const bool had_data = __any(m_ref > 0.5f * kNegBigA);  // otherwise O and l are still all zero
@@ -243,7 +240,6 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
     // ---- plan: per segment, the column range and step of this row block ------------------------
     plan_segments<BM>(p.seg, p.n_seg, r0, rs, L, !KT, s_plan, &s_ps, tid);
 
-    if (SPLAT_EXP & 128) return;
     int total_tiles = 0;
     for (int sg = 0; sg < p.n_seg; ++sg) total_tiles += s_plan[sg].n_tiles;
     total_tiles = __builtin_amdgcn_readfirstlane(total_tiles);
@@ -410,14 +406,6 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
 
     dma_wait_all();
     __syncthreads();
-    if (SPLAT_EXP & 256) {
-        if (qf[0][0].v[0] == (T)12345.f) ob[0] = (T)0.f;
-        return;
-    }
-
-    if ((SPLAT_EXP & 32768) && (blockIdx.x & 8)) {
-        for (int z = 0; z < 10; ++z) __builtin_amdgcn_s_sleep(127);
-    }
     // per-lane row maps of the segment being computed
     int cur_seg = -1, cur_tile = 0;
     RowWin win[MT];
@@ -425,15 +413,7 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
     SegPlan cpl = {0, 1, 0, 1};
     const float c2 = p.scale_log2e;
 
-#if SPLAT_EXP & 65536
-    unsigned long long tl[16][8];
-    const bool tl_on = (blockIdx.x == 4001 || blockIdx.x == 4009);
-#define TL(i_) if (tl_on && it < 16) tl[it][i_] = __builtin_readcyclecounter();
-#else
-#define TL(i_)
-#endif
     for (int it = 0; it < total_tiles; ++it) {
-        TL(0)
         // advance the compute position; reload row maps on a segment change
         if (cur_seg < 0 || cur_tile >= cpl.n_tiles) {
             do {
@@ -471,16 +451,15 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
         ++cur_tile;
 
         const bool more = (it + 1 < total_tiles);
-        if (more && !(SPLAT_EXP & 32)) {
+        if (more) {
             issue_tile(ppl, pf_tile, (it + 1) & 1);
             ++pf_tile;
             pf_normalise();
         }
 
-        TL(1)
-        const bool skip = ((SPLAT_EXP & 1) != 0) || (j0 + kBN <= w_lo_min) || (j0 >= w_hi_max);
+        const bool skip = (j0 + kBN <= w_lo_min) || (j0 >= w_hi_max);
         if (!skip) {
-            const bool full = ((SPLAT_EXP & 2) != 0) || ((j0 >= w_lo_max) && (j0 + kBN <= w_hi_min));
+            const bool full = (j0 >= w_lo_max) && (j0 + kBN <= w_hi_min);
 
             // ---- S^T = K . Q^T ----
             // All K fragments of a 32-key tile are requested from LDS before the first MFMA that needs them, so
@@ -519,28 +498,16 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
                 }
             }
             __builtin_amdgcn_sched_barrier(0);  // keep the requests above the matrix work
-            if (SPLAT_EXP & 16384) __builtin_amdgcn_s_setprio(1);
-            if (!(SPLAT_EXP & 1024)) {
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
+            for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                    for (int ks = 0; ks < KS; ++ks)
+                for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-                        for (int mt = 0; mt < MT; ++mt) mma32(s_acc[mt][nt], kfr[nt][ks], qf[mt][ks]);
-            }
+                    for (int mt = 0; mt < MT; ++mt) mma32(s_acc[mt][nt], kfr[nt][ks], qf[mt][ks]);
 
-            TL(2)
-            if (SPLAT_EXP & 16384) __builtin_amdgcn_s_setprio(0);
             // ---- mask, online softmax against a lazily updated reference ----
             Frag<T> pf[MT][NT][2];
-            if (SPLAT_EXP & 4096) {
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                        for (int j = 0; j < 16; ++j) pf[mt][nt][j >> 3].v[j & 7] = (T)s_acc[mt][nt][j];
-            } else if (full) {
+            if (full) {
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
                     softmax_tile<true, T, DT>(s_acc[mt], pf[mt], m_ref[mt], l_run[mt], o_acc[mt], win[mt], true, j0, g, c2);
@@ -550,7 +517,6 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
                     softmax_tile<false, T, DT>(s_acc[mt], pf[mt], m_ref[mt], l_run[mt], o_acc[mt], win[mt], cpl.uniform != 0, j0, g, c2);
             }
 
-            TL(3)
             // ---- O^T += V^T . P^T ----
             // V fragments are requested one 16-key step (DT fragments) ahead of the MFMAs that consume them.
             auto load_v = [&](int nt, int t, int dt) {
@@ -569,7 +535,6 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
                 return vf;
             };
             Frag<T> vfr[2][DT];
-            if (SPLAT_EXP & 16384) __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) vfr[0][dt] = load_v(0, 0, dt);
 #pragma unroll
@@ -580,36 +545,22 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
                     for (int dt = 0; dt < DT; ++dt) vfr[(step + 1) & 1][dt] = load_v((step + 1) >> 1, (step + 1) & 1, dt);
                 }
                 __builtin_amdgcn_sched_barrier(0);  // keep the requests above the matrix work
-                if (!(SPLAT_EXP & 2048)) {
 #pragma unroll
-                    for (int dt = 0; dt < DT; ++dt)
+                for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-                        for (int mt = 0; mt < MT; ++mt) mma32(o_acc[mt][dt], vfr[step & 1][dt], pf[mt][nt][t]);
-                }
+                    for (int mt = 0; mt < MT; ++mt) mma32(o_acc[mt][dt], vfr[step & 1][dt], pf[mt][nt][t]);
             }
         }
 
-        TL(4)
-        if (SPLAT_EXP & 16384) __builtin_amdgcn_s_setprio(0);
         // the other stage becomes current
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) v_addr[dt] ^= G::STAGE;
 #pragma unroll
         for (int i = 0; i < (KT ? NT : KS); ++i) k_addr[i] ^= G::STAGE;
 
-        if (!(SPLAT_EXP & 16)) dma_wait_all();   // the next tile has landed in LDS
-        TL(5)
-        if (!(SPLAT_EXP & 8192)) __syncthreads();  // ... for every wavefront, and this tile's stage may be overwritten
-        TL(6)
+        dma_wait_all();   // the next tile has landed in LDS
+        __syncthreads();  // ... for every wavefront, and this tile's stage may be overwritten
     }
-#if SPLAT_EXP & 65536
-    if (tl_on && lane == 0) {
-        unsigned long long* dbg = reinterpret_cast<unsigned long long*>(const_cast<void*>(p.q)) + ((blockIdx.x == 4009) ? 4096 : 0) + wave * 128;
-        for (int a = 0; a < 16; ++a)
-            for (int c = 0; c < 7; ++c) dbg[a * 8 + c] = (a < total_tiles) ? tl[a][c] : 0ull;
-        dbg[7] = (unsigned long long)total_tiles;
-    }
-#endif
 
     // ---- epilogue: O = O^T / l, transposed through LDS so that every global store is a contiguous run --------
     // (all wavefronts left the loop through its final barrier; each one now uses a private region of the stages)
@@ -632,15 +583,13 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
                 }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wavefront's LDS writes are visible to its own reads
             constexpr int CPR = D * ES / 16;                    // 16-byte chunks per output row
-            if (!(SPLAT_EXP & 512)) {
 #pragma unroll
-                for (int i = 0; i < 32 * CPR / 64; ++i) {
-                    const int flat = i * 64 + lane;
-                    const int row = flat / CPR, c = flat % CPR;
-                    const int r = r0 + rs * ((wave * MT + mt) * 32 + row);
-                    const u32x4 val = *reinterpret_cast<const u32x4*>(stg + row * OROW + c * 16);
-                    if (r < L) *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(ob + (int64_t)r * p.o_sl) + c * 16) = val;
-                }
+            for (int i = 0; i < 32 * CPR / 64; ++i) {
+                const int flat = i * 64 + lane;
+                const int row = flat / CPR, c = flat % CPR;
+                const int r = r0 + rs * ((wave * MT + mt) * 32 + row);
+                const u32x4 val = *reinterpret_cast<const u32x4*>(stg + row * OROW + c * 16);
+                if (r < L) *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(ob + (int64_t)r * p.o_sl) + c * 16) = val;
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // reads done before the next m-tile reuses the region
         }

@@ -66,9 +66,6 @@ __global__ __launch_bounds__(256, 2) void spmm_kernel(const SpmmParams p) {
     }
     plan_segments<BM>(p.seg, p.n_seg, r0, rs, L, true, s_plan, &s_ps, tid);
 
-    const int my_row = r0 + rs * (32 * wave + lm);  // A-operand row of this lane
-    const T* prow = pb + (int64_t)min(my_row, L - 1) * p.T;
-
     f32x16 acc[DVT];
 #pragma unroll
     for (int dt = 0; dt < DVT; ++dt)
