@@ -50,8 +50,8 @@ __device__ __forceinline__ RowMap cached_row_map(const PlanScratch<BM>* ps, int 
 }
 
 // Gather the maps of rows r0 + rs*k, k in [0, BM), of every segment into LDS and reduce what the plans need.  Called by
-// all 256 threads of the workgroup (BM <= 256: one row per thread); contains two barriers.  Afterwards
-// segment_plan() may be evaluated by any thread.
+// every thread of the workgroup (threads 0..255 take one row each, BM <= 256; further wavefronts only take part in
+// the barriers); contains two barriers.  Afterwards segment_plan() may be evaluated by any thread.
 template <int BM>
 __device__ __forceinline__ void gather_row_maps(const SegPtrs* seg, int n_seg, int r0, int rs, int n_rows,
                                                 PlanScratch<BM>* ps, int tid) {
@@ -73,7 +73,7 @@ __device__ __forceinline__ void gather_row_maps(const SegPtrs* seg, int n_seg, i
             const int cmax = wave_max_i(m.cnt > 0 ? m.a + m.lin * (m.cnt - 1) : -1);
             const int linmin = wave_min_i(m.cnt > 1 ? m.lin : 0x7fffffff);
             const int linmax = wave_max_i(m.cnt > 1 ? m.lin : 0);
-            if (lane == 0) {
+            if (lane == 0 && wave < 4) {
                 ps->part[wave][sg][0] = amin;
                 ps->part[wave][sg][1] = cmax;
                 ps->part[wave][sg][2] = linmin;
@@ -96,7 +96,7 @@ __device__ __forceinline__ void gather_row_maps(const SegPtrs* seg, int n_seg, i
             const int step = (linmax == 0) ? 1 : linmin;  // no row with 2+ columns: any step fits
             if (!bad && step > 1) bad = mine[sg].cnt > 0 && ((mine[sg].a - amin) % step) != 0;
             const int any_bad = __any(bad) ? 1 : 0;
-            if (lane == 0) ps->flag[wave][sg] = any_bad;
+            if (lane == 0 && wave < 4) ps->flag[wave][sg] = any_bad;
         }
     }
     __syncthreads();

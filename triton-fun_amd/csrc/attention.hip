@@ -19,7 +19,7 @@
 // gathered rows of K/V) and validity is a per-row range test in j; otherwise tiles are dense columns
 // and validity is the full affine test (offset, step divisibility, count).  Each wavefront skips
 // tiles that lie outside all of its rows' spans and drops the mask on tiles inside all of them.
-#include "acsr_plan.hpp"
+#include "tile_copy.hpp"
 
 namespace splat {
 
@@ -43,104 +43,7 @@ struct AttnParams {
     int row_stride;
 };
 
-template <typename T, int D, bool KT>
-struct TileGeom {
-    static constexpr int ES = sizeof(T);
-    static constexpr int EPC = 16 / ES;                       // elements per 16-byte chunk
-    static constexpr int K_ROWB = KT ? kBN * ES : D * ES;     // bytes per LDS row of the K tile (no padding)
-    static constexpr int K_ROWS = KT ? D : kBN;
-    static constexpr int V_ROWB = D * ES;
-    static constexpr int K_BYTES = K_ROWB * K_ROWS;
-    static constexpr int V_BYTES = V_ROWB * kBN;
-    static constexpr int STAGE = K_BYTES + V_BYTES;
-};
-
-// XOR swizzle of the 16-byte chunk index of a row-major LDS tile with ROWB-byte rows, chosen so that 16
-// lanes reading the same logical chunk of 16 consecutive rows hit 16 different bank groups.
-template <int ROWB>
-__device__ __forceinline__ constexpr int swz(int row) {
-    constexpr int CPR = ROWB / 16;
-    constexpr int CH = CPR < 16 ? CPR : 16;
-    constexpr int RPB = ROWB >= 256 ? 1 : 256 / ROWB;
-    return (row / RPB) & (CH - 1);
-}
-template <int ROWB, bool SWZ>
-__device__ __forceinline__ int lds_off(int row, int byte_col) {
-    if constexpr (SWZ)
-        return row * ROWB + ((((byte_col >> 4) ^ swz<ROWB>(row)) << 4) | (byte_col & 15));
-    else
-        return row * ROWB + byte_col;
-}
-
-// Swizzle of the 64-byte block index for tiles read with the transposing read, whose 64 lanes touch 8
-// consecutive rows x 64 bytes: 4 consecutive rows must fall into the 4 different 64-byte quadrants of the
-// 256-byte bank space (what a row pitch of 256+64 bytes would give, which the 1 KiB LDS-DMA blocks rule out).
-template <int ROWB>
-__device__ __forceinline__ constexpr int swz64(int row) {
-    return ROWB >= 256 ? (row & 3) : ((row >> 1) & 1);
-}
-// logical 16-byte chunk held at physical chunk position pc of `row`; MODE 0: none, 1: chunk XOR (b128 row reads),
-// 2: 64-byte block XOR (transposing reads)
-template <int ROWB, int MODE>
-__device__ __forceinline__ int logical_chunk(int row, int pc) {
-    if constexpr (MODE == 1) return pc ^ swz<ROWB>(row);
-    if constexpr (MODE == 2) return (((pc >> 2) ^ swz64<ROWB>(row)) << 2) | (pc & 3);
-    return pc;
-}
-
-typedef __attribute__((address_space(1))) const void gptr_t;
-typedef __attribute__((address_space(3))) void lptr_t;
-
-// One wavefront-wide 1 KiB copy global -> LDS without passing through registers: lane i's 16 bytes land at
-// lds_block + 16*i (lds_block must be wavefront-uniform).
-__device__ __forceinline__ void dma16(const void* src, char* lds_block) {
-    __builtin_amdgcn_global_load_lds((gptr_t*)src, (lptr_t*)lds_block, 16, 0, 0);
-}
-__device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-
-// Copy a ROWS x ROWB-byte tile into LDS; row r comes from row_ptr(r) (16-byte aligned, ROWB readable bytes).
-// Each wavefront issues ROWS*ROWB/4096 instructions of 1 KiB.
-template <typename T, int ROWB, int ROWS, int SWZ, typename RowPtr>
-__device__ __forceinline__ void dma_tile(char* tile, int wave, int lane, RowPtr row_ptr) {
-    constexpr int NI = ROWS * ROWB / 1024;  // wavefront instructions per tile
-    constexpr int CPR = ROWB / 16;          // chunks per row
-    static_assert(NI % 4 == 0 && (1024 % ROWB == 0 || ROWB % 1024 == 0), "tile shape");
-#pragma unroll
-    for (int i = 0; i < NI / 4; ++i) {
-        const int q = wave + 4 * i;
-        const int flat = q * 64 + lane;  // chunk position in the tile
-        const int row = flat / CPR, pc = flat % CPR;
-        const int c = logical_chunk<ROWB, SWZ>(row, pc);
-        dma16(reinterpret_cast<const char*>(row_ptr(row)) + c * 16, tile + q * 1024);
-    }
-}
-
-// K fragment (8 consecutive contraction values of row `row`) from a swizzled row-major tile.
-template <typename T, int ROWB>
-__device__ __forceinline__ Frag<T> lds_frag_row_swz(const char* tile, int row, int elem_col) {
-    Frag<T> f;
-    if constexpr (sizeof(T) == 2) {
-        u32x4 r = *reinterpret_cast<const u32x4*>(tile + lds_off<ROWB, true>(row, elem_col * 2));
-        f.v = __builtin_bit_cast(typename Frag<T>::vec, r);
-    } else {
-        u32x4 r0 = *reinterpret_cast<const u32x4*>(tile + lds_off<ROWB, true>(row, elem_col * 4));
-        u32x4 r1 = *reinterpret_cast<const u32x4*>(tile + lds_off<ROWB, true>(row, elem_col * 4 + 16));
-        u32x8 r = __builtin_shufflevector(r0, r1, 0, 1, 2, 3, 4, 5, 6, 7);
-        f.v = __builtin_bit_cast(typename Frag<T>::vec, r);
-    }
-    return f;
-}
-
 constexpr float kRescaleThreshold = 8.0f;  // in log2 units: exponentials stay below 2^8 before the reference moves
-
-typedef __attribute__((address_space(3))) const u32x4 lds_u32x4;
-typedef __attribute__((address_space(3))) const float lds_f32;
-
-__device__ __forceinline__ u32x4 lds_load128(uint32_t addr) { return *reinterpret_cast<lds_u32x4*>((uintptr_t)addr); }
-__device__ __forceinline__ s16x4 lds_load_tr16(uint32_t addr) {
-    return __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_s16x4*>((uintptr_t)addr));
-}
-__device__ __forceinline__ float lds_load_f32(uint32_t addr) { return *reinterpret_cast<lds_f32*>((uintptr_t)addr); }
 
 // Mask (unless FULL), fold one 64-key tile of scores of one 32-row tile into the running softmax state and
 // emit the exponentials as MFMA B fragments.  One lane owns one query row (half of its 64 positions).

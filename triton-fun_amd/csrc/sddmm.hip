@@ -45,6 +45,32 @@ __device__ __forceinline__ Frag<T> load_q_frag(const T* row, int k0, int d, bool
     return f;
 }
 
+// Store the scores of 8 consecutive tile positions jj..jj+7 of one row; `row_out` points at the row's first slot of
+// the segment.  Unit-step rows: the positions are consecutive slots, written with one 16/32-byte store (any
+// alignment) when all 8 are live and element by element under a range test at the two ends of the row's span;
+// lanes whose positions miss the span altogether do nothing.  Other rows: the full affine test per position.
+template <typename TO>
+__device__ __forceinline__ void store_piece(TO* row_out, const RowWin& w, int jj, const float (&v)[8]) {
+    const int u = jj - w.lo;
+    if (w.lin == 1) {
+        if (u >= 0 && u + 8 <= w.cnt) {
+            typedef TO v8 __attribute__((ext_vector_type(8)));
+            v8 t;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) t[e] = (TO)v[e];
+            __builtin_memcpy(row_out + u, &t, 8 * sizeof(TO));
+        } else if (u + 8 > 0 && u < w.cnt) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if ((unsigned)(u + e) < (unsigned)w.cnt) row_out[u + e] = (TO)v[e];
+        }
+    } else if (w.cnt > 0) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            if (win_live(w, jj + e)) row_out[win_slot(w, jj + e)] = (TO)v[e];
+    }
+}
+
 template <typename T, bool KT, bool QREG>
 __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
     constexpr int ES = sizeof(T);
@@ -228,31 +254,13 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
                     const f32x4 a0 = *reinterpret_cast<const f32x4*>(src);
                     const f32x4 a1 = *reinterpret_cast<const f32x4*>(src + 16);
                     const float v[8] = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
-                    const RowWin& w = wr[c];
                     const int jj = j0 + 32 * nt + 8 * (lane & 3);
-                    const int u = jj - w.lo;
-                    if (w.lin == 1 && u >= 0 && u + 8 <= w.cnt) {
-                        const int64_t o = wbase[c] + u;
-                        if (p.out_dtype == SPLAT_BF16) {
-                            typedef bf16 v8 __attribute__((ext_vector_type(8)));
-                            v8 t;
-#pragma unroll
-                            for (int e = 0; e < 8; ++e) t[e] = (bf16)v[e];
-                            __builtin_memcpy((bf16*)p.out + o, &t, 16);
-                        } else if (p.out_dtype == SPLAT_F16) {
-                            typedef f16 v8 __attribute__((ext_vector_type(8)));
-                            v8 t;
-#pragma unroll
-                            for (int e = 0; e < 8; ++e) t[e] = (f16)v[e];
-                            __builtin_memcpy((f16*)p.out + o, &t, 16);
-                        } else {
-                            __builtin_memcpy((float*)p.out + o, v, 32);
-                        }
-                    } else if (w.cnt > 0) {
-#pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            if (win_live(w, jj + e)) store_as(p.out, wbase[c] + win_slot(w, jj + e), v[e], p.out_dtype);
-                    }
+                    if (p.out_dtype == SPLAT_BF16)
+                        store_piece<bf16>((bf16*)p.out + wbase[c], wr[c], jj, v);
+                    else if (p.out_dtype == SPLAT_F16)
+                        store_piece<f16>((f16*)p.out + wbase[c], wr[c], jj, v);
+                    else
+                        store_piece<float>((float*)p.out + wbase[c], wr[c], jj, v);
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // staging reads done before it is overwritten
             }
