@@ -54,8 +54,9 @@ def time_launches(fn, steps: int, warmup: int):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50,
+                    help="untimed launches before the timed ones (the GPU clock needs some tens of launches to settle)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host baseline")
     ap.add_argument("--no-extras", action="store_true", help="skip the unfused kernels and the ACSR build")
     ap.add_argument("--cpu-heads", type=int, default=16, help="(batch, head) pairs the host baseline computes")
@@ -142,7 +143,7 @@ def main() -> int:
     if not args.no_extras:
         # the literal reference layout: K^T contiguous [B, H, d, L]
         kT_c = kT_view.contiguous()
-        _, per_c = time_launches(lambda: attn([qd, kT_c, vd]), max(5, args.steps // 2), 3)
+        _, per_c = time_launches(lambda: attn([qd, kT_c, vd]), max(5, args.steps // 2), max(3, args.warmup // 2))
         ms_c = sum(per_c) / len(per_c)
         extras["fused_kT_contiguous"] = {"ms": round(ms_c, 4), "tflops_nnz": round(flops / ms_c / 1e9, 2)}
         del kT_c
@@ -182,7 +183,7 @@ def main() -> int:
                 ("sddmm_cfg4", run_sddmm, (2 * B4 * H4 * L4 * d4 + nnz4 * B4 * H4) * 2, 2 * d4 * nnz4 * B4 * H4),
                 ("softmax_cfg4", run_soft, 2 * nnz4 * B4 * H4 * 2, 0.0),
                 ("spmm_cfg4", run_spmm, (2 * B4 * H4 * L4 * d4 + nnz4 * B4 * H4) * 2, 2 * d4 * nnz4 * B4 * H4)):
-            _, pr = time_launches(fn, 20, 5)
+            _, pr = time_launches(fn, 40, 20)
             ms = sum(pr) / len(pr)
             extras[name] = {"ms": round(ms, 4), "gbps_algorithmic": round(byt / ms / 1e6, 1),
                             "hbm_frac": round(byt / ms / 1e6 / HBM_PEAK_GBPS, 4)}
