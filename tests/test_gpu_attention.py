@@ -154,3 +154,25 @@ def test_unit_projection_wrapper(dev):
     q, k, v = [torch.einsum("bsd,dnh->bnsh", a, b) for a, b in zip(x, w)]
     want = O.dense_masked_attention(q, k.transpose(2, 3), v, np.asarray(mask), 1.0)
     assert float((got - want).abs().max()) <= 1e-5
+
+
+@pytest.mark.parametrize("L,d,w,dtype", [(32768, 128, 512, torch.bfloat16), (40003, 64, 300, torch.float16)])
+def test_long_sequences_by_properties(dev, L, d, w, dtype):
+    """Sequences longer than any BASELINE configuration, one of them not a multiple of any tile size: the mask
+    exists only on the GPU (`MaskPattern`), so the checks are size-independent ones: V = 1 gives 1 everywhere, and a few
+    rows are recomputed directly from their window."""
+    g = torch.Generator().manual_seed(L)
+    q = torch.randn(1, 1, L, d, generator=g).to(dtype).to(dev)
+    k = torch.randn(1, 1, L, d, generator=g).to(dtype).to(dev)
+    v = torch.randn(1, 1, L, d, generator=g).to(dtype).to(dev)
+    scale = d ** -0.5
+    attn = RegularAttention(1, L, 1, d, A.causal_windowed_pattern(L, w - 1), 16, 16, dev, dtype, scale=scale)
+    ones = attn([q, k.transpose(2, 3), torch.ones_like(v)]).float()
+    assert float((ones - 1).abs().max()) <= TOL[dtype]
+    out = attn([q, k.transpose(2, 3), v]).float()
+    assert torch.isfinite(out).all()
+    for r in (0, 1, w - 2, w - 1, w, L // 2 + 7, L - 2, L - 1):
+        lo = max(0, r - w + 1)
+        s = (q[0, 0, r].float() @ k[0, 0, lo:r + 1].float().T) * scale
+        want = torch.softmax(s, -1) @ v[0, 0, lo:r + 1].float()
+        assert float((out[0, 0, r] - want).abs().max()) <= TOL[dtype], r
