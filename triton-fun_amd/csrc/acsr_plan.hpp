@@ -21,7 +21,7 @@ struct SegPtrs {
 struct SegPlan {
     int c0;       // dense column of tile position j = 0
     int cs;       // column step between consecutive tile positions
-    int n_tiles;  // kBN-position tiles to walk
+    int n_tiles;  // tiles (of the kernel's tile size, kBN unless stated) to walk
     int uniform;  // 1: all rows share step and phase -> position j of row r is slot j - lo_r;
                   // 0: positions are dense columns and a row applies the full affine test
 };
@@ -103,7 +103,7 @@ __device__ __forceinline__ void gather_row_maps(const SegPtrs* seg, int n_seg, i
 }
 
 // The workgroup's plan for segment sg (valid after gather_row_maps).  `allow_gather` = false forces dense walks.
-template <int BM>
+template <int BM, int BN = kBN>
 __device__ __forceinline__ SegPlan segment_plan(const PlanScratch<BM>* ps, int sg, bool allow_gather) {
     int amin = 0x7fffffff, cmax = -1, linmin = 0x7fffffff, linmax = 0, bad = 0;
 #pragma unroll
@@ -128,18 +128,18 @@ __device__ __forceinline__ SegPlan segment_plan(const PlanScratch<BM>* ps, int s
     pl.cs = uni ? step : 1;
     // dense walks start on a tile boundary (keeps 16-byte K^T loads aligned and lets neighbouring row blocks
     // share cache lines); gathered walks start at the first live column
-    pl.c0 = (pl.cs == 1) ? (amin & ~(kBN - 1)) : amin;
+    pl.c0 = (pl.cs == 1) ? (amin & ~(BN - 1)) : amin;
     const int n_pos = (cmax - pl.c0) / pl.cs + 1;
-    pl.n_tiles = (n_pos + kBN - 1) / kBN;
+    pl.n_tiles = (n_pos + BN - 1) / BN;
     return pl;
 }
 
 // gather_row_maps + one SegPlan per segment in LDS (plan[0..n_seg)); ends with a barrier.
-template <int BM>
+template <int BM, int BN = kBN>
 __device__ __forceinline__ void plan_segments(const SegPtrs* seg, int n_seg, int r0, int rs, int n_rows,
                                               bool allow_gather, SegPlan* plan, PlanScratch<BM>* ps, int tid) {
     gather_row_maps<BM>(seg, n_seg, r0, rs, n_rows, ps, tid);
-    if (tid < n_seg) plan[tid] = segment_plan<BM>(ps, tid, allow_gather);
+    if (tid < n_seg) plan[tid] = segment_plan<BM, BN>(ps, tid, allow_gather);
     __syncthreads();
 }
 

@@ -1,10 +1,11 @@
 // Fused ACSR sparse-attention forward (online softmax), gfx950.
 //
-// A workgroup of 4 wavefronts owns BM = 128*MT consecutive query rows of one (batch, head).  It walks
-// the key range its rows' affine spans cover in tiles of 64 keys.  Per tile:
-//   * all 256 threads copy the K and V tiles global -> registers -> LDS (double buffered; the copy of
-//     tile t+1 overlaps the math of tile t);
-//   * every wavefront computes the TRANSPOSED score tile S^T = K . Q^T for its 32*MT rows with
+// A workgroup of 4 wavefronts owns 128 query rows of one (batch, head).  It walks the key range its
+// rows' affine spans cover in tiles of BN keys.  Per tile:
+//   * the K and V tiles are copied global -> LDS without passing through registers (LDS-DMA), into a
+//     ring of NSTAGE stages: the copy of tile t + NSTAGE - 1 is issued while tile t is computed, piecewise
+//     between its score MFMAs;
+//   * every wavefront computes the TRANSPOSED score tile S^T = K . Q^T for its 32 rows with
 //     32x32x16 MFMA (A = K fragment from LDS, B = Q fragment held in registers for the whole kernel).
 //     In the transposed product one lane owns one query row, so masking, the running max and the
 //     running sum need no cross-lane traffic beyond one exchange with the lane that holds the other
@@ -45,17 +46,17 @@ struct AttnParams {
 
 constexpr float kRescaleThreshold = 8.0f;  // in log2 units: exponentials stay below 2^8 before the reference moves
 
-// Mask (unless FULL), fold one 64-key tile of scores of one 32-row tile into the running softmax state and
-// emit the exponentials as MFMA B fragments.  One lane owns one query row (half of its 64 positions).
-template <bool FULL, typename T, int DT>
-__device__ __forceinline__ void softmax_tile(f32x16 (&s)[2], Frag<T> (&pf)[2][2], float& m_ref, float& l_run,
+// Mask (unless FULL), fold one tile of 32*NT keys of scores of one 32-row tile into the running softmax state
+// and emit the exponentials as MFMA B fragments.  One lane owns one query row (half of its positions).
+template <bool FULL, int NT, typename T, int DT>
+__device__ __forceinline__ void softmax_tile(f32x16 (&s)[NT], Frag<T> (&pf)[NT][2], float& m_ref, float& l_run,
                                              f32x16 (&o)[DT], const RowWin& win, bool uniform, int j0, int g, float c2) {
     if constexpr (!FULL) {
         if (uniform) {  // live iff 0 <= position - lo < cnt
             const int base = j0 + 4 * g - win.lo;
             const unsigned cnt = (unsigned)win.cnt;
 #pragma unroll
-            for (int nt = 0; nt < 2; ++nt)
+            for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                 for (int j = 0; j < 16; ++j) {
                     const unsigned u = (unsigned)(base + 32 * nt + 8 * (j >> 2) + (j & 3));
@@ -63,14 +64,14 @@ __device__ __forceinline__ void softmax_tile(f32x16 (&s)[2], Frag<T> (&pf)[2][2]
                 }
         } else {
 #pragma unroll
-            for (int nt = 0; nt < 2; ++nt)
+            for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                 for (int j = 0; j < 16; ++j) s[nt][j] = win_live(win, j0 + 32 * nt + acc_row(j, g)) ? s[nt][j] : kNegBigA;
         }
     }
     float mx = s[0][0];
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
+    for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
         for (int j = 0; j < 16; ++j) mx = fmaxf(mx, s[nt][j]);
     mx = fmaxf(mx, __shfl_xor(mx, 32));  // the other half of the row lives in lane ^ 32
@@ -95,7 +96,7 @@ __device__ __forceinline__ void softmax_tile(f32x16 (&s)[2], Frag<T> (&pf)[2][2]
     const float mb = (FULL || m_ref > 0.5f * kNegBigA) ? m_ref * c2 : 0.f;
     float rs = 0.f;
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
+    for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
             const float pv = fast_exp2(fmaf(s[nt][j], c2, -mb));
@@ -105,16 +106,17 @@ __device__ __forceinline__ void softmax_tile(f32x16 (&s)[2], Frag<T> (&pf)[2][2]
     l_run += rs;
 }
 
-template <typename T, int D, int MT, bool KT>
-__global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn_fwd_kernel(const AttnParams p) {
-    using G = TileGeom<T, D, KT>;
+template <typename T, int D, bool KT, int BN, int NSTAGE>
+__global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(const AttnParams p) {
+    using G = TileGeom<T, D, KT, BN>;
     constexpr int ES = G::ES;
-    constexpr int BM = 128 * MT;
+    constexpr int BM = 128;
     constexpr int KS = D / 16;  // contraction steps of the score product
     constexpr int DT = D / 32;  // 32-row tiles of O^T
-    constexpr int NT = kBN / 32;
-    static_assert(NT == 2, "softmax_tile assumes two 32-key tiles");
-    static_assert((G::STAGE & (G::STAGE - 1)) == 0, "the stage toggle is an XOR");
+    constexpr int NT = BN / 32;
+    constexpr int PD = NSTAGE - 1;  // tiles whose copies run ahead of the tile being computed
+    static_assert(NT == 1 || NT == 2, "tiles of 32 or 64 keys");
+    static_assert(PD == 1 || PD == 3, "the wait ladder below covers 2 and 4 stages");
     constexpr bool FAST_DMA = (ES == 2);  // lane offsets of the LDS-DMA do not depend on the instruction index
 
     extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -140,14 +142,24 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
     const T* vb = (const T*)p.v + b * p.v_sb + h * p.v_sh;
     T* ob = (T*)p.o + b * p.o_sb + h * p.o_sh;
 
+    // ---- Q fragments (B operand of S^T), resident for the whole kernel; requested before the plan so that
+    // their latency overlaps the metadata loads (the plan's barriers wait for both) ------------------------
+    Frag<T> qf[KS];
+    {
+        const int my_row = r0 + rs * (wave * 32 + lm);
+        const T* qr = qb + (int64_t)min(my_row, L - 1) * p.q_sl;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qf[ks] = global_frag<T>(qr + 16 * ks + 8 * g);
+    }
+
     // ---- plan: per segment, the column range and step of this row block ------------------------
-    plan_segments<BM>(p.seg, p.n_seg, r0, rs, L, !KT, s_plan, &s_ps, tid);
+    plan_segments<BM, BN>(p.seg, p.n_seg, r0, rs, L, !KT, s_plan, &s_ps, tid);
 
     int total_tiles = 0;
     for (int sg = 0; sg < p.n_seg; ++sg) total_tiles += s_plan[sg].n_tiles;
     total_tiles = __builtin_amdgcn_readfirstlane(total_tiles);
 
-    // ---- tile walker: asynchronous global -> LDS copies of tile (sg, tile) into a stage ----------
+    // ---- tile walker: asynchronous global -> LDS copies of a tile into a stage -------------------------
     // A tile is copied as 1 KiB blocks, one wavefront instruction each; block q holds tile rows q*RPI.. and
     // wavefront w issues blocks w, w+4, ...  Lane i of a block supplies physical chunk i, i.e. (row i / CPR,
     // chunk position i % CPR), and loads the logical chunk the tile's swizzle assigns to that position.  For
@@ -155,15 +167,17 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
     // a per-segment constant and the block's base is wavefront-uniform.
     constexpr int V_CPR = G::V_ROWB / 16, V_RPI = 1024 / G::V_ROWB;
     constexpr int K_CPR = G::K_ROWB / 16, K_RPI = 1024 / G::K_ROWB;
-    constexpr int V_NI = kBN * G::V_ROWB / 4096, K_NI = G::K_ROWS * G::K_ROWB / 4096;  // blocks per wavefront
+    constexpr int V_NI = BN * G::V_ROWB / 4096, K_NI = G::K_ROWS * G::K_ROWB / 4096;  // blocks per wavefront
+    constexpr int NDMA = V_NI + K_NI;  // copy instructions per wavefront and tile, on every path
+    static_assert(V_NI >= 1 && K_NI >= 1 && NDMA * (PD - 1) < 64, "tile shape");
     auto issue_tile_general = [&](const SegPlan& pl, int tile, int stage) {
-        const int j0 = tile * kBN;
+        const int j0 = tile * BN;
         char* ks_w = smem + stage * G::STAGE;
         char* vs_w = ks_w + G::K_BYTES;
         auto key_row = [&](int row) { return min(max(pl.c0 + pl.cs * (j0 + row), 0), L - 1); };
-        dma_tile<T, G::V_ROWB, kBN, (ES == 2 ? 2 : 0)>(vs_w, wave, lane, [&](int row) { return vb + (int64_t)key_row(row) * p.v_sl; });
+        dma_tile<T, G::V_ROWB, BN, (ES == 2 ? 2 : 0)>(vs_w, wave, lane, [&](int row) { return vb + (int64_t)key_row(row) * p.v_sl; });
         if constexpr (KT) {
-            // rows = contraction index, 64 consecutive keys per row (dense walk); a chunk that would run past
+            // rows = contraction index, BN consecutive keys per row (dense walk); a chunk that would run past
             // the last key is replaced by the last whole chunk (those positions are never live)
 #pragma unroll
             for (int i = 0; i < K_NI; ++i) {
@@ -175,7 +189,7 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
                 dma16(kb + (int64_t)row * p.k_sd + c, ks_w + q * 1024);
             }
         } else {
-            dma_tile<T, G::K_ROWB, kBN, 1>(ks_w, wave, lane, [&](int row) { return kb + (int64_t)key_row(row) * p.k_sl; });
+            dma_tile<T, G::K_ROWB, BN, 1>(ks_w, wave, lane, [&](int row) { return kb + (int64_t)key_row(row) * p.k_sl; });
         }
     };
     // FAST_DMA state for the segment being fetched: per-lane byte offsets inside a block, wavefront-uniform
@@ -203,32 +217,22 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
             }
         }
     };
-    // Tiles of a segment are issued in order, so the running pointers simply advance by one tile per call.
-    auto issue_tile = [&](const SegPlan& pl, int tile, int stage) {
-        const int j0 = tile * kBN;
-        const int key_first = pl.c0 + pl.cs * j0, key_last = pl.c0 + pl.cs * (j0 + kBN - 1);
+    // whether every key of the tile exists, so that the running pointers can be used as they are
+    auto tile_is_fast = [&](const SegPlan& pl, int tile) {
+        const int j0 = tile * BN;
+        const int key_first = pl.c0 + pl.cs * j0, key_last = pl.c0 + pl.cs * (j0 + BN - 1);
         bool fast = FAST_DMA && key_last < L;
-        if constexpr (KT) fast = fast && (key_first + kBN <= L);
-        if (!fast) {
-            issue_tile_general(pl, tile, stage);
-        } else {
-            char* ks_w = smem + stage * G::STAGE;
-            char* vs_w = ks_w + G::K_BYTES;
-            const char* vbase = v_next;
-            const char* kbase = k_next;
-#pragma unroll
-            for (int i = 0; i < V_NI; ++i) {
-                dma16(vbase + v_lane_off, vs_w + (wave + 4 * i) * 1024);
-                vbase += 4 * V_RPI * v_key;
-            }
-#pragma unroll
-            for (int i = 0; i < K_NI; ++i) {
-                dma16(kbase + k_lane_off, ks_w + (wave + 4 * i) * 1024);
-                kbase += 4 * K_RPI * k_key;
-            }
-        }
-        v_next += kBN * v_key;
-        k_next += KT ? (int64_t)(kBN * ES) : kBN * k_key;
+        if constexpr (KT) fast = fast && (key_first + BN <= L);
+        return fast;
+    };
+    // copy instruction i (0 .. NDMA-1) of the tile the running pointers stand at
+    auto issue_step = [&](int i, int stage) {
+        char* ks_w = smem + stage * G::STAGE;
+        char* vs_w = ks_w + G::K_BYTES;
+        if (i < V_NI)
+            dma16(v_next + (int64_t)(4 * V_RPI * i) * v_key + v_lane_off, vs_w + (wave + 4 * i) * 1024);
+        else
+            dma16(k_next + (int64_t)(4 * K_RPI * (i - V_NI)) * k_key + k_lane_off, ks_w + (wave + 4 * (i - V_NI)) * 1024);
     };
 
     int pf_seg = 0, pf_tile = 0;  // position of the next tile to fetch
@@ -249,38 +253,36 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
             set_lane_offsets(ppl);
         }
     };
-    pf_normalise();
-    if (total_tiles > 0) {
-        issue_tile(ppl, pf_tile, 0);
+    // Tiles of a segment are fetched in order, so the running pointers advance by one tile per fetch.
+    auto advance_fetch = [&]() {
+        v_next += BN * v_key;
+        k_next += KT ? (int64_t)(BN * ES) : BN * k_key;
         ++pf_tile;
         pf_normalise();
+    };
+    pf_normalise();
+#pragma unroll
+    for (int i = 0; i < PD; ++i) {
+        if (i < total_tiles) {
+            if (tile_is_fast(ppl, pf_tile)) {
+#pragma unroll
+                for (int s = 0; s < NDMA; ++s) issue_step(s, i);
+            } else {
+                issue_tile_general(ppl, pf_tile, i);
+            }
+            advance_fetch();
+        }
     }
 
-    // ---- Q fragments (B operand of S^T), resident for the whole kernel --------------------------
-    Frag<T> qf[MT][KS];
-    int my_row[MT];
+    f32x16 o_acc[DT];
+    float m_ref = kNegBigA, l_run = 0.f;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        my_row[mt] = r0 + rs * ((wave * MT + mt) * 32 + lm);
-        const T* qr = qb + (int64_t)min(my_row[mt], L - 1) * p.q_sl;
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) qf[mt][ks] = global_frag<T>(qr + 16 * ks + 8 * g);
-    }
-
-    f32x16 o_acc[MT][DT];
-    float m_ref[MT], l_run[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        m_ref[mt] = kNegBigA;
-        l_run[mt] = 0.f;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int j = 0; j < 16; ++j) o_acc[mt][dt][j] = 0.f;
-    }
+        for (int j = 0; j < 16; ++j) o_acc[dt][j] = 0.f;
 
     // ---- LDS read addresses: lane-dependent part + current stage; tile constants go into the instruction's
-    // immediate offset; the stage is toggled by XOR once per tile -----------------------------------------
+    // immediate offset; the stage offset is added once per tile -------------------------------------------
     const uint32_t smem_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
     // transposing reads: lane s of a 16-lane block addresses row s/4, 8 bytes at element column 16*(block%2) + 4*(s%4)
     const int tr_row = (lane & 15) >> 2;
@@ -307,17 +309,17 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
         for (int i = 0; i < (KT ? NT : KS); ++i) k_addr[i] = smem_base;
     }
 
-    dma_wait_all();
-    __syncthreads();
-    // per-lane row maps of the segment being computed
+    // per-lane row map of the segment being computed
     int cur_seg = -1, cur_tile = 0;
-    RowWin win[MT];
+    RowWin win = {0, 0, 1};
     int w_lo_min = 0, w_lo_max = 0, w_hi_min = 0, w_hi_max = 0;
     SegPlan cpl = {0, 1, 0, 1};
     const float c2 = p.scale_log2e;
+    int stage_it = 0;             // stage that holds tile `it`
+    int stage_pf = PD % NSTAGE;   // stage the next fetch goes to
 
     for (int it = 0; it < total_tiles; ++it) {
-        // advance the compute position; reload row maps on a segment change
+        // advance the compute position; reload the row map on a segment change
         if (cur_seg < 0 || cur_tile >= cpl.n_tiles) {
             do {
                 ++cur_seg;
@@ -330,50 +332,49 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
                 cpl.n_tiles = __builtin_amdgcn_readfirstlane(t.n_tiles);
                 cpl.uniform = __builtin_amdgcn_readfirstlane(t.uniform);
             }
-            int lmin = 0x3fffffff, lmax = -0x3fffffff, hmin = 0x3fffffff, hmax = -0x3fffffff;
-            bool any_empty = false;
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                win[mt] = make_row_win(cached_row_map<BM>(&s_ps, cur_seg, (wave * MT + mt) * 32 + lm), cpl);
-                if (win[mt].cnt <= 0) {
-                    any_empty = true;
-                } else {
-                    lmin = min(lmin, win[mt].lo);
-                    lmax = max(lmax, win[mt].lo);
-                    hmin = min(hmin, win[mt].lo + win[mt].cnt);
-                    hmax = max(hmax, win[mt].lo + win[mt].cnt);
-                }
-            }
-            w_lo_min = wave_min_i(lmin);
-            w_lo_max = wave_max_i(lmax);
-            w_hi_min = wave_min_i(hmin);
-            w_hi_max = wave_max_i(hmax);
-            if (__any(any_empty) || !cpl.uniform) w_lo_max = 0x3fffffff;  // such a wave never drops the mask
+            win = make_row_win(cached_row_map<BM>(&s_ps, cur_seg, wave * 32 + lm), cpl);
+            const bool empty = win.cnt <= 0;
+            w_lo_min = wave_min_i(empty ? 0x3fffffff : win.lo);
+            w_lo_max = wave_max_i(empty ? -0x3fffffff : win.lo);
+            w_hi_min = wave_min_i(empty ? 0x3fffffff : win.lo + win.cnt);
+            w_hi_max = wave_max_i(empty ? -0x3fffffff : win.lo + win.cnt);
+            if (__any(empty) || !cpl.uniform) w_lo_max = 0x3fffffff;  // such a wave never drops the mask
         }
-        const int j0 = cur_tile * kBN;
+        const int j0 = cur_tile * BN;
         ++cur_tile;
 
-        const bool more = (it + 1 < total_tiles);
-        if (more) {
-            issue_tile(ppl, pf_tile, (it + 1) & 1);
-            ++pf_tile;
-            pf_normalise();
+        // This wavefront's part of tile `it` has landed once at most the copies of the later tiles in flight
+        // are outstanding; after the barrier every part has, and every wavefront is done with tile it - 1,
+        // whose stage the next fetch overwrites.
+        {
+            const int later = total_tiles - 1 - it;
+            if (PD == 1 || later == 0)
+                wait_loads<0>();
+            else if (later == 1)
+                wait_loads<NDMA>();
+            else
+                wait_loads<NDMA*(PD > 1 ? PD - 1 : 1)>();
+        }
+        __builtin_amdgcn_s_barrier();
+
+        const bool fetch = (it + PD < total_tiles);
+        bool spread = false;  // the fetch is issued piecewise between the matrix instructions below
+        if (fetch) {
+            spread = tile_is_fast(ppl, pf_tile);
+            if (!spread) issue_tile_general(ppl, pf_tile, stage_pf);
         }
 
-        const bool skip = (j0 + kBN <= w_lo_min) || (j0 >= w_hi_max);
+        const bool skip = (j0 + BN <= w_lo_min) || (j0 >= w_hi_max);
         if (!skip) {
-            const bool full = (j0 >= w_lo_max) && (j0 + kBN <= w_hi_min);
+            const bool full = (j0 >= w_lo_max) && (j0 + BN <= w_hi_min);
 
             // ---- S^T = K . Q^T ----
-            // All K fragments of a 32-key tile are requested from LDS before the first MFMA that needs them, so
-            // that the reads of tile nt+1 are in flight while the matrix unit works on tile nt.
-            f32x16 s_acc[MT][NT];
+            // All K fragments of the tile are requested from LDS before the first MFMA that needs them.
+            f32x16 s_acc[NT];
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
+            for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                    for (int j = 0; j < 16; ++j) s_acc[mt][nt][j] = 0.f;
+                for (int j = 0; j < 16; ++j) s_acc[nt][j] = 0.f;
             Frag<T> kfr[NT][KS];
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
@@ -389,7 +390,7 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
                             kf.v = __builtin_bit_cast(typename Frag<T>::vec, lds_load128(k_addr[ks] + 32 * nt * G::K_ROWB));
                         }
                     } else {
-                        const char* ks_l = smem + (it & 1) * G::STAGE;
+                        const char* ks_l = smem + stage_it * G::STAGE;
                         if constexpr (KT) {
 #pragma unroll
                             for (int e = 0; e < 8; ++e)
@@ -401,24 +402,33 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
                 }
             }
             __builtin_amdgcn_sched_barrier(0);  // keep the requests above the matrix work
+            // the copy instructions of the fetch go between the MFMAs, so that the address path sees them at
+            // the rate it can take instead of as one burst that stalls the wavefront
+            constexpr int NMMA = NT * KS;
+            constexpr int MMA_PER_DMA = (NMMA / NDMA) > 0 ? NMMA / NDMA : 1;
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
+            for (int i = 0; i < NMMA; ++i) {
+                mma32(s_acc[i / KS], kfr[i / KS][i % KS], qf[i % KS]);
+                if constexpr (FAST_DMA) {
+                    if ((i + 1) % MMA_PER_DMA == 0 && (i + 1) / MMA_PER_DMA <= NDMA) {
+                        if (spread) issue_step((i + 1) / MMA_PER_DMA - 1, stage_pf);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            }
+            if constexpr (FAST_DMA && (NMMA / MMA_PER_DMA < NDMA)) {
+                if (spread) {
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt) mma32(s_acc[mt][nt], kfr[nt][ks], qf[mt][ks]);
+                    for (int s = NMMA / MMA_PER_DMA; s < NDMA; ++s) issue_step(s, stage_pf);
+                }
+            }
 
             // ---- mask, online softmax against a lazily updated reference ----
-            Frag<T> pf[MT][NT][2];
-            if (full) {
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-                    softmax_tile<true, T, DT>(s_acc[mt], pf[mt], m_ref[mt], l_run[mt], o_acc[mt], win[mt], true, j0, g, c2);
-            } else {
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-                    softmax_tile<false, T, DT>(s_acc[mt], pf[mt], m_ref[mt], l_run[mt], o_acc[mt], win[mt], cpl.uniform != 0, j0, g, c2);
-            }
+            Frag<T> pf[NT][2];
+            if (full)
+                softmax_tile<true, NT, T, DT>(s_acc, pf, m_ref, l_run, o_acc, win, true, j0, g, c2);
+            else
+                softmax_tile<false, NT, T, DT>(s_acc, pf, m_ref, l_run, o_acc, win, cpl.uniform != 0, j0, g, c2);
 
             // ---- O^T += V^T . P^T ----
             // V fragments are requested one 16-key step (DT fragments) ahead of the MFMAs that consume them.
@@ -449,66 +459,69 @@ __global__ __launch_bounds__(256, (MT == 1 && sizeof(T) == 2) ? 2 : 1) void attn
                 }
                 __builtin_amdgcn_sched_barrier(0);  // keep the requests above the matrix work
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt) mma32(o_acc[mt][dt], vfr[step & 1][dt], pf[mt][nt][t]);
+                for (int dt = 0; dt < DT; ++dt) mma32(o_acc[dt], vfr[step & 1][dt], pf[nt][t]);
             }
+        } else if (spread) {
+#pragma unroll
+            for (int s = 0; s < NDMA; ++s) issue_step(s, stage_pf);
         }
 
-        // the other stage becomes current
+        if (fetch) {
+            advance_fetch();
+            stage_pf = (stage_pf + 1 == NSTAGE) ? 0 : stage_pf + 1;
+        }
+        // the next stage becomes current
+        stage_it = (stage_it + 1 == NSTAGE) ? 0 : stage_it + 1;
+        const int delta = (stage_it == 0) ? -(NSTAGE - 1) * G::STAGE : G::STAGE;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) v_addr[dt] ^= G::STAGE;
+        for (int dt = 0; dt < DT; ++dt) v_addr[dt] += delta;
 #pragma unroll
-        for (int i = 0; i < (KT ? NT : KS); ++i) k_addr[i] ^= G::STAGE;
-
-        dma_wait_all();   // the next tile has landed in LDS
-        __syncthreads();  // ... for every wavefront, and this tile's stage may be overwritten
+        for (int i = 0; i < (KT ? NT : KS); ++i) k_addr[i] += delta;
     }
+    // every copy has been waited for (the last tile waits for all); the stages become staging space below once
+    // every wavefront has finished reading the last tile
+    __builtin_amdgcn_s_barrier();
 
     // ---- epilogue: O = O^T / l, transposed through LDS so that every global store is a contiguous run --------
-    // (all wavefronts left the loop through its final barrier; each one now uses a private region of the stages)
     {
         constexpr int OROW = D * ES + 16;  // padded row of the staging tile
+        static_assert(4 * 32 * OROW <= NSTAGE * G::STAGE, "staging space");
         char* stg = smem + wave * (32 * OROW);
+        const float l_tot = l_run + __shfl_xor(l_run, 32);
+        const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const float l_tot = l_run[mt] + __shfl_xor(l_run[mt], 32);
-            const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
+            for (int jj = 0; jj < 4; ++jj) {
+                typedef T vec4 __attribute__((ext_vector_type(4)));
+                vec4 o;
 #pragma unroll
-                for (int jj = 0; jj < 4; ++jj) {
-                    typedef T vec4 __attribute__((ext_vector_type(4)));
-                    vec4 o;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) o[i] = (T)(o_acc[mt][dt][4 * jj + i] * inv);
-                    *reinterpret_cast<vec4*>(stg + lm * OROW + (32 * dt + 8 * jj + 4 * g) * ES) = o;
-                }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wavefront's LDS writes are visible to its own reads
-            constexpr int CPR = D * ES / 16;                    // 16-byte chunks per output row
-#pragma unroll
-            for (int i = 0; i < 32 * CPR / 64; ++i) {
-                const int flat = i * 64 + lane;
-                const int row = flat / CPR, c = flat % CPR;
-                const int r = r0 + rs * ((wave * MT + mt) * 32 + row);
-                const u32x4 val = *reinterpret_cast<const u32x4*>(stg + row * OROW + c * 16);
-                if (r < L) *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(ob + (int64_t)r * p.o_sl) + c * 16) = val;
+                for (int i = 0; i < 4; ++i) o[i] = (T)(o_acc[dt][4 * jj + i] * inv);
+                *reinterpret_cast<vec4*>(stg + lm * OROW + (32 * dt + 8 * jj + 4 * g) * ES) = o;
             }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // reads done before the next m-tile reuses the region
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wavefront's LDS writes are visible to its own reads
+        constexpr int CPR = D * ES / 16;                    // 16-byte chunks per output row
+#pragma unroll
+        for (int i = 0; i < 32 * CPR / 64; ++i) {
+            const int flat = i * 64 + lane;
+            const int row = flat / CPR, c = flat % CPR;
+            const int r = r0 + rs * (wave * 32 + row);
+            const u32x4 val = *reinterpret_cast<const u32x4*>(stg + row * OROW + c * 16);
+            if (r < L) *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(ob + (int64_t)r * p.o_sl) + c * 16) = val;
         }
     }
 }
 
-template <typename T, int D, int MT, bool KT>
+template <typename T, int D, bool KT, int BN, int NSTAGE>
 static int launch_attn(const AttnParams& p0, hipStream_t st) {
-    using G = TileGeom<T, D, KT>;
+    using G = TileGeom<T, D, KT, BN>;
     AttnParams p = p0;
-    constexpr int BM = 128 * MT;
+    constexpr int BM = 128;
     p.n_row_blocks = count_row_blocks(p.L, BM, p.row_stride);
     p.total = p.B * p.H * p.n_row_blocks;
     const int grid = ((p.total + 7) / 8) * 8;
-    const size_t lds = 2 * (size_t)G::STAGE;
-    auto kern = attn_fwd_kernel<T, D, MT, KT>;
+    const size_t lds = NSTAGE * (size_t)G::STAGE;
+    auto kern = attn_fwd_kernel<T, D, KT, BN, NSTAGE>;
     static thread_local bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -522,13 +535,13 @@ static int launch_attn(const AttnParams& p0, hipStream_t st) {
     return check_launch("splat_attention_fwd");
 }
 
+// One 32-row tile per wavefront (128 rows per workgroup): 16-bit kernels then fit two workgroups per CU, whose
+// wavefronts hide part of each other's LDS, barrier and prologue latency.  Tiles of 64 keys, double buffered (the
+// kernel also supports 32-key tiles in a ring of 4 stages; it measured slower at d = 128 and equal at d = 64).
 template <typename T>
 static int dispatch_attn(const AttnParams& p, int d, bool kt, hipStream_t st) {
-    // One 32-row tile per wavefront (BM = 128): 16-bit kernels then fit two workgroups per CU, whose
-    // wavefronts hide each other's LDS, barrier and prologue latency.  Two tiles per wavefront (MT = 2) halve
-    // the LDS traffic per MFMA but need all 512 registers of a SIMD lane and measured slower.
-    if (d == 64) return kt ? launch_attn<T, 64, 1, true>(p, st) : launch_attn<T, 64, 1, false>(p, st);
-    return kt ? launch_attn<T, 128, 1, true>(p, st) : launch_attn<T, 128, 1, false>(p, st);
+    if (d == 64) return kt ? launch_attn<T, 64, true, 64, 2>(p, st) : launch_attn<T, 64, false, 64, 2>(p, st);
+    return kt ? launch_attn<T, 128, true, 64, 2>(p, st) : launch_attn<T, 128, false, 64, 2>(p, st);
 }
 
 }  // namespace splat

@@ -4,15 +4,15 @@
 
 namespace splat {
 
-template <typename T, int D, bool KT>
+template <typename T, int D, bool KT, int BN = kBN>
 struct TileGeom {
     static constexpr int ES = sizeof(T);
     static constexpr int EPC = 16 / ES;                       // elements per 16-byte chunk
-    static constexpr int K_ROWB = KT ? kBN * ES : D * ES;     // bytes per LDS row of the K tile (no padding)
-    static constexpr int K_ROWS = KT ? D : kBN;
+    static constexpr int K_ROWB = KT ? BN * ES : D * ES;      // bytes per LDS row of the K tile (no padding)
+    static constexpr int K_ROWS = KT ? D : BN;
     static constexpr int V_ROWB = D * ES;
     static constexpr int K_BYTES = K_ROWB * K_ROWS;
-    static constexpr int V_BYTES = V_ROWB * kBN;
+    static constexpr int V_BYTES = V_ROWB * BN;
     static constexpr int STAGE = K_BYTES + V_BYTES;
 };
 
