@@ -127,6 +127,14 @@ __global__ __launch_bounds__(256, 2) void spmm_kernel(const SpmmParams p) {
             const int u = jj - w.lo;
             if (w.lin == 1 && u >= 0 && u + 8 <= w.cnt) {
                 __builtin_memcpy(&v, wrow[c] + u, 8 * ES);  // any alignment
+            } else if (w.lin == 1) {
+                // an end of the row's span (or outside it): range test per slot, loads from a clamped slot so that
+                // they need no branch
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const T x = wrow[c][min(max(u + e, 0), max(w.cnt - 1, 0))];
+                    v[e] = ((unsigned)(u + e) < (unsigned)w.cnt) ? x : (T)0.f;
+                }
             } else {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) v[e] = win_live(w, jj + e) ? wrow[c][win_slot(w, jj + e)] : (T)0.f;
