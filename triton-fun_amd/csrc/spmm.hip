@@ -18,6 +18,7 @@ struct SpmmParams {
     int64_t v_sb, v_sh, v_sl;
     int B, H, L, n_keys, n_out, T;
     int out_dtype;
+    int out_vec;  // 16-byte stores are legal for every row of out
     int n_seg;
     SegPtrs seg[SPLAT_MAX_SEGMENTS];
     int n_row_blocks, total, n_col_chunks;
@@ -184,6 +185,44 @@ __global__ __launch_bounds__(256, 2) void spmm_kernel(const SpmmParams p) {
         }
     }
 
+    // ---- epilogue ----
+    // An accumulator register holds one row's value at column lm: stored directly, a wavefront instruction writes 32
+    // consecutive elements of two rows.  When rows of the output can take 16-byte stores, each 32 x 32 tile is instead
+    // converted, turned around in the wavefront's staging area and written as 16-byte pieces (8 or 4 per row).
+    __syncthreads();  // every wavefront is done with the staging areas and the V tile
+    const int es_out = (p.out_dtype == SPLAT_F32) ? 4 : 2;
+    const bool wide = p.out_vec && (col0 + 32 * DVT <= p.n_out);
+    if (wide) {
+        char* stg = s_p[wave];
+        static_assert(32 * P_ROW >= 32 * (32 * 4 + 16), "staging area holds a 32 x 32 fp32 tile");
+        const int row_b = 32 * es_out + 16;  // padded staging row
+        const int cpr = 32 * es_out / 16;     // 16-byte pieces per row
+#pragma unroll
+        for (int dt = 0; dt < DVT; ++dt) {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                char* dst = stg + acc_row(j, g) * row_b + lm * es_out;
+                if (p.out_dtype == SPLAT_BF16)
+                    *reinterpret_cast<bf16*>(dst) = (bf16)acc[dt][j];
+                else if (p.out_dtype == SPLAT_F16)
+                    *reinterpret_cast<f16*>(dst) = (f16)acc[dt][j];
+                else
+                    *reinterpret_cast<float*>(dst) = acc[dt][j];
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wavefront's LDS writes are visible to its own reads
+            for (int flat = lane; flat < 32 * cpr; flat += 64) {
+                const int row = flat / cpr, c = flat % cpr;
+                const int r = r0 + rs * (32 * wave + row);
+                const u32x4 val = *reinterpret_cast<const u32x4*>(stg + row * row_b + c * 16);
+                if (r < L) {
+                    char* orow = reinterpret_cast<char*>(p.out) + (((int64_t)bh * L + r) * p.n_out + col0 + 32 * dt) * es_out;
+                    *reinterpret_cast<u32x4*>(orow + c * 16) = val;
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // reads done before the next tile overwrites the staging
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
         const int r = r0 + rs * (32 * wave + acc_row(j, g));
@@ -243,6 +282,10 @@ extern "C" int splat_spmm(const void* pp, const void* v, int64_t v_sb, int64_t v
     const int es = in_dtype == SPLAT_F32 ? 4 : 2;
     const int epc = 16 / es;
     p.v_vec = ((reinterpret_cast<uintptr_t>(v) & 15) == 0 && v_sb % epc == 0 && v_sh % epc == 0 && v_sl % epc == 0) ? 1 : 0;
+    {
+        const int es_out = out_dtype == SPLAT_F32 ? 4 : 2;
+        p.out_vec = ((reinterpret_cast<uintptr_t>(out) & 15) == 0 && ((int64_t)n_out * es_out) % 16 == 0) ? 1 : 0;
+    }
     hipStream_t st = (hipStream_t)stream;
     switch (in_dtype) {
         case SPLAT_F32: return launch_spmm<float>(p, st);
