@@ -176,3 +176,43 @@ def test_long_sequences_by_properties(dev, L, d, w, dtype):
         s = (q[0, 0, r].float() @ k[0, 0, lo:r + 1].float().T) * scale
         want = torch.softmax(s, -1) @ v[0, 0, lo:r + 1].float()
         assert float((out[0, 0, r] - want).abs().max()) <= TOL[dtype], r
+
+
+def _random_affine_mask(rng, L):
+    """Every row an arbitrary affine set a + step*t, t < cnt (what ACSR can represent), with empty rows,
+    single-column rows and rows reaching the last column mixed in."""
+    mask = np.zeros((L, L), dtype=np.uint8)
+    for r in range(L):
+        kind = rng.integers(0, 10)
+        if kind == 0:
+            continue  # empty row
+        a = int(rng.integers(0, L))
+        if kind == 1:
+            mask[r, a] = 1  # single column
+            continue
+        step = int(rng.integers(1, max(2, L // 3)))
+        cnt = int(rng.integers(2, max(3, (L - 1 - a) // step + 2)))
+        cols = a + step * np.arange(cnt)
+        cols = cols[cols < L]
+        if kind == 2:  # run to the end of the row
+            cols = np.arange(a, L, step)
+        mask[r, cols] = 1
+    return mask
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_affine_rows_against_oracle(dev, seed):
+    """Rows with unrelated starts, steps and lengths (the dense-column plan, its per-position validity test, the
+    first-column side channel of single-column rows), sizes that are no multiple of any tile, all three kernels'
+    composition and the fused kernel, both 16-bit types and fp32."""
+    rng = np.random.default_rng(1234 + seed)
+    L = int(rng.integers(1, 330))
+    d = (64, 128)[seed % 2]
+    dtype = (torch.float32, torch.float16, torch.bfloat16)[seed % 3]
+    mask = _random_affine_mask(rng, L)
+    q, k, v = O.make_inputs(77 + seed, 1, 2, L, d, dtype)
+    want = O.dense_masked_attention(q, k.transpose(2, 3), v, mask, d ** -0.5)
+    for fused in (True, False):
+        got = run_module(mask, 1, 2, L, d, dtype, dev, q, k, v, d ** -0.5, fused)
+        assert float((got - want).abs().max()) <= TOL[dtype], (fused, L, d, dtype)
+        assert torch.all(got[:, :, mask.sum(1) == 0] == 0)
