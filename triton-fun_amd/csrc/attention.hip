@@ -46,27 +46,40 @@ struct AttnParams {
 
 constexpr float kRescaleThreshold = 8.0f;  // in log2 units: exponentials stay below 2^8 before the reference moves
 
-// Mask (unless FULL), fold one tile of 32*NT keys of scores of one 32-row tile into the running softmax state
-// and emit the exponentials as MFMA B fragments.  One lane owns one query row (half of its positions).
+// Live positions of one row in the tile that starts at position j0, one bit per position (bit b = position j0 + b):
+// the row's span [lo, lo + cnt) intersected with its periodic pattern.  `first` is the smallest offset >= 0 in the tile
+// whose position is congruent to the row's first one modulo its step (0 for unit step) and `pat` has a bit at every
+// multiple of the step below 64.
+__device__ __forceinline__ uint64_t row_live_bits(const RowWin& w, int j0, int first, uint64_t pat) {
+    const int a = w.lo - j0, b = a + w.cnt;  // live range [a, b) in tile offsets
+    const uint64_t lo_m = a <= 0 ? ~0ull : (a >= 64 ? 0ull : ~0ull << a);
+    const uint64_t hi_m = b >= 64 ? ~0ull : (b <= 0 ? 0ull : (1ull << b) - 1ull);
+    const uint64_t per = first < 64 ? pat << first : 0ull;
+    return lo_m & hi_m & per;
+}
+
+// x where keep is -1, the masked score -1e30 where keep is 0 (one bit-field insert)
+__device__ __forceinline__ float keep_or_mask(float x, int keep) {
+    const uint32_t xb = __builtin_bit_cast(uint32_t, x), nb = __builtin_bit_cast(uint32_t, kNegBigA);
+    return __builtin_bit_cast(float, (xb & (uint32_t)keep) | (nb & ~(uint32_t)keep));
+}
+
+// Mask (unless FULL), fold one tile of 32*NT keys of scores of one 32-row tile into the running softmax state and
+// emit the exponentials as MFMA B fragments.  One lane owns one query row (half of its positions: accumulator
+// register j of 32-key half nt holds position 32*nt + 8*(j/4) + 4*g + j%4, whose bit of `live` says whether it is
+// kept; see row_live_bits).
 template <bool FULL, int NT, typename T, int DT>
 __device__ __forceinline__ void softmax_tile(f32x16 (&s)[NT], Frag<T> (&pf)[NT][2], float& m_ref, float& l_run,
-                                             f32x16 (&o)[DT], const RowWin& win, bool uniform, int j0, int g, float c2) {
+                                             f32x16 (&o)[DT], uint64_t live, int g, float c2) {
     if constexpr (!FULL) {
-        if (uniform) {  // live iff 0 <= position - lo < cnt
-            const int base = j0 + 4 * g - win.lo;
-            const unsigned cnt = (unsigned)win.cnt;
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
+        for (int nt = 0; nt < NT; ++nt) {
+            const uint32_t bits = (uint32_t)(live >> (32 * nt)) >> (4 * g);
 #pragma unroll
-                for (int j = 0; j < 16; ++j) {
-                    const unsigned u = (unsigned)(base + 32 * nt + 8 * (j >> 2) + (j & 3));
-                    s[nt][j] = (u < cnt) ? s[nt][j] : kNegBigA;
-                }
-        } else {
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                for (int j = 0; j < 16; ++j) s[nt][j] = win_live(win, j0 + 32 * nt + acc_row(j, g)) ? s[nt][j] : kNegBigA;
+            for (int j = 0; j < 16; ++j) {
+                const int c = 8 * (j >> 2) + (j & 3);
+                s[nt][j] = keep_or_mask(s[nt][j], ((int)(bits << (31 - c))) >> 31);
+            }
         }
     }
     float mx = s[0][0];
@@ -312,6 +325,8 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
     // per-lane row map of the segment being computed
     int cur_seg = -1, cur_tile = 0;
     RowWin win = {0, 0, 1};
+    int first = 0, dec = 0;  // periodic part of the row mask of dense plans: see row_live_bits
+    uint64_t pat = ~0ull;
     int w_lo_min = 0, w_lo_max = 0, w_hi_min = 0, w_hi_max = 0;
     SegPlan cpl = {0, 1, 0, 1};
     const float c2 = p.scale_log2e;
@@ -333,6 +348,19 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
                 cpl.uniform = __builtin_amdgcn_readfirstlane(t.uniform);
             }
             win = make_row_win(cached_row_map<BM>(&s_ps, cur_seg, wave * 32 + lm), cpl);
+            if (!cpl.uniform) {
+                // periodic part of the row's live positions (position 0 of the walk is column c0)
+                const int lin = win.lin;
+                const int f = win.lo % lin;
+                first = f < 0 ? f + lin : f;
+                dec = BN % lin;
+                uint64_t pt = 0;
+                for (int q = 0; q < 64; q += lin) pt |= 1ull << q;
+                pat = pt;
+            } else {  // unit step: every position of the span
+                first = 0;
+                pat = ~0ull;
+            }
             const bool empty = win.cnt <= 0;
             w_lo_min = wave_min_i(empty ? 0x3fffffff : win.lo);
             w_lo_max = wave_max_i(empty ? -0x3fffffff : win.lo);
@@ -426,9 +454,9 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
             // ---- mask, online softmax against a lazily updated reference ----
             Frag<T> pf[NT][2];
             if (full)
-                softmax_tile<true, NT, T, DT>(s_acc, pf, m_ref, l_run, o_acc, win, true, j0, g, c2);
+                softmax_tile<true, NT, T, DT>(s_acc, pf, m_ref, l_run, o_acc, 0ull, g, c2);
             else
-                softmax_tile<false, NT, T, DT>(s_acc, pf, m_ref, l_run, o_acc, win, cpl.uniform != 0, j0, g, c2);
+                softmax_tile<false, NT, T, DT>(s_acc, pf, m_ref, l_run, o_acc, row_live_bits(win, j0, first, pat), g, c2);
 
             // ---- O^T += V^T . P^T ----
             // V fragments are requested one 16-key step (DT fragments) ahead of the MFMAs that consume them.
@@ -469,6 +497,10 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
         if (fetch) {
             advance_fetch();
             stage_pf = (stage_pf + 1 == NSTAGE) ? 0 : stage_pf + 1;
+        }
+        if (!cpl.uniform) {  // phase of the periodic mask at the next tile
+            const int f = first - dec;
+            first = f < 0 ? f + win.lin : f;
         }
         // the next stage becomes current
         stage_it = (stage_it + 1 == NSTAGE) ? 0 : stage_it + 1;
