@@ -145,6 +145,29 @@ int splat_attention_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl,
                         int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t d, float scale,
                         int32_t dtype, void* stream);
 
+/* Plan of the fused forward for one mask: per 128-row block the key tiles it walks, per row its window in
+ * tile positions.  splat_attention_fwd derives these from the ACSR arrays in every workgroup of every
+ * launch; a module that attends with one mask many times (RegularAttention, r_attention.py:14-100, whose
+ * constructor already holds every per-mask buffer) builds the plan once and calls
+ * splat_attention_fwd_planned, whose workgroups start on their first tile after two small loads.
+ * The reference has no counterpart (its kernels redo the affine index arithmetic per element).
+ *
+ * splat_attention_plan_bytes: size of the plan for these segments and L rows (0 for invalid arguments);
+ *   host-only arithmetic, reads nothing on the device.
+ * splat_attention_plan: fill `plan` (device memory, 16-byte aligned, plan_bytes >= the size above).
+ * splat_attention_fwd_planned: as splat_attention_fwd, with the plan of the same segments and L; results
+ *   are bit-identical to splat_attention_fwd.  A plan built from other segments or another L gives
+ *   undefined results (only its size is checked). */
+int64_t splat_attention_plan_bytes(const splat_acsr_seg* segs /* host */, int32_t n_seg, int32_t L);
+int splat_attention_plan(const splat_acsr_seg* segs /* host */, int32_t n_seg, int32_t L, void* plan,
+                         int64_t plan_bytes, void* stream);
+int splat_attention_fwd_planned(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT,
+                                int64_t k_sb, int64_t k_sh, int64_t k_sd, int64_t k_sl, const void* v,
+                                int64_t v_sb, int64_t v_sh, int64_t v_sl, void* out, int64_t o_sb,
+                                int64_t o_sh, int64_t o_sl, const splat_acsr_seg* segs /* host */,
+                                int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t d, float scale,
+                                int32_t dtype, const void* plan, int64_t plan_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,7 +23,8 @@ def header_symbols():
 def test_library_exports_every_declared_symbol():
     syms = header_symbols()
     assert {"splat_acsr_build", "splat_mask_generate", "splat_sddmm", "splat_softmax", "splat_spmm",
-            "splat_attention_fwd", "splat_version", "splat_last_error"} <= set(syms)
+            "splat_attention_fwd", "splat_attention_plan_bytes", "splat_attention_plan", "splat_attention_fwd_planned",
+            "splat_version", "splat_last_error"} <= set(syms)
     handle = ctypes.CDLL(hip.LIB_PATH)
     for s in syms:
         assert hasattr(handle, s), s
@@ -48,8 +49,27 @@ def test_null_and_shape_arguments_are_rejected_without_a_device():
     assert lib.splat_attention_fwd(8, 0, 0, 64, 8, 0, 0, 1, 64, 8, 0, 0, 64, 8, 0, 0, 64, seg, 1, 1, 1, 16, 48, 1.0, 2,
                                    None) == -5                                   # d = 48 unsupported
     assert b"64 or 128" in lib.splat_last_error()
+    assert lib.splat_attention_fwd_planned(8, 0, 0, 64, 8, 0, 0, 1, 64, 8, 0, 0, 64, 8, 0, 0, 64, seg, 1, 1, 1, 16, 48, 1.0, 2,
+                                           16, 1 << 20, None) == -5
+    assert b"splat_attention_fwd_planned" in lib.splat_last_error()
     assert lib.splat_sddmm(8, 0, 0, 8, 8, 0, 0, 3, 5, 8, seg, 1, 1, 1, 4, 4, 8, 4, 1.0, 0, 0, None) == -4  # no unit stride
     assert lib.splat_spmm(8, 8, 0, 0, 8, 8, seg, 1, 1, 1, 4, 4, 8, 4, 7, 0, None) == -3                    # bad dtype
+
+
+def test_plan_size_is_host_arithmetic():
+    lib = hip.lib()
+    seg = (hip.AcsrSeg * 2)()
+    # per variant and segment: per 128-row block one plan record, four wavefront spans and 128 row windows of 16 bytes
+    assert lib.splat_attention_plan_bytes(seg, 1, 16384) == 2 * 128 * (5 + 128) * 16
+    assert lib.splat_attention_plan_bytes(seg, 2, 130) == 2 * 2 * 2 * (5 + 128) * 16
+    seg[0].row_stride_hint = seg[1].row_stride_hint = 2        # rows 0, 2, 4, .. and 1, 3, 5, .. in separate blocks
+    assert lib.splat_attention_plan_bytes(seg, 2, 130) == 2 * 2 * 2 * (5 + 128) * 16
+    assert lib.splat_attention_plan_bytes(seg, 2, 300) == 2 * 2 * 4 * (5 + 128) * 16
+    assert lib.splat_attention_plan_bytes(seg, 0, 16) == 0 and lib.splat_attention_plan_bytes(None, 1, 16) == 0
+    assert lib.splat_attention_plan(seg, 1, 16, None, 0, None) == -1
+    seg[0].sTod_lin = seg[0].sTod_trans = seg[0].nnz = 8
+    assert lib.splat_attention_plan(seg, 1, 16, 16, 100, None) == -2 and b"bytes" in lib.splat_last_error()
+    assert lib.splat_attention_plan(seg, 1, 16, 24, 1 << 20, None) == -4      # misaligned plan
 
 
 def test_operators_refuse_the_host():

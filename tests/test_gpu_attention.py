@@ -216,3 +216,53 @@ def test_random_affine_rows_against_oracle(dev, seed):
         got = run_module(mask, 1, 2, L, d, dtype, dev, q, k, v, d ** -0.5, fused)
         assert float((got - want).abs().max()) <= TOL[dtype], (fused, L, d, dtype)
         assert torch.all(got[:, :, mask.sum(1) == 0] == 0)
+
+
+def _plan_cases():
+    rng = np.random.default_rng(99)
+    return [
+        ("causal window", lambda: A.causal_windowed_pattern(1000, 100), 1000, 64, torch.float16),
+        ("two-sided window, ragged L", lambda: A.windowed_pattern(333, 40), 333, 128, torch.bfloat16),
+        ("dilated (row-stride blocks)", lambda: A.dilated_pattern(1024, 128, 2), 1024, 128, torch.bfloat16),
+        ("strided, two segments", lambda: A.strided_patterns(1024, 128, 128), 1024, 64, torch.bfloat16),
+        ("blocked", lambda: O.create_blocked_mask(640, 128), 640, 64, torch.float32),
+        ("random affine rows", lambda: _random_affine_mask(rng, 300), 300, 128, torch.float16),
+    ]
+
+
+@pytest.mark.parametrize("case", _plan_cases(), ids=lambda c: c[0])
+def test_planned_forward_equals_unplanned(dev, case):
+    """splat_attention_fwd derives every workgroup's tiles from the ACSR arrays, splat_attention_fwd_planned reads
+    them from the plan built once per mask: the same kernel otherwise, so the outputs agree bit for bit, for row-major
+    and key-contiguous K (the plan's two variants)."""
+    _, make, L, d, dtype = case
+    B, H = 2, 3
+    attn = RegularAttention(B, L, H, d, make(), 16, 16, dev, dtype, scale=d ** -0.5)
+    q, k, v = [t.to(dev) for t in O.make_inputs(L, B, H, L, d, dtype)]
+    plan = A_plan(attn, L, dev)
+    epc = 4 if dtype == torch.float32 else 8
+    for contig in ((False, True) if L % epc == 0 else (False,)):
+        kT = k.transpose(2, 3).contiguous() if contig else k.transpose(2, 3)
+        a = torch.full((B, H, L, d), 7, dtype=dtype, device=dev)
+        b = torch.full((B, H, L, d), 9, dtype=dtype, device=dev)
+        attention_launcher(q, kT, v, a, attn.segments, attn.scale)
+        attention_launcher(q, kT, v, b, attn.segments, attn.scale, plan)
+        assert torch.equal(a, b), contig
+        assert torch.equal(attn([q, kT, v]), a), contig  # the module plans by itself
+
+
+def A_plan(attn, L, dev):
+    from r_attention import attention_plan
+    return attention_plan(attn.segments, L, dev)
+
+
+def test_plan_arguments_are_checked(dev):
+    import _splat_hip as hip
+    L, d = 256, 64
+    attn = RegularAttention(1, L, 1, d, A.causal_windowed_pattern(L, 31), 16, 16, dev, torch.float16)
+    q = torch.zeros(1, 1, L, d, dtype=torch.float16, device=dev)
+    plan = A_plan(attn, L, dev)
+    with pytest.raises(hip.SplatError, match="bytes"):
+        attention_launcher(q, q.transpose(2, 3), q, torch.empty_like(q), attn.segments, 1.0, plan[:-16])
+    with pytest.raises(hip.SplatError):
+        attention_launcher(q, q.transpose(2, 3), q, torch.empty_like(q), attn.segments, 1.0, plan.cpu())

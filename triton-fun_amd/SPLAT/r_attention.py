@@ -29,11 +29,27 @@ def _is_segment_list(mask) -> bool:
     return isinstance(mask, (list, tuple)) and len(mask) > 0 and isinstance(mask[0], (MaskPattern, torch.Tensor))
 
 
+def attention_plan(segments: ACSRSegments, L: int, device) -> torch.Tensor:
+    """The fused kernel's plan for these segments and ``L`` rows (which key tiles each 128-row block walks, every
+    row's window): an opaque uint8 device tensor, built once per mask and handed to ``attention_launcher``."""
+    dev = _hip.resolve_device(device)
+    arr = _hip.seg_array(segments.seg_args())
+    nbytes = int(_hip.lib().splat_attention_plan_bytes(arr, len(segments), L))
+    if nbytes <= 0:
+        raise _hip.SplatError(f"no plan for {len(segments)} segments and L={L}")
+    plan = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        rc = _hip.lib().splat_attention_plan(arr, len(segments), L, plan.data_ptr(), nbytes, _hip.stream_ptr(dev))
+    _hip.check(rc, "splat_attention_plan")
+    return plan
+
+
 def attention_launcher(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor, output: torch.Tensor,
-                       segments: ACSRSegments, scale: float = 1.0) -> torch.Tensor:
+                       segments: ACSRSegments, scale: float = 1.0, plan: torch.Tensor | None = None) -> torch.Tensor:
     """Fused forward: output[b, h, r, :] = softmax over the live columns of (scale * q.kT)[b, h, r, :] times v.
     q [B, H, L, d], kT [B, H, d, L] (unit stride along d or along L), v [B, H, L, d], output [B, H, L, d];
-    d in {64, 128}; one dtype for all four."""
+    d in {64, 128}; one dtype for all four.  ``plan`` (from ``attention_plan`` for the same segments and L) spares
+    every workgroup the derivation of its tiles from the ACSR arrays; the results are the same."""
     for name, t in (("q", q), ("kT", kT), ("v", v), ("output", output)):
         _hip.require_device_tensor(t, name)
         if t.dim() != 4:
@@ -55,12 +71,20 @@ def attention_launcher(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor, outpu
     qs, ks, vs, os_ = q.stride(), kT.stride(), v.stride(), output.stride()
     dev = q.device
     arr = _hip.seg_array(segments.seg_args())
+    args = (q.data_ptr(), qs[0], qs[1], qs[2], kT.data_ptr(), ks[0], ks[1], ks[2], ks[3],
+            v.data_ptr(), vs[0], vs[1], vs[2], output.data_ptr(), os_[0], os_[1], os_[2],
+            arr, len(segments), B, H, L, d, float(scale), _hip.dtype_code(q.dtype))
     with torch.cuda.device(dev):
-        rc = _hip.lib().splat_attention_fwd(q.data_ptr(), qs[0], qs[1], qs[2], kT.data_ptr(), ks[0], ks[1], ks[2], ks[3],
-                                            v.data_ptr(), vs[0], vs[1], vs[2], output.data_ptr(), os_[0], os_[1], os_[2],
-                                            arr, len(segments), B, H, L, d, float(scale), _hip.dtype_code(q.dtype),
-                                            _hip.stream_ptr(dev))
-    _hip.check(rc, "splat_attention_fwd")
+        if plan is None:
+            rc = _hip.lib().splat_attention_fwd(*args, _hip.stream_ptr(dev))
+            _hip.check(rc, "splat_attention_fwd")
+        else:
+            _hip.require_device_tensor(plan, "plan")
+            if plan.device != dev:
+                raise _hip.SplatError(f"the plan lives on {plan.device}, the tensors on {dev}")
+            rc = _hip.lib().splat_attention_fwd_planned(*args, plan.data_ptr(), plan.numel() * plan.element_size(),
+                                                        _hip.stream_ptr(dev))
+            _hip.check(rc, "splat_attention_fwd_planned")
     return output
 
 
@@ -101,6 +125,7 @@ class RegularAttention(nn.Module):
         self.rspmm_output = torch.empty(self._shape, dtype=out_dtype, device=self._device)
         self.rspmm_grid_dim = (-(-head_dim // BLOCK_SIZE_X), -(-seq_length // BLOCK_SIZE_Y), batch * num_heads)
         self._unfused_ready = False
+        self._plan = None  # the fused kernel's plan of this mask, built on the first fused forward
 
     # The two [B, H, L, T] intermediates and the reference's launch geometry exist only for the unfused path.
     def _prepare_unfused(self):
@@ -138,7 +163,9 @@ class RegularAttention(nn.Module):
         q, k, v = x
         fusable = self.fused and q.shape[-1] in (64, 128) and q.dtype == k.dtype == v.dtype == self._out_dtype
         if fusable:
-            return attention_launcher(q, k, v, self.rspmm_output, self.segments, self.scale)
+            if self._plan is None:
+                self._plan = attention_plan(self.segments, self._shape[2], self._device)
+            return attention_launcher(q, k, v, self.rspmm_output, self.segments, self.scale, self._plan)
 
         multi = self.segments if len(self.segments) > 1 else None
         rsddmm_launcher(q, k, self.rsddmm_output,

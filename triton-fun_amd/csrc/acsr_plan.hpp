@@ -191,6 +191,50 @@ __device__ __forceinline__ int win_slot(const RowWin& w, int j) {
     return (w.lin == 1) ? u : u / w.lin;
 }
 
+// Width of a wavefront's rows in tile positions: the tiles before lo_min / from hi_max on hold nothing for it, the
+// tiles from lo_max on and up to hi_min need no mask.
+struct WaveSpan {
+    int lo_min, lo_max, hi_min, hi_max;
+};
+// Evaluated by the 64 lanes of a wavefront, each holding the window of one of its rows (both halves of the wavefront
+// hold the same 32 rows).
+__device__ __forceinline__ WaveSpan wave_span(const RowWin& win, bool uniform) {
+    const bool empty = win.cnt <= 0;
+    WaveSpan s;
+    s.lo_min = wave_min_i(empty ? 0x3fffffff : win.lo);
+    s.lo_max = wave_max_i(empty ? -0x3fffffff : win.lo);
+    s.hi_min = wave_min_i(empty ? 0x3fffffff : win.lo + win.cnt);
+    s.hi_max = wave_max_i(empty ? -0x3fffffff : win.lo + win.cnt);
+    if (__any(empty) || !uniform) s.lo_max = 0x3fffffff;  // such a wavefront never drops the mask
+    return s;
+}
+// smallest offset >= 0 from position 0 of the walk that is congruent to the row's first position modulo its step
+__device__ __forceinline__ int win_phase(const RowWin& w) {
+    const int f = w.lo % w.lin;
+    return f < 0 ? f + w.lin : f;
+}
+
+// ---- plan table: what a workgroup of the fused kernel derives from the ACSR metadata, stored once per mask ----
+// 16-byte records, two variants (0: gathered walks allowed, 1: dense walks only, for K^T-contiguous keys), each
+//   seg  [row block][segment]            SegPlan
+//   span [row block][segment][wavefront] WaveSpan
+//   row  [segment][row block][row k]     RowWin + phase (row k of the block is row first + stride * k)
+typedef int PlanRec __attribute__((ext_vector_type(4)));
+constexpr int kPlanBM = 128;  // rows per row block of the fused kernel
+__host__ __device__ inline int64_t plan_variant_recs(int n_rb, int n_seg) { return (int64_t)n_rb * n_seg * (5 + kPlanBM); }
+__host__ __device__ inline int64_t plan_seg_at(int n_seg, int rb, int sg) { return (int64_t)rb * n_seg + sg; }
+__host__ __device__ inline int64_t plan_span_at(int n_rb, int n_seg, int rb, int sg, int wave) {
+    return (int64_t)n_rb * n_seg + ((int64_t)rb * n_seg + sg) * 4 + wave;
+}
+__host__ __device__ inline int64_t plan_row_at(int n_rb, int n_seg, int rb, int sg, int k) {
+    return (int64_t)n_rb * n_seg * 5 + ((int64_t)sg * n_rb + rb) * kPlanBM + k;
+}
+// A record whose address is the same for the whole wavefront, through the scalar (constant) load path.
+typedef __attribute__((address_space(4))) const PlanRec const_plan_rec;
+__device__ __forceinline__ PlanRec plan_uniform_load(const PlanRec* p) {
+    return *reinterpret_cast<const_plan_rec*>(reinterpret_cast<uintptr_t>(p));
+}
+
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
 // Transposing LDS read: the 16 lanes of a block address 4 rows x 16 columns of 16-bit elements (lane s:

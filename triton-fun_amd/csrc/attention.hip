@@ -42,6 +42,7 @@ struct AttnParams {
     int n_row_blocks;
     int total;
     int row_stride;
+    const PlanRec* plan;  // plan table of this mask (PLANNED kernels), variant already selected
 };
 
 constexpr float kRescaleThreshold = 8.0f;  // in log2 units: exponentials stay below 2^8 before the reference moves
@@ -119,7 +120,7 @@ __device__ __forceinline__ void softmax_tile(f32x16 (&s)[NT], Frag<T> (&pf)[NT][
     l_run += rs;
 }
 
-template <typename T, int D, bool KT, int BN, int NSTAGE>
+template <typename T, int D, bool KT, int BN, int NSTAGE, bool PLANNED>
 __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(const AttnParams p) {
     using G = TileGeom<T, D, KT, BN>;
     constexpr int ES = G::ES;
@@ -164,12 +165,29 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) qf[ks] = global_frag<T>(qr + 16 * ks + 8 * g);
     }
-
-    // ---- plan: per segment, the column range and step of this row block ------------------------
-    plan_segments<BM, BN>(p.seg, p.n_seg, r0, rs, L, !KT, s_plan, &s_ps, tid);
+    // ---- plan: per segment, the column range and step of this row block; computed here from the rows' maps or
+    // taken from the mask's plan table (scalar loads: no LDS, no barrier) ------------------------
+    static_assert(!PLANNED || (BM == kPlanBM && PD == 1), "the plan table is laid out for 128-row blocks");
+    const PlanRec* const pt = p.plan;
+    const int n_rb = p.n_row_blocks;
+    auto seg_plan_of = [&](int sg) {
+        SegPlan t;
+        if constexpr (PLANNED) {
+            const PlanRec r = plan_uniform_load(pt + plan_seg_at(p.n_seg, rb, sg));
+            t.c0 = r.x, t.cs = r.y, t.n_tiles = r.z, t.uniform = r.w;
+        } else {
+            const SegPlan l = s_plan[sg];  // the same for every lane: keep it in scalar registers
+            t.c0 = __builtin_amdgcn_readfirstlane(l.c0);
+            t.cs = __builtin_amdgcn_readfirstlane(l.cs);
+            t.n_tiles = __builtin_amdgcn_readfirstlane(l.n_tiles);
+            t.uniform = __builtin_amdgcn_readfirstlane(l.uniform);
+        }
+        return t;
+    };
+    if constexpr (!PLANNED) plan_segments<BM, BN>(p.seg, p.n_seg, r0, rs, L, !KT, s_plan, &s_ps, tid);
 
     int total_tiles = 0;
-    for (int sg = 0; sg < p.n_seg; ++sg) total_tiles += s_plan[sg].n_tiles;
+    for (int sg = 0; sg < p.n_seg; ++sg) total_tiles += seg_plan_of(sg).n_tiles;
     total_tiles = __builtin_amdgcn_readfirstlane(total_tiles);
 
     // ---- tile walker: asynchronous global -> LDS copies of a tile into a stage -------------------------
@@ -250,30 +268,32 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
 
     int pf_seg = 0, pf_tile = 0;  // position of the next tile to fetch
     SegPlan ppl = {0, 1, 0, 1};
-    auto pf_normalise = [&]() {
-        bool moved = (pf_seg == 0 && pf_tile == 0);
-        while (pf_seg < p.n_seg && pf_tile >= s_plan[pf_seg].n_tiles) {
+    // move on to the first segment at or after pf_seg that has tiles and take its plan into scalar registers
+    auto pf_enter_segment = [&]() {
+        pf_tile = 0;
+        while (pf_seg < p.n_seg) {
+            ppl = seg_plan_of(pf_seg);
+            if (ppl.n_tiles > 0) break;
             ++pf_seg;
-            pf_tile = 0;
-            moved = true;
         }
-        if (moved && pf_seg < p.n_seg) {
-            const SegPlan t = s_plan[pf_seg];  // the same for every lane: keep it in scalar registers
-            ppl.c0 = __builtin_amdgcn_readfirstlane(t.c0);
-            ppl.cs = __builtin_amdgcn_readfirstlane(t.cs);
-            ppl.n_tiles = __builtin_amdgcn_readfirstlane(t.n_tiles);
-            ppl.uniform = __builtin_amdgcn_readfirstlane(t.uniform);
-            set_lane_offsets(ppl);
-        }
+        if (pf_seg < p.n_seg) set_lane_offsets(ppl);
     };
-    // Tiles of a segment are fetched in order, so the running pointers advance by one tile per fetch.
+    // Tiles of a segment are fetched in order, so the running pointers advance by one tile per fetch; LDS is
+    // only consulted at the end of a segment.
     auto advance_fetch = [&]() {
         v_next += BN * v_key;
         k_next += KT ? (int64_t)(BN * ES) : BN * k_key;
-        ++pf_tile;
-        pf_normalise();
+        if (++pf_tile >= ppl.n_tiles) {
+            ++pf_seg;
+            pf_enter_segment();
+        }
     };
-    pf_normalise();
+    pf_enter_segment();
+    // the row windows of the first segment with tiles: requested here, long before the loop needs them
+    PlanRec win_rec = {0, 0, 1, 0};
+    if constexpr (PLANNED) {
+        if (pf_seg < p.n_seg) win_rec = pt[plan_row_at(n_rb, p.n_seg, rb, pf_seg, wave * 32 + lm)];
+    }
 #pragma unroll
     for (int i = 0; i < PD; ++i) {
         if (i < total_tiles) {
@@ -286,7 +306,6 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
             advance_fetch();
         }
     }
-
     f32x16 o_acc[DT];
     float m_ref = kNegBigA, l_run = 0.f;
 #pragma unroll
@@ -332,41 +351,43 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
     const float c2 = p.scale_log2e;
     int stage_it = 0;             // stage that holds tile `it`
     int stage_pf = PD % NSTAGE;   // stage the next fetch goes to
-
     for (int it = 0; it < total_tiles; ++it) {
         // advance the compute position; reload the row map on a segment change
         if (cur_seg < 0 || cur_tile >= cpl.n_tiles) {
             do {
                 ++cur_seg;
-            } while (s_plan[cur_seg].n_tiles == 0);
+                cpl = seg_plan_of(cur_seg);
+            } while (cpl.n_tiles == 0);
             cur_tile = 0;
-            {
-                const SegPlan t = s_plan[cur_seg];
-                cpl.c0 = __builtin_amdgcn_readfirstlane(t.c0);
-                cpl.cs = __builtin_amdgcn_readfirstlane(t.cs);
-                cpl.n_tiles = __builtin_amdgcn_readfirstlane(t.n_tiles);
-                cpl.uniform = __builtin_amdgcn_readfirstlane(t.uniform);
+            WaveSpan sp;
+            if constexpr (PLANNED) {
+                if (it > 0) win_rec = pt[plan_row_at(n_rb, p.n_seg, rb, cur_seg, wave * 32 + lm)];
+                win.lo = win_rec.x, win.cnt = win_rec.y, win.lin = win_rec.z;
+                first = win_rec.w;
+                const PlanRec r = plan_uniform_load(pt + plan_span_at(n_rb, p.n_seg, rb, cur_seg, wave));
+                sp.lo_min = r.x, sp.lo_max = r.y, sp.hi_min = r.z, sp.hi_max = r.w;
+            } else {
+                win = make_row_win(cached_row_map<BM>(&s_ps, cur_seg, wave * 32 + lm), cpl);
+                first = cpl.uniform ? 0 : win_phase(win);
+                sp = wave_span(win, cpl.uniform != 0);
             }
-            win = make_row_win(cached_row_map<BM>(&s_ps, cur_seg, wave * 32 + lm), cpl);
             if (!cpl.uniform) {
                 // periodic part of the row's live positions (position 0 of the walk is column c0)
-                const int lin = win.lin;
-                const int f = win.lo % lin;
-                first = f < 0 ? f + lin : f;
-                dec = BN % lin;
-                uint64_t pt = 0;
-                for (int q = 0; q < 64; q += lin) pt |= 1ull << q;
-                pat = pt;
+                dec = BN % win.lin;
+                uint64_t pt_bits = 0;
+                for (int q = 0; q < 64; q += win.lin) pt_bits |= 1ull << q;
+                pat = pt_bits;
             } else {  // unit step: every position of the span
-                first = 0;
                 pat = ~0ull;
             }
-            const bool empty = win.cnt <= 0;
-            w_lo_min = wave_min_i(empty ? 0x3fffffff : win.lo);
-            w_lo_max = wave_max_i(empty ? -0x3fffffff : win.lo);
-            w_hi_min = wave_min_i(empty ? 0x3fffffff : win.lo + win.cnt);
-            w_hi_max = wave_max_i(empty ? -0x3fffffff : win.lo + win.cnt);
-            if (__any(empty) || !cpl.uniform) w_lo_max = 0x3fffffff;  // such a wave never drops the mask
+            w_lo_min = sp.lo_min, w_lo_max = sp.lo_max, w_hi_min = sp.hi_min, w_hi_max = sp.hi_max;
+            if constexpr (PLANNED) {
+                // keep the spans in vector registers, as the reductions of the other path leave them
+                asm volatile("v_mov_b32 %0, %0" : "+v"(w_lo_min));
+                asm volatile("v_mov_b32 %0, %0" : "+v"(w_lo_max));
+                asm volatile("v_mov_b32 %0, %0" : "+v"(w_hi_min));
+                asm volatile("v_mov_b32 %0, %0" : "+v"(w_hi_max));
+            }
         }
         const int j0 = cur_tile * BN;
         ++cur_tile;
@@ -450,14 +471,12 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
                     for (int s = NMMA / MMA_PER_DMA; s < NDMA; ++s) issue_step(s, stage_pf);
                 }
             }
-
             // ---- mask, online softmax against a lazily updated reference ----
             Frag<T> pf[NT][2];
             if (full)
                 softmax_tile<true, NT, T, DT>(s_acc, pf, m_ref, l_run, o_acc, 0ull, g, c2);
             else
                 softmax_tile<false, NT, T, DT>(s_acc, pf, m_ref, l_run, o_acc, row_live_bits(win, j0, first, pat), g, c2);
-
             // ---- O^T += V^T . P^T ----
             // V fragments are requested one 16-key step (DT fragments) ahead of the MFMAs that consume them.
             auto load_v = [&](int nt, int t, int dt) {
@@ -544,16 +563,17 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
     }
 }
 
-template <typename T, int D, bool KT, int BN, int NSTAGE>
+template <typename T, int D, bool KT, int BN, int NSTAGE, bool PLANNED>
 static int launch_attn(const AttnParams& p0, hipStream_t st) {
     using G = TileGeom<T, D, KT, BN>;
     AttnParams p = p0;
     constexpr int BM = 128;
     p.n_row_blocks = count_row_blocks(p.L, BM, p.row_stride);
     p.total = p.B * p.H * p.n_row_blocks;
+    if (PLANNED && KT) p.plan += plan_variant_recs(p.n_row_blocks, p.n_seg);  // the dense-walk variant
     const int grid = ((p.total + 7) / 8) * 8;
     const size_t lds = NSTAGE * (size_t)G::STAGE;
-    auto kern = attn_fwd_kernel<T, D, KT, BN, NSTAGE>;
+    auto kern = attn_fwd_kernel<T, D, KT, BN, NSTAGE, PLANNED>;
     static thread_local bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -572,28 +592,60 @@ static int launch_attn(const AttnParams& p0, hipStream_t st) {
 // kernel also supports 32-key tiles in a ring of 4 stages; it measured slower at d = 128 and equal at d = 64).
 template <typename T>
 static int dispatch_attn(const AttnParams& p, int d, bool kt, hipStream_t st) {
-    if (d == 64) return kt ? launch_attn<T, 64, true, 64, 2>(p, st) : launch_attn<T, 64, false, 64, 2>(p, st);
-    return kt ? launch_attn<T, 128, true, 64, 2>(p, st) : launch_attn<T, 128, false, 64, 2>(p, st);
+    if (p.plan) {
+        if (d == 64) return kt ? launch_attn<T, 64, true, 64, 2, true>(p, st) : launch_attn<T, 64, false, 64, 2, true>(p, st);
+        return kt ? launch_attn<T, 128, true, 64, 2, true>(p, st) : launch_attn<T, 128, false, 64, 2, true>(p, st);
+    }
+    if (d == 64) return kt ? launch_attn<T, 64, true, 64, 2, false>(p, st) : launch_attn<T, 64, false, 64, 2, false>(p, st);
+    return kt ? launch_attn<T, 128, true, 64, 2, false>(p, st) : launch_attn<T, 128, false, 64, 2, false>(p, st);
+}
+
+// One workgroup per (row block, variant): the same planning code the unplanned kernel runs in its prologue, with
+// the results written to the table.
+struct PlanParams {
+    PlanRec* table;
+    SegPtrs seg[SPLAT_MAX_SEGMENTS];
+    int n_seg, L, rs, n_rb;
+};
+__global__ __launch_bounds__(256) void attn_plan_kernel(const PlanParams p) {
+    constexpr int BM = kPlanBM, BN = 64;
+    __shared__ SegPlan s_plan[SPLAT_MAX_SEGMENTS];
+    __shared__ PlanScratch<BM> s_ps;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lm = lane & 31;
+    const int rb = blockIdx.x, variant = blockIdx.y;
+    const int n_seg = p.n_seg, n_rb = p.n_rb;
+    PlanRec* const pt = p.table + variant * plan_variant_recs(n_rb, n_seg);
+    plan_segments<BM, BN>(p.seg, n_seg, block_first_row(rb, BM, p.rs), p.rs, p.L, variant == 0, s_plan, &s_ps, tid);
+    for (int sg = 0; sg < n_seg; ++sg) {
+        const SegPlan pl = s_plan[sg];
+        const RowWin win = make_row_win(cached_row_map<BM>(&s_ps, sg, wave * 32 + lm), pl);
+        const WaveSpan sp = wave_span(win, pl.uniform != 0);
+        if (tid == 0) pt[plan_seg_at(n_seg, rb, sg)] = PlanRec{pl.c0, pl.cs, pl.n_tiles, pl.uniform};
+        if (lane == 0) pt[plan_span_at(n_rb, n_seg, rb, sg, wave)] = PlanRec{sp.lo_min, sp.lo_max, sp.hi_min, sp.hi_max};
+        if (lane < 32)
+            pt[plan_row_at(n_rb, n_seg, rb, sg, wave * 32 + lm)] = PlanRec{win.lo, win.cnt, win.lin, pl.uniform ? 0 : win_phase(win)};
+    }
 }
 
 }  // namespace splat
 
 using namespace splat;
 
-extern "C" int splat_attention_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT, int64_t k_sb,
-                                   int64_t k_sh, int64_t k_sd, int64_t k_sl, const void* v, int64_t v_sb, int64_t v_sh,
-                                   int64_t v_sl, void* out, int64_t o_sb, int64_t o_sh, int64_t o_sl,
-                                   const splat_acsr_seg* segs, int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t d,
-                                   float scale, int32_t dtype, void* stream) {
-    if (!q || !kT || !v || !out || !segs) return fail(SPLAT_E_NULL, "splat_attention_fwd: null pointer argument");
-    if (B <= 0 || H <= 0 || L <= 0) return fail(SPLAT_E_SHAPE, "splat_attention_fwd: need B, H, L > 0 (got %d, %d, %d)", B, H, L);
-    if (L > (1 << 23)) return fail(SPLAT_E_SHAPE, "splat_attention_fwd: L is limited to 2^23 (got %d)", L);
-    if (d != 64 && d != 128) return fail(SPLAT_E_UNSUPPORTED, "splat_attention_fwd: head dim must be 64 or 128 (got %d)", d);
+static int attention_fwd_common(const char* who, const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT,
+                                int64_t k_sb, int64_t k_sh, int64_t k_sd, int64_t k_sl, const void* v, int64_t v_sb,
+                                int64_t v_sh, int64_t v_sl, void* out, int64_t o_sb, int64_t o_sh, int64_t o_sl,
+                                const splat_acsr_seg* segs, int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t d,
+                                float scale, int32_t dtype, const void* plan, int64_t plan_bytes, bool planned,
+                                void* stream) {
+    if (!q || !kT || !v || !out || !segs) return fail(SPLAT_E_NULL, "%s: null pointer argument", who);
+    if (B <= 0 || H <= 0 || L <= 0) return fail(SPLAT_E_SHAPE, "%s: need B, H, L > 0 (got %d, %d, %d)", who, B, H, L);
+    if (L > (1 << 23)) return fail(SPLAT_E_SHAPE, "%s: L is limited to 2^23 (got %d)", who, L);
+    if (d != 64 && d != 128) return fail(SPLAT_E_UNSUPPORTED, "%s: head dim must be 64 or 128 (got %d)", who, d);
     if (dtype != SPLAT_F32 && dtype != SPLAT_F16 && dtype != SPLAT_BF16)
-        return fail(SPLAT_E_DTYPE, "splat_attention_fwd: unknown dtype %d", dtype);
+        return fail(SPLAT_E_DTYPE, "%s: unknown dtype %d", who, dtype);
     // the running max is taken over unscaled scores (needs scale >= 0) and masked scores are zeroed through
     // the underflow of exp2(-1e30 * scale) (needs scale > 0)
-    if (!(scale > 0.f)) return fail(SPLAT_E_UNSUPPORTED, "splat_attention_fwd: scale must be > 0 (got %g)", (double)scale);
+    if (!(scale > 0.f)) return fail(SPLAT_E_UNSUPPORTED, "%s: scale must be > 0 (got %g)", who, (double)scale);
     const int es = dtype == SPLAT_F32 ? 4 : 2;
     const int epc = 16 / es;
     bool kt;
@@ -602,17 +654,17 @@ extern "C" int splat_attention_fwd(const void* q, int64_t q_sb, int64_t q_sh, in
     else if (k_sl == 1)
         kt = true;  // K^T contiguous: [.., d, L] memory
     else
-        return fail(SPLAT_E_ALIGN, "splat_attention_fwd: kT needs unit stride along d (k_sd == 1) or along keys (k_sl == 1); got k_sd=%lld k_sl=%lld",
+        return fail(SPLAT_E_ALIGN, "%s: kT needs unit stride along d (k_sd == 1) or along keys (k_sl == 1); got k_sd=%lld k_sl=%lld", who,
                     (long long)k_sd, (long long)k_sl);
     if (kt && ((L % epc) != 0 || (k_sd % epc) != 0 || L < epc))
-        return fail(SPLAT_E_ALIGN, "splat_attention_fwd: with K^T contiguous along keys, L and the d-stride must be multiples of %d (got L=%d, k_sd=%lld)",
+        return fail(SPLAT_E_ALIGN, "%s: with K^T contiguous along keys, L and the d-stride must be multiples of %d (got L=%d, k_sd=%lld)", who,
                     epc, L, (long long)k_sd);
     auto mis = [&](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) != 0; };
     auto bad = [&](int64_t s) { return (s % epc) != 0; };
-    if (mis(q) || mis(kT) || mis(v) || mis(out)) return fail(SPLAT_E_ALIGN, "splat_attention_fwd: q, kT, v and out must be 16-byte aligned");
+    if (mis(q) || mis(kT) || mis(v) || mis(out)) return fail(SPLAT_E_ALIGN, "%s: q, kT, v and out must be 16-byte aligned", who);
     if (bad(q_sb) || bad(q_sh) || bad(q_sl) || bad(k_sb) || bad(k_sh) || bad(v_sb) || bad(v_sh) || bad(v_sl) || bad(o_sb) || bad(o_sh) || bad(o_sl))
-        return fail(SPLAT_E_ALIGN, "splat_attention_fwd: every batch/head/row stride must be a multiple of %d elements (16 bytes)", epc);
-    if (q_sl < d || v_sl < d || o_sl < d) return fail(SPLAT_E_SHAPE, "splat_attention_fwd: row strides must be >= d");
+        return fail(SPLAT_E_ALIGN, "%s: every batch/head/row stride must be a multiple of %d elements (16 bytes)", who, epc);
+    if (q_sl < d || v_sl < d || o_sl < d) return fail(SPLAT_E_SHAPE, "%s: row strides must be >= d", who);
 
     AttnParams p;
     p.q = q; p.k = kT; p.v = v; p.o = out;
@@ -623,12 +675,67 @@ extern "C" int splat_attention_fwd(const void* q, int64_t q_sb, int64_t q_sh, in
     p.B = B; p.H = H; p.L = L;
     p.scale_log2e = scale * 1.4426950408889634f;
     p.n_seg = n_seg;
-    if (int rc = fill_segs("splat_attention_fwd", segs, n_seg, p.seg, -1)) return rc;
+    if (int rc = fill_segs(who, segs, n_seg, p.seg, -1)) return rc;
     p.row_stride = common_row_stride(segs, n_seg);
+    p.plan = nullptr;
+    if (planned) {
+        if (!plan) return fail(SPLAT_E_NULL, "%s: null plan", who);
+        if ((reinterpret_cast<uintptr_t>(plan) & 15) != 0) return fail(SPLAT_E_ALIGN, "%s: the plan must be 16-byte aligned", who);
+        const int64_t need = splat_attention_plan_bytes(segs, n_seg, L);
+        if (plan_bytes < need)
+            return fail(SPLAT_E_SHAPE, "%s: the plan holds %lld bytes, this mask needs %lld", who, (long long)plan_bytes, (long long)need);
+        p.plan = static_cast<const PlanRec*>(plan);
+    }
     hipStream_t st = (hipStream_t)stream;
     switch (dtype) {
         case SPLAT_F32: return dispatch_attn<float>(p, d, kt, st);
         case SPLAT_F16: return dispatch_attn<f16>(p, d, kt, st);
         default: return dispatch_attn<bf16>(p, d, kt, st);
     }
+}
+
+extern "C" int splat_attention_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT, int64_t k_sb,
+                                   int64_t k_sh, int64_t k_sd, int64_t k_sl, const void* v, int64_t v_sb, int64_t v_sh,
+                                   int64_t v_sl, void* out, int64_t o_sb, int64_t o_sh, int64_t o_sl,
+                                   const splat_acsr_seg* segs, int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t d,
+                                   float scale, int32_t dtype, void* stream) {
+    return attention_fwd_common("splat_attention_fwd", q, q_sb, q_sh, q_sl, kT, k_sb, k_sh, k_sd, k_sl, v, v_sb, v_sh, v_sl, out,
+                                o_sb, o_sh, o_sl, segs, n_seg, B, H, L, d, scale, dtype, nullptr, 0, false, stream);
+}
+
+extern "C" int splat_attention_fwd_planned(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT,
+                                           int64_t k_sb, int64_t k_sh, int64_t k_sd, int64_t k_sl, const void* v,
+                                           int64_t v_sb, int64_t v_sh, int64_t v_sl, void* out, int64_t o_sb, int64_t o_sh,
+                                           int64_t o_sl, const splat_acsr_seg* segs, int32_t n_seg, int32_t B, int32_t H,
+                                           int32_t L, int32_t d, float scale, int32_t dtype, const void* plan,
+                                           int64_t plan_bytes, void* stream) {
+    return attention_fwd_common("splat_attention_fwd_planned", q, q_sb, q_sh, q_sl, kT, k_sb, k_sh, k_sd, k_sl, v, v_sb, v_sh,
+                                v_sl, out, o_sb, o_sh, o_sl, segs, n_seg, B, H, L, d, scale, dtype, plan, plan_bytes, true,
+                                stream);
+}
+
+extern "C" int64_t splat_attention_plan_bytes(const splat_acsr_seg* segs, int32_t n_seg, int32_t L) {
+    if (!segs || n_seg < 1 || n_seg > SPLAT_MAX_SEGMENTS || L <= 0) return 0;
+    const int n_rb = count_row_blocks(L, kPlanBM, common_row_stride(segs, n_seg));
+    return 2 * plan_variant_recs(n_rb, n_seg) * (int64_t)sizeof(PlanRec);
+}
+
+extern "C" int splat_attention_plan(const splat_acsr_seg* segs, int32_t n_seg, int32_t L, void* plan, int64_t plan_bytes,
+                                    void* stream) {
+    const char* who = "splat_attention_plan";
+    if (!segs || !plan) return fail(SPLAT_E_NULL, "%s: null pointer argument", who);
+    if (L <= 0 || L > (1 << 23)) return fail(SPLAT_E_SHAPE, "%s: need 0 < L <= 2^23 (got %d)", who, L);
+    if ((reinterpret_cast<uintptr_t>(plan) & 15) != 0) return fail(SPLAT_E_ALIGN, "%s: the plan must be 16-byte aligned", who);
+    PlanParams p;
+    if (int rc = fill_segs(who, segs, n_seg, p.seg, -1)) return rc;
+    const int64_t need = splat_attention_plan_bytes(segs, n_seg, L);
+    if (plan_bytes < need)
+        return fail(SPLAT_E_SHAPE, "%s: the plan needs %lld bytes for this mask, got %lld", who, (long long)need, (long long)plan_bytes);
+    p.table = static_cast<PlanRec*>(plan);
+    p.n_seg = n_seg;
+    p.L = L;
+    p.rs = common_row_stride(segs, n_seg);
+    p.n_rb = count_row_blocks(L, kPlanBM, p.rs);
+    attn_plan_kernel<<<dim3(p.n_rb, 2), 256, 0, (hipStream_t)stream>>>(p);
+    return check_launch(who);
 }
