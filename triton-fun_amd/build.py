@@ -15,7 +15,7 @@ LIB = os.path.join(LIB_DIR, "libsplat_hip.so")
 
 SOURCES = ["api_common.cpp", "acsr_build.hip", "softmax.hip", "sddmm.hip", "spmm.hip", "attention.hip"]
 # packed fp32 VALU forms are switched off for every device compile
-FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
+FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function", "-Wno-inline-asm",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
@@ -48,6 +48,11 @@ def build(jobs: int = 8, verbose: bool = True) -> str:
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stderr}")
+    # a kernel stub the host pass failed to emit only shows up when the library is loaded: check here
+    undefined = subprocess.run(["nm", "-D", "--undefined-only", LIB], capture_output=True, text=True).stdout
+    missing = [l.split()[-1] for l in undefined.splitlines() if "splat" in l]
+    if missing:
+        raise RuntimeError(f"{LIB} has undefined symbols of its own: {missing[:4]}")
     if verbose:
         print(f"built {LIB}")
     return LIB

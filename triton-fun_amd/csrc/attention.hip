@@ -261,9 +261,9 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
         char* ks_w = smem + stage * G::STAGE;
         char* vs_w = ks_w + G::K_BYTES;
         if (i < V_NI)
-            dma16(v_next + (int64_t)(4 * V_RPI * i) * v_key + v_lane_off, vs_w + (wave + 4 * i) * 1024);
+            dma16_uniform(v_next + (int64_t)(4 * V_RPI * i) * v_key, v_lane_off, vs_w + (wave + 4 * i) * 1024);
         else
-            dma16(k_next + (int64_t)(4 * K_RPI * (i - V_NI)) * k_key + k_lane_off, ks_w + (wave + 4 * (i - V_NI)) * 1024);
+            dma16_uniform(k_next + (int64_t)(4 * K_RPI * (i - V_NI)) * k_key, k_lane_off, ks_w + (wave + 4 * (i - V_NI)) * 1024);
     };
 
     int pf_seg = 0, pf_tile = 0;  // position of the next tile to fetch
@@ -351,6 +351,14 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
     const float c2 = p.scale_log2e;
     int stage_it = 0;             // stage that holds tile `it`
     int stage_pf = PD % NSTAGE;   // stage the next fetch goes to
+    // The Q fragments have to be in their registers before the loop: otherwise the compiler puts its waits for them
+    // in front of the first score MFMAs of every tile, counted against the loads it knows of, and those waits would
+    // then hold for the copies of the next tile that are in flight at that point.
+#if defined(__HIP_DEVICE_COMPILE__)  // the register constraint means something else to the host pass
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(qf[ks].v));
+#endif
+
     for (int it = 0; it < total_tiles; ++it) {
         // advance the compute position; reload the row map on a segment change
         if (cur_seg < 0 || cur_tile >= cpl.n_tiles) {
@@ -418,46 +426,52 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
             const bool full = (j0 >= w_lo_max) && (j0 + BN <= w_hi_min);
 
             // ---- S^T = K . Q^T ----
-            // All K fragments of the tile are requested from LDS before the first MFMA that needs them.
+            // K fragments are requested from LDS a few MFMAs ahead of their use, never more than 12 read
+            // instructions at a time: the counter that tracks them holds 15, and the compiler falls back to
+            // waiting for every outstanding read once it could overflow.
             f32x16 s_acc[NT];
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                 for (int j = 0; j < 16; ++j) s_acc[nt][j] = 0.f;
             Frag<T> kfr[NT][KS];
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    Frag<T>& kf = kfr[nt][ks];
-                    if constexpr (ES == 2) {
-                        if constexpr (KT) {
-                            // rows 16ks + 8g + {0..3} and +4: multiples of 4 rows leave the lane's swizzle term alone
-                            const uint32_t a0 = k_addr[nt] + 16 * ks * G::K_ROWB;
-                            kf = frag_from_tr<T>(lds_load_tr16(a0), lds_load_tr16(a0 + 4 * G::K_ROWB));
-                        } else {
-                            kf.v = __builtin_bit_cast(typename Frag<T>::vec, lds_load128(k_addr[ks] + 32 * nt * G::K_ROWB));
-                        }
+            auto load_k = [&](int nt, int ks) {
+                Frag<T> kf;
+                if constexpr (ES == 2) {
+                    if constexpr (KT) {
+                        // rows 16ks + 8g + {0..3} and +4: multiples of 4 rows leave the lane's swizzle term alone
+                        const uint32_t a0 = k_addr[nt] + 16 * ks * G::K_ROWB;
+                        kf = frag_from_tr<T>(lds_load_tr16(a0), lds_load_tr16(a0 + 4 * G::K_ROWB));
                     } else {
-                        const char* ks_l = smem + stage_it * G::STAGE;
-                        if constexpr (KT) {
+                        kf.v = __builtin_bit_cast(typename Frag<T>::vec, lds_load128(k_addr[ks] + 32 * nt * G::K_ROWB));
+                    }
+                } else {
+                    const char* ks_l = smem + stage_it * G::STAGE;
+                    if constexpr (KT) {
 #pragma unroll
-                            for (int e = 0; e < 8; ++e)
-                                kf.v[e] = *reinterpret_cast<const float*>(ks_l + (16 * ks + 8 * g + e) * G::K_ROWB + (32 * nt + lm) * 4);
-                        } else {
-                            kf = lds_frag_row_swz<T, G::K_ROWB>(ks_l, 32 * nt + lm, 16 * ks + 8 * g);
-                        }
+                        for (int e = 0; e < 8; ++e)
+                            kf.v[e] = *reinterpret_cast<const float*>(ks_l + (16 * ks + 8 * g + e) * G::K_ROWB + (32 * nt + lm) * 4);
+                    } else {
+                        kf = lds_frag_row_swz<T, G::K_ROWB>(ks_l, 32 * nt + lm, 16 * ks + 8 * g);
                     }
                 }
-            }
+                return kf;
+            };
+            constexpr int NMMA = NT * KS;
+            constexpr int K_AHEAD = (ES != 2) ? NMMA : ((KT ? 6 : 12) < NMMA ? (KT ? 6 : 12) : NMMA);  // fragments
+#pragma unroll
+            for (int i = 0; i < K_AHEAD; ++i) kfr[i / KS][i % KS] = load_k(i / KS, i % KS);
             __builtin_amdgcn_sched_barrier(0);  // keep the requests above the matrix work
             // the copy instructions of the fetch go between the MFMAs, so that the address path sees them at
             // the rate it can take instead of as one burst that stalls the wavefront
-            constexpr int NMMA = NT * KS;
             constexpr int MMA_PER_DMA = (NMMA / NDMA) > 0 ? NMMA / NDMA : 1;
 #pragma unroll
             for (int i = 0; i < NMMA; ++i) {
                 mma32(s_acc[i / KS], kfr[i / KS][i % KS], qf[i % KS]);
+                if (i + K_AHEAD < NMMA) {
+                    kfr[(i + K_AHEAD) / KS][(i + K_AHEAD) % KS] = load_k((i + K_AHEAD) / KS, (i + K_AHEAD) % KS);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
                 if constexpr (FAST_DMA) {
                     if ((i + 1) % MMA_PER_DMA == 0 && (i + 1) / MMA_PER_DMA <= NDMA) {
                         if (spread) issue_step((i + 1) / MMA_PER_DMA - 1, stage_pf);
@@ -497,16 +511,18 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
             Frag<T> vfr[2][DT];
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) vfr[0][dt] = load_v(0, 0, dt);
+            __builtin_amdgcn_sched_barrier(0);  // keep the requests above the matrix work
 #pragma unroll
             for (int step = 0; step < 2 * NT; ++step) {
                 const int nt = step >> 1, t = step & 1;
-                if (step + 1 < 2 * NT) {
 #pragma unroll
-                    for (int dt = 0; dt < DT; ++dt) vfr[(step + 1) & 1][dt] = load_v((step + 1) >> 1, (step + 1) & 1, dt);
+                for (int dt = 0; dt < DT; ++dt) {
+                    mma32(o_acc[dt], vfr[step & 1][dt], pf[nt][t]);
+                    if (step + 1 < 2 * NT) {
+                        vfr[(step + 1) & 1][dt] = load_v((step + 1) >> 1, (step + 1) & 1, dt);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
-                __builtin_amdgcn_sched_barrier(0);  // keep the requests above the matrix work
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) mma32(o_acc[dt], vfr[step & 1][dt], pf[nt][t]);
             }
         } else if (spread) {
 #pragma unroll

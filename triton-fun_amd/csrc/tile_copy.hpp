@@ -54,8 +54,29 @@ typedef __attribute__((address_space(3))) void lptr_t;
 
 // One wavefront-wide 1 KiB copy global -> LDS without passing through registers: lane i's 16 bytes land at
 // lds_block + 16*i (lds_block must be wavefront-uniform).
+//
+// The copies are written as inline asm on purpose.  The compiler orders every LDS read behind every copy instruction it
+// knows of (it cannot tell which LDS bytes a copy writes) and, while one is outstanding, turns all its counted waits
+// into waits for everything; that would stall each tile on the copies of the next one.  Copies it does not see are
+// ordered by the kernels themselves: wait_loads<N>() for this wavefront's copies, then a barrier, before any wavefront
+// reads the stage.  The waits the compiler emits for loads it does know stay safe: loads complete in order, so extra
+// copies in flight only make such a wait cover more than it needs to.
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+// per-lane 64-bit source address
 __device__ __forceinline__ void dma16(const void* src, char* lds_block) {
-    __builtin_amdgcn_global_load_lds((gptr_t*)src, (lptr_t*)lds_block, 16, 0, 0);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(lds_address(lds_block)), "v"(src)
+                 : "memory", "m0");
+}
+// wavefront-uniform 64-bit base + per-lane 32-bit byte offset
+__device__ __forceinline__ void dma16_uniform(const void* base, uint32_t lane_off, char* lds_block) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_address(lds_block)), "v"(lane_off), "s"(base)
+                 : "memory", "m0");
 }
 __device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
