@@ -163,3 +163,20 @@ def test_spmm_patterns(dev, dtype, make, n_out):
     r_spmm.rspmm_launcher(p.to(dev), v.to(dev), out, acsr[0], acsr[1], acsr[2], acsr[3], acsr[6], acsr[7], T, acsr[4],
                           (1, 1, 1), 16, 16)
     assert float((out.float().cpu() - want).abs().max()) <= TOL[dtype]
+
+
+def test_comparison_sweeps_run_and_agree_with_dense(dev):
+    """The sweep harness (successor of the reference's comparison.py:76-106) at toy size: one record per doubling of
+    the sparsity parameter, nnz as the pattern's closed form, fused forward equal to dense attention with the same mask."""
+    import comparison
+    rows = comparison.benchmark("Windowed", 64, 16, 16, dev, verbose=False)
+    assert [r["sparsity_parameter"] for r in rows] == [2, 4, 8, 16, 32, 64]
+    for r in rows:
+        p = r["sparsity_parameter"]
+        assert r["nnz"] == sum(min(63, i + p) - max(0, i - p) + 1 for i in range(64))
+        assert r["splat_ms"] > 0 and r["dense_ms"] > 0
+    att = comparison.benchmark_attention("Blocked", 128, dev, batch=1, num_heads=2, head_dim=64, dtype=torch.float16,
+                                         verbose=False)
+    assert len(att) == 7 and max(r["max_abs_diff"] for r in att) <= 1e-2
+    with pytest.raises(Exception, match="Not implemented!"):
+        comparison.benchmark("Strided", 64, 16, 16, dev, verbose=False)
