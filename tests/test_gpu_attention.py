@@ -266,3 +266,23 @@ def test_plan_arguments_are_checked(dev):
         attention_launcher(q, q.transpose(2, 3), q, torch.empty_like(q), attn.segments, 1.0, plan[:-16])
     with pytest.raises(hip.SplatError):
         attention_launcher(q, q.transpose(2, 3), q, torch.empty_like(q), attn.segments, 1.0, plan.cpu())
+
+
+@pytest.mark.parametrize("dtype,slope", [(torch.bfloat16, 0.5), (torch.float16, 0.125), (torch.float32, 0.5)])
+def test_scores_that_outrun_the_first_tiles_reference(dev, dtype, slope):
+    """Scores that grow along the keys: a row's later tiles exceed the maximum of its first tile by far more than the
+    exponent range of the probabilities (e^96 for slope 0.5 over 192 keys; e^24 against fp16's 65504), so the kernel
+    cannot keep the references its rows settled on and has to repeat the row block with moving references.  The same
+    inputs with a short window never leave the fast path; both must match the oracle."""
+    L, d = 512, 128
+    q = torch.ones(1, 2, L, d)
+    k = (slope * torch.arange(L, dtype=torch.float32) / d).view(1, 1, L, 1).expand(1, 2, L, d).contiguous()
+    g = torch.Generator().manual_seed(11)
+    v = torch.randn(1, 2, L, d, generator=g)
+    q, k, v = [t.to(dtype) for t in (q, k, v)]
+    for w in (255, 15):
+        mask = O.create_causal_windowed_mask(L, w)
+        want = O.dense_masked_attention(q, k.transpose(2, 3), v, mask, 1.0)
+        got = run_module(mask, 1, 2, L, d, dtype, dev, q, k, v, 1.0, True)
+        assert torch.isfinite(got).all(), w
+        assert float((got - want).abs().max()) <= TOL[dtype], w

@@ -65,24 +65,43 @@ __device__ __forceinline__ float keep_or_mask(float x, int keep) {
     return __builtin_bit_cast(float, (xb & (uint32_t)keep) | (nb & ~(uint32_t)keep));
 }
 
-// Mask (unless FULL), fold one tile of 32*NT keys of scores of one 32-row tile into the running softmax state and
-// emit the exponentials as MFMA B fragments.  One lane owns one query row (half of its positions: accumulator
-// register j of 32-key half nt holds position 32*nt + 8*(j/4) + 4*g + j%4, whose bit of `live` says whether it is
-// kept; see row_live_bits).
-template <bool FULL, int NT, typename T, int DT>
-__device__ __forceinline__ void softmax_tile(f32x16 (&s)[NT], Frag<T> (&pf)[NT][2], float& m_ref, float& l_run,
-                                             f32x16 (&o)[DT], uint64_t live, int g, float c2) {
-    if constexpr (!FULL) {
+// Accumulator register j of 32-key half nt of a lane holds position 32*nt + 8*(j/4) + 4*g + j%4 of the tile; its bit
+// of `live` (see row_live_bits) says whether the score is kept.
+template <int NT>
+__device__ __forceinline__ void mask_tile(f32x16 (&s)[NT], uint64_t live, int g) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            const uint32_t bits = (uint32_t)(live >> (32 * nt)) >> (4 * g);
+    for (int nt = 0; nt < NT; ++nt) {
+        const uint32_t bits = (uint32_t)(live >> (32 * nt)) >> (4 * g);
 #pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                const int c = 8 * (j >> 2) + (j & 3);
-                s[nt][j] = keep_or_mask(s[nt][j], ((int)(bits << (31 - c))) >> 31);
-            }
+        for (int j = 0; j < 16; ++j) {
+            const int c = 8 * (j >> 2) + (j & 3);
+            s[nt][j] = keep_or_mask(s[nt][j], ((int)(bits << (31 - c))) >> 31);
         }
     }
+}
+
+// Exponentials of one tile of scores against the rows' references (mb = reference * c2), as MFMA B fragments; returns
+// the lane's sum.
+template <int NT, typename T>
+__device__ __forceinline__ float exp_tile(const f32x16 (&s)[NT], Frag<T> (&pf)[NT][2], float mb, float c2) {
+    float rs = 0.f;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const float pv = fast_exp2(fmaf(s[nt][j], c2, -mb));
+            rs += pv;
+            pf[nt][j >> 3].v[j & 7] = (T)pv;
+        }
+    return rs;
+}
+
+// Fold one tile of 32*NT keys of (masked) scores of one 32-row tile into the running softmax state and emit the
+// exponentials.  One lane owns one query row (half of its positions).  Returns whether every row of the wavefront
+// has a real reference afterwards.
+template <int NT, typename T, int DT>
+__device__ __forceinline__ bool softmax_tile(f32x16 (&s)[NT], Frag<T> (&pf)[NT][2], float& m_ref, float& l_run,
+                                             f32x16 (&o)[DT], float c2) {
     float mx = s[0][0];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
@@ -107,17 +126,9 @@ __device__ __forceinline__ void softmax_tile(f32x16 (&s)[NT], Frag<T> (&pf)[NT][
     // Masked scores are -1e30: their exponential underflows to exactly 0 as long as the reference is a real
     // score.  A row that has seen no live score yet keeps the -1e30 reference; give it offset 0 so that its
     // (all masked) entries still map to 0 instead of exp2(0).
-    const float mb = (FULL || m_ref > 0.5f * kNegBigA) ? m_ref * c2 : 0.f;
-    float rs = 0.f;
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            const float pv = fast_exp2(fmaf(s[nt][j], c2, -mb));
-            rs += pv;
-            pf[nt][j >> 3].v[j & 7] = (T)pv;
-        }
-    l_run += rs;
+    const bool real = m_ref > 0.5f * kNegBigA;
+    l_run += exp_tile<NT, T>(s, pf, real ? m_ref * c2 : 0.f, c2);
+    return !__any(!real);
 }
 
 template <typename T, int D, bool KT, int BN, int NSTAGE, bool PLANNED>
@@ -288,30 +299,8 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
             pf_enter_segment();
         }
     };
-    pf_enter_segment();
-    // the row windows of the first segment with tiles: requested here, long before the loop needs them
-    PlanRec win_rec = {0, 0, 1, 0};
-    if constexpr (PLANNED) {
-        if (pf_seg < p.n_seg) win_rec = pt[plan_row_at(n_rb, p.n_seg, rb, pf_seg, wave * 32 + lm)];
-    }
-#pragma unroll
-    for (int i = 0; i < PD; ++i) {
-        if (i < total_tiles) {
-            if (tile_is_fast(ppl, pf_tile)) {
-#pragma unroll
-                for (int s = 0; s < NDMA; ++s) issue_step(s, i);
-            } else {
-                issue_tile_general(ppl, pf_tile, i);
-            }
-            advance_fetch();
-        }
-    }
     f32x16 o_acc[DT];
     float m_ref = kNegBigA, l_run = 0.f;
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) o_acc[dt][j] = 0.f;
 
     // ---- LDS read addresses: lane-dependent part + current stage; tile constants go into the instruction's
     // immediate offset; the stage offset is added once per tile -------------------------------------------
@@ -341,213 +330,258 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
         for (int i = 0; i < (KT ? NT : KS); ++i) k_addr[i] = smem_base;
     }
 
-    // per-lane row map of the segment being computed
-    int cur_seg = -1, cur_tile = 0;
-    RowWin win = {0, 0, 1};
-    int first = 0, dec = 0;  // periodic part of the row mask of dense plans: see row_live_bits
-    uint64_t pat = ~0ull;
-    int w_lo_min = 0, w_lo_max = 0, w_hi_min = 0, w_hi_max = 0;
-    SegPlan cpl = {0, 1, 0, 1};
-    const float c2 = p.scale_log2e;
-    int stage_it = 0;             // stage that holds tile `it`
-    int stage_pf = PD % NSTAGE;   // stage the next fetch goes to
-    // The Q fragments have to be in their registers before the loop: otherwise the compiler puts its waits for them
-    // in front of the first score MFMAs of every tile, counted against the loads it knows of, and those waits would
-    // then hold for the copies of the next tile that are in flight at that point.
+    // Two ways to take a tile's exponentials.  The careful one tracks the row maxima and moves the reference (with a
+    // rescale of O and l) when they outrun it.  Once every row of the wavefront has a reference, the fast one leaves the
+    // references where they are: no maxima, no exchange between the half rows, no data-dependent branch between the
+    // score MFMAs and the exponentials.  That is exact as long as nothing overflows (float range for 32-bit and bf16
+    // probabilities, 65504 for fp16 ones); if a later score outruns a row's reference by more than that, the row's sum
+    // or output turns infinite or NaN and stays so, which is checked after the last tile, and the workgroup then
+    // repeats its tiles on the careful path alone.
+    bool careful_only = false;
+    for (;;) {
+        pf_seg = 0;
+        pf_enter_segment();
+        // the row windows of the first segment with tiles: requested here, long before the loop needs them
+        PlanRec win_rec = {0, 0, 1, 0};
+        if constexpr (PLANNED) {
+            if (pf_seg < p.n_seg) win_rec = pt[plan_row_at(n_rb, p.n_seg, rb, pf_seg, wave * 32 + lm)];
+        }
+#pragma unroll
+        for (int i = 0; i < PD; ++i) {
+            if (i < total_tiles) {
+                if (tile_is_fast(ppl, pf_tile)) {
+#pragma unroll
+                    for (int s = 0; s < NDMA; ++s) issue_step(s, i);
+                } else {
+                    issue_tile_general(ppl, pf_tile, i);
+                }
+                advance_fetch();
+            }
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) o_acc[dt][j] = 0.f;
+        m_ref = kNegBigA;
+        l_run = 0.f;
+
+        // per-lane row map of the segment being computed
+        int cur_seg = -1, cur_tile = 0;
+        RowWin win = {0, 0, 1};
+        int first = 0, dec = 0;  // periodic part of the row mask of dense plans: see row_live_bits
+        uint64_t pat = ~0ull;
+        int w_lo_min = 0, w_lo_max = 0, w_hi_min = 0, w_hi_max = 0;
+        SegPlan cpl = {0, 1, 0, 1};
+        const float c2 = p.scale_log2e;
+        bool settled = false;         // every row of this wavefront has a reference
+        int stage_it = 0;             // stage that holds tile `it`
+        int stage_pf = PD % NSTAGE;   // stage the next fetch goes to
+        // The Q fragments have to be in their registers before the loop: otherwise the compiler puts its waits for them
+        // in front of the first score MFMAs of every tile, counted against the loads it knows of, and those waits would
+        // then hold for the copies of the next tile that are in flight at that point.
 #if defined(__HIP_DEVICE_COMPILE__)  // the register constraint means something else to the host pass
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(qf[ks].v));
+        for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(qf[ks].v));
 #endif
 
-    for (int it = 0; it < total_tiles; ++it) {
-        // advance the compute position; reload the row map on a segment change
-        if (cur_seg < 0 || cur_tile >= cpl.n_tiles) {
-            do {
-                ++cur_seg;
-                cpl = seg_plan_of(cur_seg);
-            } while (cpl.n_tiles == 0);
-            cur_tile = 0;
-            WaveSpan sp;
-            if constexpr (PLANNED) {
-                if (it > 0) win_rec = pt[plan_row_at(n_rb, p.n_seg, rb, cur_seg, wave * 32 + lm)];
-                win.lo = win_rec.x, win.cnt = win_rec.y, win.lin = win_rec.z;
-                first = win_rec.w;
-                const PlanRec r = plan_uniform_load(pt + plan_span_at(n_rb, p.n_seg, rb, cur_seg, wave));
-                sp.lo_min = r.x, sp.lo_max = r.y, sp.hi_min = r.z, sp.hi_max = r.w;
-            } else {
-                win = make_row_win(cached_row_map<BM>(&s_ps, cur_seg, wave * 32 + lm), cpl);
-                first = cpl.uniform ? 0 : win_phase(win);
-                sp = wave_span(win, cpl.uniform != 0);
-            }
-            if (!cpl.uniform) {
-                // periodic part of the row's live positions (position 0 of the walk is column c0)
-                dec = BN % win.lin;
-                uint64_t pt_bits = 0;
-                for (int q = 0; q < 64; q += win.lin) pt_bits |= 1ull << q;
-                pat = pt_bits;
-            } else {  // unit step: every position of the span
-                pat = ~0ull;
-            }
-            w_lo_min = sp.lo_min, w_lo_max = sp.lo_max, w_hi_min = sp.hi_min, w_hi_max = sp.hi_max;
-            if constexpr (PLANNED) {
-                // keep the spans in vector registers, as the reductions of the other path leave them
-                asm volatile("v_mov_b32 %0, %0" : "+v"(w_lo_min));
-                asm volatile("v_mov_b32 %0, %0" : "+v"(w_lo_max));
-                asm volatile("v_mov_b32 %0, %0" : "+v"(w_hi_min));
-                asm volatile("v_mov_b32 %0, %0" : "+v"(w_hi_max));
-            }
-        }
-        const int j0 = cur_tile * BN;
-        ++cur_tile;
-
-        // This wavefront's part of tile `it` has landed once at most the copies of the later tiles in flight
-        // are outstanding; after the barrier every part has, and every wavefront is done with tile it - 1,
-        // whose stage the next fetch overwrites.
-        {
-            const int later = total_tiles - 1 - it;
-            if (PD == 1 || later == 0)
-                wait_loads<0>();
-            else if (later == 1)
-                wait_loads<NDMA>();
-            else
-                wait_loads<NDMA*(PD > 1 ? PD - 1 : 1)>();
-        }
-        __builtin_amdgcn_s_barrier();
-
-        const bool fetch = (it + PD < total_tiles);
-        bool spread = false;  // the fetch is issued piecewise between the matrix instructions below
-        if (fetch) {
-            spread = tile_is_fast(ppl, pf_tile);
-            if (!spread) issue_tile_general(ppl, pf_tile, stage_pf);
-        }
-
-        const bool skip = (j0 + BN <= w_lo_min) || (j0 >= w_hi_max);
-        if (!skip) {
-            const bool full = (j0 >= w_lo_max) && (j0 + BN <= w_hi_min);
-
-            // ---- S^T = K . Q^T ----
-            // K fragments are requested from LDS a few MFMAs ahead of their use, never more than 12 read
-            // instructions at a time: the counter that tracks them holds 15, and the compiler falls back to
-            // waiting for every outstanding read once it could overflow.
-            f32x16 s_acc[NT];
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                for (int j = 0; j < 16; ++j) s_acc[nt][j] = 0.f;
-            Frag<T> kfr[NT][KS];
-            auto load_k = [&](int nt, int ks) {
-                Frag<T> kf;
-                if constexpr (ES == 2) {
-                    if constexpr (KT) {
-                        // rows 16ks + 8g + {0..3} and +4: multiples of 4 rows leave the lane's swizzle term alone
-                        const uint32_t a0 = k_addr[nt] + 16 * ks * G::K_ROWB;
-                        kf = frag_from_tr<T>(lds_load_tr16(a0), lds_load_tr16(a0 + 4 * G::K_ROWB));
-                    } else {
-                        kf.v = __builtin_bit_cast(typename Frag<T>::vec, lds_load128(k_addr[ks] + 32 * nt * G::K_ROWB));
-                    }
+        for (int it = 0; it < total_tiles; ++it) {
+            // advance the compute position; reload the row map on a segment change
+            if (cur_seg < 0 || cur_tile >= cpl.n_tiles) {
+                do {
+                    ++cur_seg;
+                    cpl = seg_plan_of(cur_seg);
+                } while (cpl.n_tiles == 0);
+                cur_tile = 0;
+                WaveSpan sp;
+                if constexpr (PLANNED) {
+                    if (it > 0) win_rec = pt[plan_row_at(n_rb, p.n_seg, rb, cur_seg, wave * 32 + lm)];
+                    win.lo = win_rec.x, win.cnt = win_rec.y, win.lin = win_rec.z;
+                    first = win_rec.w;
+                    const PlanRec r = plan_uniform_load(pt + plan_span_at(n_rb, p.n_seg, rb, cur_seg, wave));
+                    sp.lo_min = r.x, sp.lo_max = r.y, sp.hi_min = r.z, sp.hi_max = r.w;
                 } else {
-                    const char* ks_l = smem + stage_it * G::STAGE;
-                    if constexpr (KT) {
+                    win = make_row_win(cached_row_map<BM>(&s_ps, cur_seg, wave * 32 + lm), cpl);
+                    first = cpl.uniform ? 0 : win_phase(win);
+                    sp = wave_span(win, cpl.uniform != 0);
+                }
+                if (!cpl.uniform) {
+                    // periodic part of the row's live positions (position 0 of the walk is column c0)
+                    dec = BN % win.lin;
+                    uint64_t pt_bits = 0;
+                    for (int q = 0; q < 64; q += win.lin) pt_bits |= 1ull << q;
+                    pat = pt_bits;
+                } else {  // unit step: every position of the span
+                    pat = ~0ull;
+                }
+                w_lo_min = sp.lo_min, w_lo_max = sp.lo_max, w_hi_min = sp.hi_min, w_hi_max = sp.hi_max;
+                if constexpr (PLANNED) {
+                    // keep the spans in vector registers, as the reductions of the other path leave them
+                    asm volatile("v_mov_b32 %0, %0" : "+v"(w_lo_min));
+                    asm volatile("v_mov_b32 %0, %0" : "+v"(w_lo_max));
+                    asm volatile("v_mov_b32 %0, %0" : "+v"(w_hi_min));
+                    asm volatile("v_mov_b32 %0, %0" : "+v"(w_hi_max));
+                }
+            }
+            const int j0 = cur_tile * BN;
+            ++cur_tile;
+
+            // This wavefront's part of tile `it` has landed once at most the copies of the later tiles in flight
+            // are outstanding; after the barrier every part has, and every wavefront is done with tile it - 1,
+            // whose stage the next fetch overwrites.
+            {
+                const int later = total_tiles - 1 - it;
+                if (PD == 1 || later == 0)
+                    wait_loads<0>();
+                else if (later == 1)
+                    wait_loads<NDMA>();
+                else
+                    wait_loads<NDMA*(PD > 1 ? PD - 1 : 1)>();
+            }
+            __builtin_amdgcn_s_barrier();
+
+            const bool fetch = (it + PD < total_tiles);
+            bool spread = false;  // the fetch is issued piecewise between the matrix instructions below
+            if (fetch) {
+                spread = tile_is_fast(ppl, pf_tile);
+                if (!spread) issue_tile_general(ppl, pf_tile, stage_pf);
+            }
+
+            const bool skip = (j0 + BN <= w_lo_min) || (j0 >= w_hi_max);
+            if (!skip) {
+                const bool full = (j0 >= w_lo_max) && (j0 + BN <= w_hi_min);
+
+                // ---- S^T = K . Q^T ----
+                // K fragments are requested from LDS a few MFMAs ahead of their use, never more than 12 read
+                // instructions at a time: the counter that tracks them holds 15, and the compiler falls back to
+                // waiting for every outstanding read once it could overflow.
+                f32x16 s_acc[NT];
 #pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            kf.v[e] = *reinterpret_cast<const float*>(ks_l + (16 * ks + 8 * g + e) * G::K_ROWB + (32 * nt + lm) * 4);
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) s_acc[nt][j] = 0.f;
+                Frag<T> kfr[NT][KS];
+                auto load_k = [&](int nt, int ks) {
+                    Frag<T> kf;
+                    if constexpr (ES == 2) {
+                        if constexpr (KT) {
+                            // rows 16ks + 8g + {0..3} and +4: multiples of 4 rows leave the lane's swizzle term alone
+                            const uint32_t a0 = k_addr[nt] + 16 * ks * G::K_ROWB;
+                            kf = frag_from_tr<T>(lds_load_tr16(a0), lds_load_tr16(a0 + 4 * G::K_ROWB));
+                        } else {
+                            kf.v = __builtin_bit_cast(typename Frag<T>::vec, lds_load128(k_addr[ks] + 32 * nt * G::K_ROWB));
+                        }
                     } else {
-                        kf = lds_frag_row_swz<T, G::K_ROWB>(ks_l, 32 * nt + lm, 16 * ks + 8 * g);
+                        const char* ks_l = smem + stage_it * G::STAGE;
+                        if constexpr (KT) {
+#pragma unroll
+                            for (int e = 0; e < 8; ++e)
+                                kf.v[e] = *reinterpret_cast<const float*>(ks_l + (16 * ks + 8 * g + e) * G::K_ROWB + (32 * nt + lm) * 4);
+                        } else {
+                            kf = lds_frag_row_swz<T, G::K_ROWB>(ks_l, 32 * nt + lm, 16 * ks + 8 * g);
+                        }
                     }
-                }
-                return kf;
-            };
-            constexpr int NMMA = NT * KS;
-            constexpr int K_AHEAD = (ES != 2) ? NMMA : ((KT ? 6 : 12) < NMMA ? (KT ? 6 : 12) : NMMA);  // fragments
+                    return kf;
+                };
+                constexpr int NMMA = NT * KS;
+                constexpr int K_AHEAD = (ES != 2) ? NMMA : ((KT ? 6 : 12) < NMMA ? (KT ? 6 : 12) : NMMA);  // fragments
 #pragma unroll
-            for (int i = 0; i < K_AHEAD; ++i) kfr[i / KS][i % KS] = load_k(i / KS, i % KS);
-            __builtin_amdgcn_sched_barrier(0);  // keep the requests above the matrix work
-            // the copy instructions of the fetch go between the MFMAs, so that the address path sees them at
-            // the rate it can take instead of as one burst that stalls the wavefront
-            constexpr int MMA_PER_DMA = (NMMA / NDMA) > 0 ? NMMA / NDMA : 1;
+                for (int i = 0; i < K_AHEAD; ++i) kfr[i / KS][i % KS] = load_k(i / KS, i % KS);
+                __builtin_amdgcn_sched_barrier(0);  // keep the requests above the matrix work
+                // the copy instructions of the fetch go between the MFMAs, so that the address path sees them at
+                // the rate it can take instead of as one burst that stalls the wavefront
+                constexpr int MMA_PER_DMA = (NMMA / NDMA) > 0 ? NMMA / NDMA : 1;
 #pragma unroll
-            for (int i = 0; i < NMMA; ++i) {
-                mma32(s_acc[i / KS], kfr[i / KS][i % KS], qf[i % KS]);
-                if (i + K_AHEAD < NMMA) {
-                    kfr[(i + K_AHEAD) / KS][(i + K_AHEAD) % KS] = load_k((i + K_AHEAD) / KS, (i + K_AHEAD) % KS);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-                if constexpr (FAST_DMA) {
-                    if ((i + 1) % MMA_PER_DMA == 0 && (i + 1) / MMA_PER_DMA <= NDMA) {
-                        if (spread) issue_step((i + 1) / MMA_PER_DMA - 1, stage_pf);
+                for (int i = 0; i < NMMA; ++i) {
+                    mma32(s_acc[i / KS], kfr[i / KS][i % KS], qf[i % KS]);
+                    if (i + K_AHEAD < NMMA) {
+                        kfr[(i + K_AHEAD) / KS][(i + K_AHEAD) % KS] = load_k((i + K_AHEAD) / KS, (i + K_AHEAD) % KS);
                         __builtin_amdgcn_sched_barrier(0);
                     }
-                }
-            }
-            if constexpr (FAST_DMA && (NMMA / MMA_PER_DMA < NDMA)) {
-                if (spread) {
-#pragma unroll
-                    for (int s = NMMA / MMA_PER_DMA; s < NDMA; ++s) issue_step(s, stage_pf);
-                }
-            }
-            // ---- mask, online softmax against a lazily updated reference ----
-            Frag<T> pf[NT][2];
-            if (full)
-                softmax_tile<true, NT, T, DT>(s_acc, pf, m_ref, l_run, o_acc, 0ull, g, c2);
-            else
-                softmax_tile<false, NT, T, DT>(s_acc, pf, m_ref, l_run, o_acc, row_live_bits(win, j0, first, pat), g, c2);
-            // ---- O^T += V^T . P^T ----
-            // V fragments are requested one 16-key step (DT fragments) ahead of the MFMAs that consume them.
-            auto load_v = [&](int nt, int t, int dt) {
-                Frag<T> vf;
-                if constexpr (ES == 2) {
-                    const uint32_t a0 = v_addr[dt] + (32 * nt + 16 * t) * G::V_ROWB;
-                    vf = frag_from_tr<T>(lds_load_tr16(a0), lds_load_tr16(a0 + 8 * G::V_ROWB));
-                } else {
-                    const int rbase = 32 * nt + 16 * t + 4 * g;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        vf.v[e] = lds_load_f32(v_addr[dt] + (rbase + e) * G::V_ROWB);
-                        vf.v[4 + e] = lds_load_f32(v_addr[dt] + (rbase + 8 + e) * G::V_ROWB);
+                    if constexpr (FAST_DMA) {
+                        if ((i + 1) % MMA_PER_DMA == 0 && (i + 1) / MMA_PER_DMA <= NDMA) {
+                            if (spread) issue_step((i + 1) / MMA_PER_DMA - 1, stage_pf);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
                     }
                 }
-                return vf;
-            };
-            Frag<T> vfr[2][DT];
+                if constexpr (FAST_DMA && (NMMA / MMA_PER_DMA < NDMA)) {
+                    if (spread) {
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) vfr[0][dt] = load_v(0, 0, dt);
-            __builtin_amdgcn_sched_barrier(0);  // keep the requests above the matrix work
-#pragma unroll
-            for (int step = 0; step < 2 * NT; ++step) {
-                const int nt = step >> 1, t = step & 1;
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-                    mma32(o_acc[dt], vfr[step & 1][dt], pf[nt][t]);
-                    if (step + 1 < 2 * NT) {
-                        vfr[(step + 1) & 1][dt] = load_v((step + 1) >> 1, (step + 1) & 1, dt);
-                        __builtin_amdgcn_sched_barrier(0);
+                        for (int s = NMMA / MMA_PER_DMA; s < NDMA; ++s) issue_step(s, stage_pf);
                     }
                 }
-            }
-        } else if (spread) {
-#pragma unroll
-            for (int s = 0; s < NDMA; ++s) issue_step(s, stage_pf);
-        }
+                // ---- mask, online softmax against a lazily updated reference ----
+                Frag<T> pf[NT][2];
+                if (!full) mask_tile<NT>(s_acc, row_live_bits(win, j0, first, pat), g);
+                if (settled && !careful_only)
+                    l_run += exp_tile<NT, T>(s_acc, pf, m_ref * c2, c2);
+                else
+                    settled = softmax_tile<NT, T, DT>(s_acc, pf, m_ref, l_run, o_acc, c2);
 
-        if (fetch) {
-            advance_fetch();
-            stage_pf = (stage_pf + 1 == NSTAGE) ? 0 : stage_pf + 1;
-        }
-        if (!cpl.uniform) {  // phase of the periodic mask at the next tile
-            const int f = first - dec;
-            first = f < 0 ? f + win.lin : f;
-        }
-        // the next stage becomes current
-        stage_it = (stage_it + 1 == NSTAGE) ? 0 : stage_it + 1;
-        const int delta = (stage_it == 0) ? -(NSTAGE - 1) * G::STAGE : G::STAGE;
+                // ---- O^T += V^T . P^T ----
+                // V fragments are requested one 16-key step (DT fragments) ahead of the MFMAs that consume them.
+                auto load_v = [&](int nt, int t, int dt) {
+                    Frag<T> vf;
+                    if constexpr (ES == 2) {
+                        const uint32_t a0 = v_addr[dt] + (32 * nt + 16 * t) * G::V_ROWB;
+                        vf = frag_from_tr<T>(lds_load_tr16(a0), lds_load_tr16(a0 + 8 * G::V_ROWB));
+                    } else {
+                        const int rbase = 32 * nt + 16 * t + 4 * g;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) v_addr[dt] += delta;
+                        for (int e = 0; e < 4; ++e) {
+                            vf.v[e] = lds_load_f32(v_addr[dt] + (rbase + e) * G::V_ROWB);
+                            vf.v[4 + e] = lds_load_f32(v_addr[dt] + (rbase + 8 + e) * G::V_ROWB);
+                        }
+                    }
+                    return vf;
+                };
+                Frag<T> vfr[2][DT];
 #pragma unroll
-        for (int i = 0; i < (KT ? NT : KS); ++i) k_addr[i] += delta;
+                for (int dt = 0; dt < DT; ++dt) vfr[0][dt] = load_v(0, 0, dt);
+                __builtin_amdgcn_sched_barrier(0);  // keep the requests above the matrix work
+#pragma unroll
+                for (int step = 0; step < 2 * NT; ++step) {
+                    const int nt = step >> 1, t = step & 1;
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) {
+                        mma32(o_acc[dt], vfr[step & 1][dt], pf[nt][t]);
+                        if (step + 1 < 2 * NT) {
+                            vfr[(step + 1) & 1][dt] = load_v((step + 1) >> 1, (step + 1) & 1, dt);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
+                }
+            } else if (spread) {
+#pragma unroll
+                for (int s = 0; s < NDMA; ++s) issue_step(s, stage_pf);
+            }
+
+            if (fetch) {
+                advance_fetch();
+                stage_pf = (stage_pf + 1 == NSTAGE) ? 0 : stage_pf + 1;
+            }
+            if (!cpl.uniform) {  // phase of the periodic mask at the next tile
+                const int f = first - dec;
+                first = f < 0 ? f + win.lin : f;
+            }
+            // the next stage becomes current
+            stage_it = (stage_it + 1 == NSTAGE) ? 0 : stage_it + 1;
+            const int delta = (stage_it == 0) ? -(NSTAGE - 1) * G::STAGE : G::STAGE;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) v_addr[dt] += delta;
+#pragma unroll
+            for (int i = 0; i < (KT ? NT : KS); ++i) k_addr[i] += delta;
+        }
+        // Every copy has been waited for (the last tile waits for all).  The barrier in here also makes the stages free
+        // for the epilogue (or the second pass): every wavefront has finished reading the last tile.
+        const bool bad = !careful_only && (!(l_run < 1.0e30f) || !(fabsf(o_acc[0][0]) < 1.0e30f));
+        if (!__syncthreads_or(bad ? 1 : 0)) break;
+        careful_only = true;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) v_addr[dt] -= stage_it * G::STAGE;
+#pragma unroll
+        for (int i = 0; i < (KT ? NT : KS); ++i) k_addr[i] -= stage_it * G::STAGE;
     }
-    // every copy has been waited for (the last tile waits for all); the stages become staging space below once
-    // every wavefront has finished reading the last tile
-    __builtin_amdgcn_s_barrier();
 
     // ---- epilogue: O = O^T / l, transposed through LDS so that every global store is a contiguous run --------
     {
