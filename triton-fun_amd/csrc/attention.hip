@@ -338,6 +338,7 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
     // or output turns infinite or NaN and stays so, which is checked after the last tile, and the workgroup then
     // repeats its tiles on the careful path alone.
     bool careful_only = false;
+    int stage_it = 0;  // stage that holds the tile being computed (the LDS read addresses stand at it)
     for (;;) {
         pf_seg = 0;
         pf_enter_segment();
@@ -351,9 +352,9 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
             if (i < total_tiles) {
                 if (tile_is_fast(ppl, pf_tile)) {
 #pragma unroll
-                    for (int s = 0; s < NDMA; ++s) issue_step(s, i);
+                    for (int s = 0; s < NDMA; ++s) issue_step(s, (stage_it + i) % NSTAGE);
                 } else {
-                    issue_tile_general(ppl, pf_tile, i);
+                    issue_tile_general(ppl, pf_tile, (stage_it + i) % NSTAGE);
                 }
                 advance_fetch();
             }
@@ -374,8 +375,7 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
         SegPlan cpl = {0, 1, 0, 1};
         const float c2 = p.scale_log2e;
         bool settled = false;         // every row of this wavefront has a reference
-        int stage_it = 0;             // stage that holds tile `it`
-        int stage_pf = PD % NSTAGE;   // stage the next fetch goes to
+        int stage_pf = (stage_it + PD) % NSTAGE;  // stage the next fetch goes to
         // The Q fragments have to be in their registers before the loop: otherwise the compiler puts its waits for them
         // in front of the first score MFMAs of every tile, counted against the loads it knows of, and those waits would
         // then hold for the copies of the next tile that are in flight at that point.
@@ -576,11 +576,7 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
         // for the epilogue (or the second pass): every wavefront has finished reading the last tile.
         const bool bad = !careful_only && (!(l_run < 1.0e30f) || !(fabsf(o_acc[0][0]) < 1.0e30f));
         if (!__syncthreads_or(bad ? 1 : 0)) break;
-        careful_only = true;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) v_addr[dt] -= stage_it * G::STAGE;
-#pragma unroll
-        for (int i = 0; i < (KT ? NT : KS); ++i) k_addr[i] -= stage_it * G::STAGE;
+        careful_only = true;  // the ring goes on from the stage it stands at
     }
 
     // ---- epilogue: O = O^T / l, transposed through LDS so that every global store is a contiguous run --------

@@ -57,79 +57,90 @@ struct Vec8 {
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kNegBig = -1.0e30f;
 
-// LPR lanes share one row (64 / LPR rows per wavefront): rows shorter than 512 slots still fill every lane.
-template <typename Tin, typename Tout, int NCH, int LPR>
+// LPR lanes share one row (64 / LPR rows per wavefront): rows shorter than 512 slots still fill every lane.  A wavefront
+// takes RIF such row groups at once and requests all of their chunks before it looks at any (bytes in flight per
+// wavefront are what a streaming kernel lives on).
+template <typename Tin, typename Tout, int NCH, int LPR, int RIF>
 __global__ __launch_bounds__(256) void softmax_rows_vec(const Tin* __restrict__ x, Tout* __restrict__ y, SoftmaxSegs segs,
                                                         int64_t n_rows, int L, int T) {
     typedef typename Vec8<Tin>::type vin;
     typedef typename Vec8<Tout>::type vout;
-    constexpr int RPW = 64 / LPR;  // rows per wavefront
+    constexpr int RPW = 64 / LPR;  // rows per wavefront and group
     const int lane = threadIdx.x & (LPR - 1);
-    const int64_t row_raw = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW + ((threadIdx.x & 63) / LPR);
-    const bool row_ok = row_raw < n_rows;
-    if (RPW == 1 && !row_ok) return;
-    const int64_t row = row_ok ? row_raw : n_rows - 1;  // surplus lane groups shadow the last row and store nothing
-    LiveRanges lr;
-    const Tin* xr = x + row * (int64_t)T;
-    Tout* yr = y + row * (int64_t)T;
+    const int64_t row0 = (((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * RIF) * RPW + ((threadIdx.x & 63) / LPR);
+    if (RPW == 1 && row0 >= n_rows) return;
     const int nchunk = T >> 3;
 
-    float v[NCH][8];
-    uint32_t live[NCH];
-    float mx = kNegBig;
-    // the loads do not wait for the row's live counts: a chunk inside the row is fetched whole and the dead
+    // the loads do not wait for the rows' live counts: a chunk inside the row is fetched whole and the dead
     // slots in it are discarded afterwards
-    vin raw[NCH];
+    vin raw[RIF][NCH];
+    bool row_ok[RIF];
+    int64_t row[RIF];
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-        const int ch = lane + LPR * c;
-        if (ch < nchunk) raw[c] = __builtin_nontemporal_load(reinterpret_cast<const vin*>(xr + (ch << 3)));
-    }
-    lr.load(segs, (int)(row % L), T);
+    for (int i = 0; i < RIF; ++i) {
+        const int64_t row_raw = row0 + (int64_t)i * RPW;
+        row_ok[i] = row_raw < n_rows;
+        row[i] = row_ok[i] ? row_raw : n_rows - 1;  // surplus lane groups shadow the last row and store nothing
+        const Tin* xr = x + row[i] * (int64_t)T;
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-        const int ch = lane + LPR * c;
-        live[c] = (ch < nchunk) ? lr.live8(ch << 3) : 0u;
-        if (live[c]) {
-            const vin t = raw[c];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                v[c][e] = ((live[c] >> e) & 1u) ? (float)t[e] : kNegBig;
-                mx = fmaxf(mx, v[c][e]);
-            }
-        }
-    }
-#pragma unroll
-    for (int o = LPR / 2; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
-    const float mb = mx * kLog2e;
-    float sum = 0.f;
-#pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-        if (live[c]) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                float p = ((live[c] >> e) & 1u) ? fast_exp2(fmaf(v[c][e], kLog2e, -mb)) : 0.f;
-                v[c][e] = p;
-                sum += p;
-            }
-        }
-    }
-#pragma unroll
-    for (int o = LPR / 2; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
-    const float inv = sum > 0.f ? 1.0f / sum : 0.f;
-#pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-        if (live[c] && row_ok) {
+        for (int c = 0; c < NCH; ++c) {
             const int ch = lane + LPR * c;
-            if (live[c] == 0xffu) {
-                vout o;
+            if (ch < nchunk) raw[i][c] = __builtin_nontemporal_load(reinterpret_cast<const vin*>(xr + (ch << 3)));
+        }
+    }
 #pragma unroll
-                for (int e = 0; e < 8; ++e) o[e] = (Tout)(v[c][e] * inv);
-                *reinterpret_cast<vout*>(yr + (ch << 3)) = o;
-            } else {
+    for (int i = 0; i < RIF; ++i) {
+        LiveRanges lr;
+        lr.load(segs, (int)(row[i] % L), T);
+        Tout* yr = y + row[i] * (int64_t)T;
+        float v[NCH][8];
+        uint32_t live[NCH];
+        float mx = kNegBig;
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    if ((live[c] >> e) & 1u) yr[(ch << 3) + e] = (Tout)(v[c][e] * inv);
+        for (int c = 0; c < NCH; ++c) {
+            const int ch = lane + LPR * c;
+            live[c] = (ch < nchunk) ? lr.live8(ch << 3) : 0u;
+            if (live[c]) {
+                const vin t = raw[i][c];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    v[c][e] = ((live[c] >> e) & 1u) ? (float)t[e] : kNegBig;
+                    mx = fmaxf(mx, v[c][e]);
+                }
+            }
+        }
+#pragma unroll
+        for (int o = LPR / 2; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+        const float mb = mx * kLog2e;
+        float sum = 0.f;
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            if (live[c]) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    float p = ((live[c] >> e) & 1u) ? fast_exp2(fmaf(v[c][e], kLog2e, -mb)) : 0.f;
+                    v[c][e] = p;
+                    sum += p;
+                }
+            }
+        }
+#pragma unroll
+        for (int o = LPR / 2; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+        const float inv = sum > 0.f ? 1.0f / sum : 0.f;
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            if (live[c] && row_ok[i]) {
+                const int ch = lane + LPR * c;
+                if (live[c] == 0xffu) {
+                    vout o;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) o[e] = (Tout)(v[c][e] * inv);
+                    *reinterpret_cast<vout*>(yr + (ch << 3)) = o;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if ((live[c] >> e) & 1u) yr[(ch << 3) + e] = (Tout)(v[c][e] * inv);
+                }
             }
         }
     }
@@ -168,18 +179,19 @@ static int launch_softmax(const void* x, void* y, const SoftmaxSegs& segs, int64
     Tout* yo = (Tout*)y;
     if (aligned && (T & 7) == 0 && T <= 2048) {
         const int nch = (T / 8 + 63) / 64;
-        if (T <= 128) {
-            grid = (unsigned)((n_rows + 15) / 16);
-            softmax_rows_vec<Tin, Tout, 1, 16><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
-        } else if (T <= 256) {
-            grid = (unsigned)((n_rows + 7) / 8);
-            softmax_rows_vec<Tin, Tout, 1, 32><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
-        } else if (nch <= 1)
-            softmax_rows_vec<Tin, Tout, 1, 64><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+        // row groups in flight per wavefront: 4 where a row is 512 bytes or more (+7 % at T = 512, +4 % at T = 256 over
+        // one group, measured), one for shorter rows (more was slower there)
+        auto groups = [&](int rows_per_wave) { return (unsigned)((n_rows + 4 * rows_per_wave - 1) / (4 * rows_per_wave)); };
+        if (T <= 128)
+            softmax_rows_vec<Tin, Tout, 1, 16, 1><<<groups(4), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+        else if (T <= 256)
+            softmax_rows_vec<Tin, Tout, 1, 32, 4><<<groups(2 * 4), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+        else if (nch <= 1)
+            softmax_rows_vec<Tin, Tout, 1, 64, 4><<<groups(4), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
         else if (nch <= 2)
-            softmax_rows_vec<Tin, Tout, 2, 64><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+            softmax_rows_vec<Tin, Tout, 2, 64, 1><<<groups(1), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
         else
-            softmax_rows_vec<Tin, Tout, 4, 64><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+            softmax_rows_vec<Tin, Tout, 4, 64, 1><<<groups(1), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
     } else {
         softmax_rows_any<Tin, Tout><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
     }
