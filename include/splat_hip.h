@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define SPLAT_VERSION 100 /* major*10000 + minor*100 + patch */
+#define SPLAT_VERSION 200 /* major*10000 + minor*100 + patch; 0.2.0 added the planned forward */
 
 /* element types of q/k/v/score/output buffers */
 #define SPLAT_F32 0
