@@ -165,6 +165,8 @@ class RegularAttention(nn.Module):
         if fusable:
             if self._plan is None:
                 self._plan = attention_plan(self.segments, self._shape[2], self._device)
+                # once, so that later forwards may run on any stream without ordering themselves after the plan kernel
+                torch.cuda.current_stream(self._device).synchronize()
             return attention_launcher(q, k, v, self.rspmm_output, self.segments, self.scale, self._plan)
 
         multi = self.segments if len(self.segments) > 1 else None
