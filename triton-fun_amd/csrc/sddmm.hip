@@ -71,8 +71,11 @@ __device__ __forceinline__ void store_piece(TO* row_out, const RowWin& w, int jj
     }
 }
 
-template <typename T, bool KT, bool QREG>
+// KSU: 0 = the contraction is longer than one LDS chunk (Q fragments are re-read per chunk); otherwise Q stays in
+// registers, and KSU > 0 says at compile time how many MFMA steps hold data (-1: known at run time only).
+template <typename T, bool KT, int KSU>
 __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
+    constexpr bool QREG = KSU != 0;
     constexpr int ES = sizeof(T);
     constexpr int BM = 128;
     constexpr int NT = kBN / 32;
@@ -216,25 +219,49 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
                 }
                 __syncthreads();
                 if (skip) continue;
-#pragma unroll
-                for (int ks = 0; ks < KSC; ++ks) {
-                    if (QREG && ks >= ks_used) break;
-                    Frag<T> qv;
-                    if constexpr (QREG)
-                        qv = qf[ks];
+                auto load_k = [&](int ks, int nt) {
+                    if constexpr (KT)
+                        return lds_frag_cols<T>(s_k, K_ROW, 16 * ks + 8 * g, 16 * ks + 8 * g + 4, 32 * nt, lane);
                     else
-                        qv = load_q_frag<T>(qr, kd0 + 16 * ks + 8 * g, d, p.q_vec != 0);
+                        return lds_frag_rowmajor<T>(s_k + (32 * nt + lm) * K_ROW + (16 * ks + 8 * g) * ES);
+                };
+                if constexpr (KSU > 0 && !KT) {
+                    // the step count is a constant: no test per step, and fragments are requested four MFMAs ahead
+                    // (deeper read-ahead costs the third workgroup per CU its registers)
+                                        constexpr int NF = KSU * NT, AHEAD = NF < 4 ? NF : 4;
+                    Frag<T> kfr[NF];
 #pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) {
-                        Frag<T> kf;
-                        if constexpr (KT)
-                            kf = lds_frag_cols<T>(s_k, K_ROW, 16 * ks + 8 * g, 16 * ks + 8 * g + 4, 32 * nt, lane);
+                    for (int i = 0; i < AHEAD; ++i) kfr[i] = load_k(i / NT, i % NT);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int i = 0; i < NF; ++i) {
+                        mma32(acc[i % NT], kfr[i], qf[i / NT]);  // rows = keys, columns = queries
+                        if (i + AHEAD < NF) {
+                            kfr[i + AHEAD] = load_k((i + AHEAD) / NT, (i + AHEAD) % NT);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int ks = 0; ks < KSC; ++ks) {
+                        if (QREG && ks >= ks_used) break;
+                        Frag<T> qv;
+                        if constexpr (QREG)
+                            qv = qf[ks];
                         else
-                            kf = lds_frag_rowmajor<T>(s_k + (32 * nt + lm) * K_ROW + (16 * ks + 8 * g) * ES);
-                        mma32(acc[nt], kf, qv);  // rows = keys, columns = queries
+                            qv = load_q_frag<T>(qr, kd0 + 16 * ks + 8 * g, d, p.q_vec != 0);
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt) mma32(acc[nt], load_k(ks, nt), qv);  // rows = keys, columns = queries
                     }
                 }
             }
+            // The K loads of the next tile have to be back before this tile's stores are issued: loads and stores
+            // complete out of order with respect to each other, so a wait for the loads that comes after the stores
+            // is a wait for the stores as well.
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+            for (int i = 0; i < CPT; ++i) asm volatile("" ::"v"(kreg[i]));
+#endif
             if (skip) continue;
 
 #pragma unroll
@@ -273,17 +300,22 @@ static int launch_sddmm(SddmmParams p, bool kt, hipStream_t st) {
     p.n_row_blocks = count_row_blocks(p.L, 128, p.row_stride);
     p.total = p.B * p.H * p.n_row_blocks;
     const int grid = ((p.total + 7) / 8) * 8;
-    const bool qreg = p.d <= SddmmGeom<T>::DC;
+    constexpr int DC = SddmmGeom<T>::DC, KSC = DC / 16;
+    const int steps = (p.d + 15) / 16;
     if (kt) {
-        if (qreg)
-            sddmm_kernel<T, true, true><<<grid, 256, 0, st>>>(p);
+        if (p.d <= DC)
+            sddmm_kernel<T, true, -1><<<grid, 256, 0, st>>>(p);
         else
-            sddmm_kernel<T, true, false><<<grid, 256, 0, st>>>(p);
+            sddmm_kernel<T, true, 0><<<grid, 256, 0, st>>>(p);
     } else {
-        if (qreg)
-            sddmm_kernel<T, false, true><<<grid, 256, 0, st>>>(p);
+        if (p.d > DC)
+            sddmm_kernel<T, false, 0><<<grid, 256, 0, st>>>(p);
+        else if (steps == KSC)
+            sddmm_kernel<T, false, KSC><<<grid, 256, 0, st>>>(p);
+        else if (steps == KSC / 2)
+            sddmm_kernel<T, false, KSC / 2><<<grid, 256, 0, st>>>(p);
         else
-            sddmm_kernel<T, false, false><<<grid, 256, 0, st>>>(p);
+            sddmm_kernel<T, false, -1><<<grid, 256, 0, st>>>(p);
     }
     return check_launch("splat_sddmm");
 }
