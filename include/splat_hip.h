@@ -8,6 +8,7 @@
  *
  *   splat_acsr_build      <- acsr_helpers.py:99-160   instantiate_metadata + create_acsr
  *   splat_mask_generate   <- acsr_helpers.py:18-55    create_*_mask (device-side equivalent)
+ *   splat_acsr_build_pattern <- both of the above for the closed-form patterns, without the mask
  *   splat_sddmm           <- r_sddmm.py:15-115,171-184   rsddmm_kernel / rsddmm_launcher
  *   splat_softmax         <- r_softmax.py:16-59,126-150  r_softmax_1d_kernel / rsoftmax_launcher
  *   splat_spmm            <- r_spmm.py:13-126,148-164    r_spmm_kernel_row_maj_row_comp / rspmm_launcher
@@ -103,6 +104,16 @@ int splat_acsr_build(const uint8_t* mask, int64_t rows, int64_t cols, int64_t ld
  * Device-side equivalent of the O(s^2) Python loops at acsr_helpers.py:18-55. */
 int splat_mask_generate(uint8_t* mask, int64_t rows, int64_t cols, int64_t ld, int32_t pattern,
                         int64_t p0, int64_t p1, void* stream);
+
+/* The ACSR of one of the closed-form s x s patterns above, without the mask: every row of such a pattern is an
+ * arithmetic progression of columns, so what splat_acsr_build finds by scanning s*s bytes follows from
+ * (pattern, p0, p1, row) directly.  Same outputs, bit for bit, as splat_mask_generate + splat_acsr_build
+ * (instantiate_metadata / create_acsr, acsr_helpers.py:99-160, on create_*_mask, acsr_helpers.py:18-55), in
+ * O(s) work and no s*s buffer: what makes L in the hundreds of thousands practical. */
+int splat_acsr_build_pattern(int32_t pattern, int64_t s, int64_t p0, int64_t p1, int32_t block_height,
+                             float* dTos_lin, float* dTos_trans, float* sTod_lin, float* sTod_trans,
+                             float* nnz, float* span_start, float* span_end, int32_t* row_first,
+                             int32_t* row_last, int32_t* summary, void* stream);
 
 /* SDDMM: out[b,h,r,off+s] = scale * sum_k q[b,h,r,k] * kT[b,h,k,c(r,s)], s < nnz[r], per segment.
  * Replaces rsddmm_launcher / rsddmm_kernel, r_sddmm.py:15-115,171-184 (x = q, y = kT).

@@ -134,3 +134,44 @@ def test_preambles(dev, n, p, BH, BW):
 def test_preamble_assertion(dev):
     with pytest.raises(AssertionError, match="Issues with generating arrangement"):
         r_sddmm.rsddmm_preamble(np.eye(4, dtype=np.uint8), (1, 1, 4, 1), 2, 1, dev, torch.float32)
+
+
+def _pattern_cases():
+    cases = []
+    for s, p in [(1, 1), (10, 2), (130, 7), (128, 128), (100, 300), (1024, 328)]:
+        cases.append(("blocked", A.blocked_pattern(s, p)))
+    for s, p in [(1, 0), (64, 0), (100, 9), (333, 40), (50, 49), (50, 500)]:
+        cases.append(("windowed", A.windowed_pattern(s, p)))
+        cases.append(("causal", A.causal_windowed_pattern(s, p)))
+    for s, w, dil in [(200, 16, 3), (300, 16, 3), (520, 64, 3), (2048, 512, 2), (64, 512, 2), (100, 1, 5), (77, 8, 1), (90, 7, 4)]:
+        cases.append(("dilated", A.dilated_pattern(s, w, dil)))
+    for s, loc, st in [(300, 32, 16), (1024, 128, 128), (100, 1, 1), (64, 200, 7), (257, 5, 300)]:
+        for k, pat in enumerate(A.strided_patterns(s, loc, st)):
+            cases.append((f"strided{k}", pat))
+    return cases
+
+
+@pytest.mark.parametrize("case", _pattern_cases(), ids=lambda c: f"{c[0]}-{c[1].s}-{c[1].p0}-{c[1].p1}")
+@pytest.mark.parametrize("BH", [2, 16])
+def test_closed_form_pattern_builder_equals_mask_scan(dev, case, BH):
+    """splat_acsr_build_pattern (rows of the pattern in closed form, no mask) against splat_acsr_build on the
+    rasterised pattern, which the tests above pin to the oracle: every output array bit for bit, T and the row-stride
+    summary included; windows wider than the matrix, single-row matrices, dilations that run off either side."""
+    pat = case[1]
+    dev_t = torch.device(dev)
+    a = A.build_acsr(pat, BH, dev_t)                       # closed form
+    b = A.build_acsr(pat.device_mask(dev_t), BH, dev_t)    # scan of the rasterised mask
+    for name in ("dTos_lin", "dTos_trans", "sTod_lin", "sTod_trans", "nnz", "span_start", "span_end"):
+        assert np.array_equal(bits(getattr(a, name)), bits(getattr(b, name))), name
+    assert torch.equal(a.row_first, b.row_first) and torch.equal(a.row_last, b.row_last)
+    assert a.T == b.T and a.row_stride == b.row_stride
+
+
+def test_pattern_builder_needs_no_mask_for_long_sequences(dev):
+    """L = 2^20 rows (a 1 TiB mask): metadata in closed form, checked against the per-pattern formulas."""
+    L, w = 1 << 20, 512
+    got = A.create_acsr(A.causal_windowed_pattern(L, w - 1), 16, dev)
+    i = np.arange(L)
+    a = np.maximum(0, i - w + 1).astype(np.float64)
+    assert np.array_equal(bits(got[3]), bits(a)) and np.array_equal(bits(got[4]), bits(np.minimum(i + 1, w)))
+    assert got[5] == w

@@ -40,6 +40,7 @@ _SIGNATURES = {
     "splat_last_error": (ctypes.c_char_p, []),
     "splat_acsr_build": (ctypes.c_int, [_vp, _i64, _i64, _i64, _i32] + [_vp] * 10 + [_vp]),
     "splat_mask_generate": (ctypes.c_int, [_vp, _i64, _i64, _i64, _i32, _i64, _i64, _vp]),
+    "splat_acsr_build_pattern": (ctypes.c_int, [_i32, _i64, _i64, _i64, _i32] + [_vp] * 10 + [_vp]),
     "splat_sddmm": (ctypes.c_int, [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, ctypes.POINTER(AcsrSeg), _i32,
                                    _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _i32, _vp]),
     "splat_softmax": (ctypes.c_int, [_vp, _vp, ctypes.POINTER(AcsrSeg), _i32, _i64, _i32, _i32, _i32, _i32, _vp]),

@@ -178,7 +178,7 @@ def _mask_entry(mask, dev: torch.device) -> _MaskEntry:
         if e.key_obj[0] == key:
             return e
     if isinstance(mask, MaskPattern):
-        dm = mask.device_mask(dev)
+        dm = None  # never rasterised for the builder: its rows are known in closed form
     elif isinstance(mask, torch.Tensor):
         dm = mask.to(device=dev, dtype=torch.uint8).contiguous()
     else:
@@ -188,7 +188,7 @@ def _mask_entry(mask, dev: torch.device) -> _MaskEntry:
         if arr.size and (arr.min() < 0 or arr.max() > 255):
             raise ValueError("mask entries must fit in a byte")
         dm = torch.from_numpy(np.ascontiguousarray(arr, dtype=np.uint8)).to(dev)
-    if dm.dim() != 2:
+    if dm is not None and dm.dim() != 2:
         raise ValueError("mask must be 2-D")
     entry = _MaskEntry((key, mask), dm)
     _MASK_CACHE.append(entry)
@@ -215,7 +215,7 @@ def build_acsr(mask, BLOCK_HEIGHT: int, dev: torch.device) -> AcsrBuild:
     if BLOCK_HEIGHT in entry.builds:
         return entry.builds[BLOCK_HEIGHT]
     dm = entry.mask
-    rows, cols = dm.shape
+    rows, cols = mask_shape(mask) if dm is None else dm.shape
     n_blocks = ceil(rows / BLOCK_HEIGHT)
     f32 = dict(dtype=torch.float32, device=dev)
     b = AcsrBuild()
@@ -226,13 +226,17 @@ def build_acsr(mask, BLOCK_HEIGHT: int, dev: torch.device) -> AcsrBuild:
     b.row_first = torch.empty(rows, dtype=torch.int32, device=dev)
     b.row_last = torch.empty(rows, dtype=torch.int32, device=dev)
     summary = torch.empty(8, dtype=torch.int32, device=dev)
+    outs = (b.dTos_lin.data_ptr(), b.dTos_trans.data_ptr(), b.sTod_lin.data_ptr(), b.sTod_trans.data_ptr(), b.nnz.data_ptr(),
+            b.span_start.data_ptr(), b.span_end.data_ptr(), b.row_first.data_ptr(), b.row_last.data_ptr(), summary.data_ptr())
     with torch.cuda.device(dev):
-        rc = _hip.lib().splat_acsr_build(dm.data_ptr(), rows, cols, dm.stride(0), BLOCK_HEIGHT, b.dTos_lin.data_ptr(),
-                                         b.dTos_trans.data_ptr(), b.sTod_lin.data_ptr(), b.sTod_trans.data_ptr(),
-                                         b.nnz.data_ptr(), b.span_start.data_ptr(), b.span_end.data_ptr(),
-                                         b.row_first.data_ptr(), b.row_last.data_ptr(), summary.data_ptr(),
-                                         _hip.stream_ptr(dev))
-    _hip.check(rc, "splat_acsr_build")
+        if dm is None:  # a MaskPattern: O(rows) work, no rows x cols buffer
+            rc = _hip.lib().splat_acsr_build_pattern(mask.kind, mask.s, mask.p0, mask.p1, BLOCK_HEIGHT, *outs,
+                                                     _hip.stream_ptr(dev))
+            _hip.check(rc, "splat_acsr_build_pattern")
+        else:
+            rc = _hip.lib().splat_acsr_build(dm.data_ptr(), rows, cols, dm.stride(0), BLOCK_HEIGHT, *outs,
+                                             _hip.stream_ptr(dev))
+            _hip.check(rc, "splat_acsr_build")
     host = summary.cpu()  # the one synchronisation: T is returned as a Python int, like the reference
     assert int(host[1]) == 0, "Incorrect unpacking of affine-indices."
     b.T = int(host[0])

@@ -268,6 +268,70 @@ __device__ __forceinline__ bool mask_pred(int pattern, int64_t i, int64_t j, int
     return false;
 }
 
+// What a scan of row i of the s x s pattern would find, in closed form: every pattern's row is an arithmetic
+// progression of columns (first, step, count), clipped to [0, s).
+__device__ __forceinline__ RowScan pattern_row(int pattern, int64_t i, int64_t s, int64_t p0, int64_t p1) {
+    int64_t first = 0, step = 1, count = 0;
+    switch (pattern) {
+        case SPLAT_MASK_BLOCKED: {
+            const int64_t start = (i < p0) ? 0 : (i / p0 - 1) * p0;
+            const int64_t end = (i < p0) ? p0 : start + 2 * p0;  // exclusive
+            first = start;
+            count = min(end, s) - start;
+            break;
+        }
+        case SPLAT_MASK_WINDOWED:
+            first = max((int64_t)0, i - p0);
+            count = min(s - 1, i + p0) - first + 1;
+            break;
+        case SPLAT_MASK_CAUSAL_WINDOWED:
+            first = max((int64_t)0, i - p0);
+            count = min(s - 1, i) - first + 1;
+            break;
+        case SPLAT_MASK_STRIDED_LOCAL:
+            first = max((int64_t)0, i - p0 + 1);
+            count = min(s - 1, i) - first + 1;
+            break;
+        case SPLAT_MASK_DILATED: {
+            const int64_t base = i - (p0 * p1) / 2;  // column of t = 0; columns base + t * p1, t in [0, p0)
+            const int64_t t_lo = base < 0 ? (-base + p1 - 1) / p1 : 0;
+            const int64_t room = s - 1 - base;
+            const int64_t t_hi = room < 0 ? -1 : min(p0 - 1, room / p1);
+            step = p1;
+            first = base + t_lo * p1;
+            count = t_hi - t_lo + 1;
+            break;
+        }
+        case SPLAT_MASK_STRIDED_FAR: {
+            const int64_t room = min(i - p0, s - 1) - (p1 - 1);  // columns p1 - 1 + t * p1 <= i - p0
+            step = p1;
+            first = p1 - 1;
+            count = room < 0 ? 0 : room / p1 + 1;
+            break;
+        }
+    }
+    RowScan r;
+    r.init();
+    if (count > 0) {
+        r.sum = (uint32_t)count;
+        r.m1 = r.first = (int)first;
+        if (count > 1) r.m2 = (int)(first + step);
+        r.last = (int)(first + (count - 1) * step);
+    }
+    return r;
+}
+
+__global__ __launch_bounds__(256) void acsr_rows_pattern_kernel(int pattern, int s, int64_t p0, int64_t p1,
+                                                                float* __restrict__ dTos_lin, float* __restrict__ dTos_trans,
+                                                                float* __restrict__ sTod_lin, float* __restrict__ sTod_trans,
+                                                                float* __restrict__ nnz_out, int32_t* __restrict__ row_first,
+                                                                int32_t* __restrict__ row_last, int32_t* __restrict__ summary) {
+    const int row = blockIdx.x * blockDim.x + threadIdx.x;
+    if (row >= s) return;
+    finish_row(pattern_row(pattern, row, s, p0, p1), row, s, dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnz_out, row_first,
+               row_last, summary);
+}
+
 __global__ __launch_bounds__(256) void mask_generate_kernel(uint8_t* __restrict__ mask, int rows, int cols,
                                                             int64_t ld, int pattern, int64_t p0, int64_t p1,
                                                             int vec_ok) {
@@ -319,6 +383,36 @@ extern "C" int splat_acsr_build(const uint8_t* mask, int64_t rows, int64_t cols,
     acsr_spans_kernel<<<(n_blocks + 255) / 256, 256, 0, st>>>(sTod_lin, sTod_trans, nnz, (int)rows, (int)cols, block_height,
                                                                span_start, span_end, summary);
     return check_launch("splat_acsr_build");
+}
+
+static int check_pattern(const char* who, int64_t s, int32_t pattern, int64_t p0, int64_t p1) {
+    if (s <= 0 || s > (1 << 23)) return fail(SPLAT_E_SHAPE, "%s: need 0 < s <= 2^23 (got %lld)", who, (long long)s);
+    if (pattern < SPLAT_MASK_BLOCKED || pattern > SPLAT_MASK_STRIDED_FAR)
+        return fail(SPLAT_E_UNSUPPORTED, "%s: unknown pattern %d", who, pattern);
+    const bool needs_p1 = pattern == SPLAT_MASK_DILATED || pattern == SPLAT_MASK_STRIDED_FAR;
+    if (p0 < 0 || (pattern == SPLAT_MASK_BLOCKED && p0 <= 0) || (needs_p1 && p1 <= 0))
+        return fail(SPLAT_E_SHAPE, "%s: bad pattern parameters p0=%lld p1=%lld", who, (long long)p0, (long long)p1);
+    return 0;
+}
+
+extern "C" int splat_acsr_build_pattern(int32_t pattern, int64_t s, int64_t p0, int64_t p1, int32_t block_height,
+                                        float* dTos_lin, float* dTos_trans, float* sTod_lin, float* sTod_trans, float* nnz,
+                                        float* span_start, float* span_end, int32_t* row_first, int32_t* row_last,
+                                        int32_t* summary, void* stream) {
+    const char* who = "splat_acsr_build_pattern";
+    if (!dTos_lin || !dTos_trans || !sTod_lin || !sTod_trans || !nnz || !span_start || !span_end || !summary)
+        return fail(SPLAT_E_NULL, "%s: null pointer argument", who);
+    if (block_height <= 0) return fail(SPLAT_E_SHAPE, "%s: block_height must be > 0 (got %d)", who, block_height);
+    if (int rc = check_pattern(who, s, pattern, p0, p1)) return rc;
+    if (p0 > (1 << 23) || p1 > (1 << 23)) return fail(SPLAT_E_SHAPE, "%s: pattern parameters are limited to 2^23", who);
+    hipStream_t st = (hipStream_t)stream;
+    acsr_init_summary<<<1, 64, 0, st>>>(summary);
+    acsr_rows_pattern_kernel<<<(unsigned)((s + 255) / 256), 256, 0, st>>>(pattern, (int)s, p0, p1, dTos_lin, dTos_trans, sTod_lin,
+                                                                         sTod_trans, nnz, row_first, row_last, summary);
+    const int n_blocks = (int)((s + block_height - 1) / block_height);
+    acsr_spans_kernel<<<(n_blocks + 255) / 256, 256, 0, st>>>(sTod_lin, sTod_trans, nnz, (int)s, (int)s, block_height, span_start,
+                                                               span_end, summary);
+    return check_launch(who);
 }
 
 extern "C" int splat_mask_generate(uint8_t* mask, int64_t rows, int64_t cols, int64_t ld, int32_t pattern, int64_t p0,
