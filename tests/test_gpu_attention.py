@@ -156,11 +156,12 @@ def test_unit_projection_wrapper(dev):
     assert float((got - want).abs().max()) <= 1e-5
 
 
-@pytest.mark.parametrize("L,d,w,dtype", [(32768, 128, 512, torch.bfloat16), (40003, 64, 300, torch.float16)])
+@pytest.mark.parametrize("L,d,w,dtype", [(32768, 128, 512, torch.bfloat16), (40003, 64, 300, torch.float16),
+                                         (1 << 20, 128, 512, torch.bfloat16)])
 def test_long_sequences_by_properties(dev, L, d, w, dtype):
-    """Sequences longer than any BASELINE configuration, one of them not a multiple of any tile size: the mask
-    exists only on the GPU (`MaskPattern`), so the checks are size-independent ones: V = 1 gives 1 everywhere, and a few
-    rows are recomputed directly from their window."""
+    """Sequences longer than any BASELINE configuration, one of them not a multiple of any tile size, one of a million
+    rows: the mask never exists (`MaskPattern`: metadata in closed form), so the checks are size-independent ones:
+    V = 1 gives 1 everywhere, and a few rows are recomputed directly from their window."""
     g = torch.Generator().manual_seed(L)
     q = torch.randn(1, 1, L, d, generator=g).to(dtype).to(dev)
     k = torch.randn(1, 1, L, d, generator=g).to(dtype).to(dev)
