@@ -165,7 +165,8 @@ int splat_attention_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl,
  *
  * splat_attention_plan_bytes: size of the plan for these segments and L rows (0 for invalid arguments);
  *   host-only arithmetic, reads nothing on the device.
- * splat_attention_plan: fill `plan` (device memory, 16-byte aligned, plan_bytes >= the size above).
+ * splat_attention_plan: fill `plan` (device memory, 16-byte aligned, plan_bytes >= the size above); the
+ *   work is enqueued on `stream`, and forwards that use the plan must be ordered after it.
  * splat_attention_fwd_planned: as splat_attention_fwd, with the plan of the same segments and L; results
  *   are bit-identical to splat_attention_fwd.  A plan built from other segments or another L gives
  *   undefined results (only its size is checked). */
