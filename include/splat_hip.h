@@ -180,6 +180,26 @@ int splat_attention_fwd_planned(const void* q, int64_t q_sb, int64_t q_sh, int64
                                 int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t d, float scale,
                                 int32_t dtype, const void* plan, int64_t plan_bytes, void* stream);
 
+/* ---- backward pass (the reference has none: r_attention.py:77-100 is forward only) ----
+ * With S~ the compressed scores, P~ = softmax(S~), O = P~ . V:
+ *   dP~ = splat_sddmm(x = dO, y = V viewed as [d, L])           dQ = splat_spmm(p = dS~, v = K)
+ *   dS~ = splat_softmax_bwd(P~, dP~)                              dV = splat_spmm(P~ transposed, dO)
+ *                                                                 dK = splat_spmm(dS~ transposed, Q)
+ * where "transposed" is the compressed matrix in the layout of the ACSR of the transposed mask
+ * (splat_acsr_build on mask^T, whose rows are affine for every pattern above), produced by
+ * splat_compressed_transpose, and the last two products run with that ACSR.
+ *
+ * splat_softmax_bwd: ds[r, s] = p[r, s] * (dp[r, s] - sum_s' p[r, s'] dp[r, s']) * scale over the live slots of
+ *   each row; [BH, L, T] contiguous, one dtype; ds may alias dp; dead slots are not touched.
+ * splat_compressed_transpose: dst[bh, j, t] = src[bh, i(j, t), s(i, j)]: segment k of `segs_t` must be the ACSR of
+ *   the transpose of segment k of `segs`; src [BH, L, T], dst [BH, Lt, Tt] contiguous, distinct, one dtype. */
+int splat_softmax_bwd(const void* p, const void* dp, void* ds, const splat_acsr_seg* segs /* host */,
+                      int32_t n_seg, int64_t BH, int32_t L, int32_t T, float scale, int32_t dtype,
+                      void* stream);
+int splat_compressed_transpose(const void* src, void* dst, const splat_acsr_seg* segs /* host */,
+                               const splat_acsr_seg* segs_t /* host */, int32_t n_seg, int64_t BH,
+                               int32_t L, int32_t T, int32_t Lt, int32_t Tt, int32_t dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -362,3 +362,38 @@ def make_inputs(cfg_seed: int, B: int, H: int, L: int, d: int, dtype: torch.dtyp
     k = torch.randn(B, H, L, d, generator=g, dtype=torch.float32) * mul
     v = torch.randn(B, H, L, d, generator=g, dtype=torch.float32) * mul
     return q.to(dtype), k.to(dtype), v.to(dtype)
+
+
+# ----------------------------------------------------------------------------------------------
+# Backward pass.  The reference has none (r_attention.py:77-100 is forward only); these are the textbook gradients of
+# dense masked attention, in two independent forms that tests/test_oracle_numerics.py checks against each other and
+# against finite differences.
+# ----------------------------------------------------------------------------------------------
+
+
+def dense_masked_attention_grads(q, kT, v, mask, scale: float, grad_out):
+    """(dq, dk, dv) by reverse-mode differentiation of :func:`dense_masked_attention` in fp32."""
+    q32 = q.detach().float().requires_grad_(True)
+    k32 = kT.detach().float().transpose(2, 3).contiguous().requires_grad_(True)
+    v32 = v.detach().float().requires_grad_(True)
+    out = dense_masked_attention(q32, k32.transpose(2, 3), v32, mask, scale)
+    out.backward(grad_out.float())
+    return q32.grad, k32.grad, v32.grad
+
+
+def dense_masked_attention_grads_explicit(q, kT, v, mask, scale: float, grad_out):
+    """The same gradients from the closed formulas: dV = P^T dO, dP = dO V^T, dS = P o (dP - rowsum(P o dP)) * scale,
+    dQ = dS K, dK = dS^T Q."""
+    m = torch.as_tensor(np.asarray(mask) != 0)
+    q32, k32, v32, g = q.float(), kT.float().transpose(2, 3), v.float(), grad_out.float()
+    s = (q32 @ k32.transpose(2, 3)) * scale
+    s = s.masked_fill(~m, float("-inf"))
+    mx = s.amax(dim=-1, keepdim=True)
+    mx = torch.where(torch.isfinite(mx), mx, torch.zeros_like(mx))
+    e = torch.exp(s - mx)
+    den = e.sum(dim=-1, keepdim=True)
+    p = torch.where(den > 0, e / den, torch.zeros_like(e))
+    dv = p.transpose(2, 3) @ g
+    dp = g @ v32.transpose(2, 3)
+    ds = p * (dp - (p * dp).sum(dim=-1, keepdim=True)) * scale
+    return ds @ k32, ds.transpose(2, 3) @ q32, dv

@@ -1,0 +1,87 @@
+"""Backward pass (absent from the reference) against the oracle's dense gradients, and its two own kernels against
+their definitions on the compressed layout."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import splat_oracle as O
+import acsr_helpers as A
+from r_attention import RegularAttention, attention_with_grad
+from r_backward import compressed_transpose_launcher, softmax_backward_launcher, transposed_segments
+
+pytestmark = pytest.mark.gpu
+
+# Gradients pass through two 16-bit compressed matrices (probabilities and dS) before the last products: the bounds
+# below are this build's own (the reference states none), about 4x what was measured on these inputs.
+TOL = {torch.float32: 5e-5, torch.float16: 1.5e-2, torch.bfloat16: 8e-2}
+
+
+def _cases():
+    return [
+        ("causal window", lambda: A.causal_windowed_pattern(300, 40), lambda: O.create_causal_windowed_mask(300, 40), 300),
+        ("window", lambda: A.windowed_pattern(257, 33), lambda: O.create_windowed_mask(257, 33), 257),
+        ("blocked", lambda: A.blocked_pattern(256, 64), lambda: O.create_blocked_mask(256, 64), 256),
+        ("dilated", lambda: A.dilated_pattern(320, 32, 3), lambda: O.create_dilated_mask(320, 32, 3), 320),
+        ("strided, two segments", lambda: A.strided_patterns(384, 32, 16),
+         lambda: sum(O.create_strided_segment_masks(384, 32, 16)), 384),
+    ]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", _cases(), ids=lambda c: c[0])
+def test_gradients_against_dense_attention(dev, case, dtype):
+    _, make, dense, L = case
+    B, H, d = 1, 2, 64
+    scale = d ** -0.5
+    q, k, v = O.make_inputs(L, B, H, L, d, dtype)
+    go = O.make_inputs(L + 1, B, H, L, d, dtype)[0]
+    want = O.dense_masked_attention_grads(q, k.transpose(2, 3), v, np.asarray(dense()), scale, go)
+    attn = RegularAttention(B, L, H, d, make(), 16, 16, dev, dtype, scale=scale)
+    qd, kd, vd = [t.to(dev) for t in (q, k, v)]
+    got = attn.backward_pass([qd, kd.transpose(2, 3), vd], go.to(dev))
+    for name, g, w in zip(("dq", "dk", "dv"), got, want):
+        assert float((g.float().cpu() - w).abs().max()) <= TOL[dtype], name
+    # the same through autograd, K given as a contiguous [B, H, d, L] tensor underneath
+    qa, ka, va = [t.clone().requires_grad_(True) for t in (qd, kd, vd)]
+    out = attention_with_grad(qa, ka, va, attn)
+    (out.float() * go.to(dev).float()).sum().backward()
+    for name, g, w in zip(("dq", "dk", "dv"), (qa.grad, ka.grad, va.grad), want):
+        assert float((g.float().cpu() - w).abs().max()) <= TOL[dtype], name
+
+
+def test_softmax_backward_on_compressed_rows(dev):
+    L = 200
+    acsr = O.create_acsr(O.create_causal_windowed_mask(L, 30), 16)
+    segs = A.create_acsr_segments([A.causal_windowed_pattern(L, 30)], 16, dev)
+    T = segs.T
+    g = torch.Generator().manual_seed(0)
+    p = torch.rand(2, 3, L, T, generator=g)
+    dp = torch.randn(2, 3, L, T, generator=g)
+    valid = torch.from_numpy(O.slot_columns(acsr)[1])
+    pm = torch.where(valid, p, torch.zeros_like(p))
+    want = pm * (dp - (pm * dp).sum(-1, keepdim=True)) * 0.7
+    ds = torch.full_like(p, 5.0).to(dev)
+    softmax_backward_launcher(p.to(dev), dp.to(dev), ds, segs, 0.7)
+    got = ds.cpu()
+    assert float((got - want)[valid.expand_as(got)].abs().max()) <= 1e-5
+    assert torch.all(got[~valid.expand_as(got)] == 5.0)  # dead slots untouched
+
+
+@pytest.mark.parametrize("make,dense", [
+    (lambda: [A.dilated_pattern(150, 16, 3)], lambda: [O.create_dilated_mask(150, 16, 3)]),
+    (lambda: A.strided_patterns(200, 16, 8), lambda: O.create_strided_segment_masks(200, 16, 8))])
+def test_compressed_transpose(dev, make, dense):
+    masks, dms = make(), dense()
+    L = dms[0].shape[0]
+    segs = A.create_acsr_segments(masks, 16, dev)
+    segs_t = transposed_segments(masks, 16, dev)
+    g = torch.Generator().manual_seed(1)
+    full = torch.randn(1, 2, L, L, generator=g)
+    # (rows with a single live column keep that column only in the first-column side channel)
+    src = torch.cat([O.compress(full, O.create_acsr(m, 16), first_col=O.row_extents(m)[0]) for m in dms], dim=-1)
+    want = torch.cat([O.compress(full.transpose(2, 3).contiguous(), O.create_acsr(m.T.copy(), 16),
+                                 first_col=O.row_extents(m.T.copy())[0]) for m in dms], dim=-1)
+    dst = torch.zeros(1, 2, L, segs_t.T).to(dev)
+    compressed_transpose_launcher(src.to(dev), dst, segs, segs_t)
+    assert src.shape[-1] == segs.T and want.shape[-1] == segs_t.T
+    assert torch.equal(dst.cpu(), want)

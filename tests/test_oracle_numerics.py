@@ -106,3 +106,26 @@ def test_two_segments_equal_union_mask():
     T0 = acsrs[0][5]
     out = O.spmm(p[..., :T0], v, acsrs[0], first_col=firsts[0]) + O.spmm(p[..., T0:], v, acsrs[1], first_col=firsts[1])
     assert torch.allclose(out, ref, atol=1e-5)
+
+
+def test_backward_reverse_mode_equals_closed_formulas_and_finite_differences():
+    """The two statements of the gradients (autograd through the dense forward; dV = P^T dO, dS = P o (dP - rowsum)
+    * scale, dQ = dS K, dK = dS^T Q) agree, and a central difference of the forward along a random direction matches
+    their inner product with that direction."""
+    L, d = 40, 8
+    mask = O.create_windowed_mask(L, 5)
+    mask[7] = 0  # an empty row: zero output, zero gradients through it
+    g = torch.Generator().manual_seed(3)
+    q, k, v, go = [torch.randn(1, 2, L, d, generator=g, dtype=torch.float64) for _ in range(4)]
+    a = O.dense_masked_attention_grads(q, k.transpose(2, 3), v, mask, 0.3, go)
+    b = O.dense_masked_attention_grads_explicit(q, k.transpose(2, 3), v, mask, 0.3, go)
+    for x, y in zip(a, b):
+        assert float((x - y).abs().max()) <= 2e-5
+    dq_, dk_, dv_ = [torch.randn(1, 2, L, d, generator=g, dtype=torch.float64) for _ in range(3)]
+    f = lambda t: float((O.dense_masked_attention((q + t * dq_).float(), (k + t * dk_).float().transpose(2, 3),
+                                                  (v + t * dv_).float(), mask, 0.3).double() * go).sum())
+    h = 1e-2
+    fd = (f(h) - f(-h)) / (2 * h)
+    an = float((a[0].double() * dq_).sum() + (a[1].double() * dk_).sum() + (a[2].double() * dv_).sum())
+    assert abs(fd - an) <= 2e-2 * max(1.0, abs(an))
+    assert float(a[0][0, :, 7].abs().max()) == 0.0

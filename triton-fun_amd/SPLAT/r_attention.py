@@ -126,6 +126,8 @@ class RegularAttention(nn.Module):
         self.rspmm_grid_dim = (-(-head_dim // BLOCK_SIZE_X), -(-seq_length // BLOCK_SIZE_Y), batch * num_heads)
         self._unfused_ready = False
         self._plan = None  # the fused kernel's plan of this mask, built on the first fused forward
+        self._segments_t = None  # ACSR of the transposed mask(s), built on the first backward
+        self._BLOCK_HEIGHT = BLOCK_SIZE_Y
 
     # The two [B, H, L, T] intermediates and the reference's launch geometry exist only for the unfused path.
     def _prepare_unfused(self):
@@ -187,6 +189,37 @@ class RegularAttention(nn.Module):
                        self.span_loop_start, self.span_loop_end, self.acsr_trailing_dim,
                        self.nnzs, self.rspmm_grid_dim, self.BLOCK_SIZE_Y, self.BLOCK_SIZE_X, segments=multi)
         return self.rspmm_output
+
+
+    def backward_pass(self, x, grad_out: torch.Tensor):
+        """Gradients (dq, dk, dv), each [B, H, L, d], of ``forward(x)`` for x = [q, kT, v] and the upstream gradient
+        ``grad_out`` [B, H, L, d].  The ACSR of the transposed mask is built on first use; see ``r_backward``."""
+        from r_backward import attention_backward, transposed_segments
+        q, kT, v = x
+        if self._segments_t is None:
+            masks = self._mask if _is_segment_list(self._mask) else [self._mask]
+            self._segments_t = transposed_segments(masks, self._BLOCK_HEIGHT, self._GPU_ID)
+        return attention_backward(q, kT, v, grad_out, self.segments, self._segments_t, self.scale)
+
+
+class _AttentionFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, attn):
+        ctx.save_for_backward(q, k, v)
+        ctx.attn = attn
+        return attn([q, k.transpose(2, 3), v]).clone()  # the module's buffer is reused by the next call
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        q, k, v = ctx.saved_tensors
+        dq, dk, dv = ctx.attn.backward_pass([q, k.transpose(2, 3), v], grad_out)
+        return dq, dk, dv, None
+
+
+def attention_with_grad(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, attn: RegularAttention) -> torch.Tensor:
+    """``attn([q, k^T, v])`` for q, k, v [B, H, L, d] as a differentiable operation (fused forward, backward from
+    ``RegularAttention.backward_pass``)."""
+    return _AttentionFunction.apply(q, k, v, attn)
 
 
 def unit(q, k, v, w_q, w_k, w_v, attn: RegularAttention):

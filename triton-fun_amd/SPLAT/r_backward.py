@@ -1,0 +1,125 @@
+"""Backward pass of ACSR sparse attention, composed from the forward operators plus two kernels of its own.
+
+The reference stops at the forward (``r_attention.py:77-100``); this module gives the gradients of
+``out = softmax_over_live_columns(scale * q.kT) . v`` with respect to q, k and v.  Everything stays in the compressed
+[B, H, L, T] layout:
+
+    S~  = rsddmm(q, kT) * scale            P~ = rsoftmax(S~)
+    dP~ = rsddmm(dO, v^T)                  dS~ = P~ o (dP~ - rowsum(P~ o dP~)) * scale     (splat_softmax_bwd)
+    dQ  = rspmm(dS~, k)
+    dV  = rspmm(P~ in the layout of the transposed mask's ACSR, dO)
+    dK  = rspmm(dS~ in that layout, q)                                                     (splat_compressed_transpose)
+
+The transposed mask must have affine rows as well, which holds for every closed-form pattern (band, blocked, dilated,
+strided); for arbitrary affine-row masks it need not, and the gradients with respect to k and v would then be wrong.
+"""
+from __future__ import annotations
+
+from typing import Any, Sequence
+
+import numpy as np
+import torch
+
+import _splat_hip as _hip
+from acsr_helpers import ACSRSegments, MaskPattern, create_acsr_segments
+from r_sddmm import rsddmm_launcher
+from r_softmax import rsoftmax_launcher
+from r_spmm import rspmm_launcher
+
+
+def transposed_mask(mask, device: Any) -> torch.Tensor:
+    """mask^T as a contiguous uint8 device tensor (patterns are rasterised on the device)."""
+    dev = _hip.resolve_device(device)
+    if isinstance(mask, MaskPattern):
+        m = mask.device_mask(dev)
+    elif isinstance(mask, torch.Tensor):
+        m = mask.to(device=dev, dtype=torch.uint8)
+    else:
+        m = torch.from_numpy(np.ascontiguousarray(np.asarray(mask), dtype=np.uint8)).to(dev)
+    return m.t().contiguous()
+
+
+def transposed_segments(masks: Sequence, BLOCK_HEIGHT: int, GPU_ID: Any) -> ACSRSegments:
+    """The ACSR of the transpose of every segment mask, in the same order."""
+    return create_acsr_segments([transposed_mask(m, GPU_ID) for m in masks], BLOCK_HEIGHT, GPU_ID)
+
+
+def softmax_backward_launcher(p: torch.Tensor, dp: torch.Tensor, ds: torch.Tensor, segments: ACSRSegments,
+                              scale: float = 1.0) -> torch.Tensor:
+    """ds[.., r, s] = p * (dp - sum over the row's live slots of p * dp) * scale; [B, H, L, T] contiguous tensors of
+    one dtype; ``ds`` may be ``dp``."""
+    for name, t in (("p", p), ("dp", dp), ("ds", ds)):
+        _hip.require_device_tensor(t, name)
+        if t.dim() != 4 or not t.is_contiguous() or tuple(t.shape) != tuple(p.shape) or t.dtype != p.dtype:
+            raise _hip.SplatError(f"{name} must be a contiguous [B, H, L, T] tensor like p")
+    B, H, L, T = p.shape
+    if T != segments.T:
+        raise _hip.SplatError(f"trailing dimension {T} does not match the segments' {segments.T}")
+    dev = p.device
+    arr = _hip.seg_array(segments.seg_args())
+    with torch.cuda.device(dev):
+        rc = _hip.lib().splat_softmax_bwd(p.data_ptr(), dp.data_ptr(), ds.data_ptr(), arr, len(segments), B * H, L, T,
+                                          float(scale), _hip.dtype_code(p.dtype), _hip.stream_ptr(dev))
+    _hip.check(rc, "splat_softmax_bwd")
+    return ds
+
+
+def compressed_transpose_launcher(src: torch.Tensor, dst: torch.Tensor, segments: ACSRSegments,
+                                  segments_t: ACSRSegments) -> torch.Tensor:
+    """src [B, H, L, T] in the layout of ``segments`` -> dst [B, H, Lt, Tt] in the layout of ``segments_t`` (the ACSR
+    of the transposed segment masks): dst[j, t] is the entry of src that sits at (row i(j, t), column j)."""
+    for name, t in (("src", src), ("dst", dst)):
+        _hip.require_device_tensor(t, name)
+        if t.dim() != 4 or not t.is_contiguous():
+            raise _hip.SplatError(f"{name} must be a contiguous 4-D tensor")
+    if src.dtype != dst.dtype or src.shape[:2] != dst.shape[:2] or len(segments) != len(segments_t):
+        raise _hip.SplatError("src and dst must share dtype, batch and heads; both ACSRs the same number of segments")
+    B, H, L, T = src.shape
+    Lt, Tt = dst.shape[2], dst.shape[3]
+    if T != segments.T or Tt != segments_t.T:
+        raise _hip.SplatError("trailing dimensions do not match the segments")
+    dev = src.device
+    a, b = _hip.seg_array(segments.seg_args()), _hip.seg_array(segments_t.seg_args())
+    with torch.cuda.device(dev):
+        rc = _hip.lib().splat_compressed_transpose(src.data_ptr(), dst.data_ptr(), a, b, len(segments), B * H, L, T, Lt, Tt,
+                                                   _hip.dtype_code(src.dtype), _hip.stream_ptr(dev))
+    _hip.check(rc, "splat_compressed_transpose")
+    return dst
+
+
+def _sddmm(x, y, out, segs, scale):
+    rsddmm_launcher(x, y, out, None, None, None, None, segs.T, None, None, None, None, 16, 16, scale=scale, segments=segs)
+
+
+def _spmm(p, v, out, segs):
+    rspmm_launcher(p, v, out, None, None, None, None, None, None, segs.T, None, None, 16, 16, segments=segs)
+
+
+def attention_backward(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor, grad_out: torch.Tensor,
+                       segments: ACSRSegments, segments_t: ACSRSegments, scale: float = 1.0):
+    """(dq, dk, dv), each [B, H, L, d], for out = softmax_over_live_columns(scale * q.kT) . v and the upstream gradient
+    ``grad_out`` [B, H, L, d].  q, v [B, H, L, d]; kT [B, H, d, L] (a view or a copy); one dtype throughout.  The
+    probabilities are recomputed (SDDMM + softmax), as the fused forward never materialises them."""
+    B, H, L, d = q.shape
+    dt, dev = q.dtype, q.device
+    k = kT.transpose(2, 3)
+    if k.stride(3) != 1:
+        k = k.contiguous()
+    grad_out = grad_out.contiguous() if grad_out.stride(3) != 1 else grad_out
+    T, Tt = segments.T, segments_t.T
+    probs = torch.empty((B, H, L, T), dtype=dt, device=dev)
+    _sddmm(q, kT, probs, segments, scale)
+    rsoftmax_launcher(probs, probs, None, None, None, None, T, 0, None, None, 16, segments=segments)
+    dprobs = torch.empty_like(probs)
+    _sddmm(grad_out, v.transpose(2, 3), dprobs, segments, 1.0)
+    softmax_backward_launcher(probs, dprobs, dprobs, segments, scale)  # dprobs now holds dS~
+    dq = torch.empty((B, H, L, d), dtype=dt, device=dev)
+    _spmm(dprobs, k, dq, segments)
+    turned = torch.empty((B, H, L, Tt), dtype=dt, device=dev)
+    compressed_transpose_launcher(probs, turned, segments, segments_t)
+    dv = torch.empty((B, H, L, d), dtype=dt, device=dev)
+    _spmm(turned, grad_out, dv, segments_t)
+    compressed_transpose_launcher(dprobs, turned, segments, segments_t)
+    dk = torch.empty((B, H, L, d), dtype=dt, device=dev)
+    _spmm(turned, q if q.stride(3) == 1 else q.contiguous(), dk, segments_t)
+    return dq, dk, dv
