@@ -197,7 +197,14 @@ def main() -> int:
             if fl:
                 extras[name]["tflops_nnz"] = round(fl / ms / 1e9, 2)
         out["softmax_gbps"] = extras["softmax_cfg4"]["gbps_algorithmic"]
-        del s_buf, p_buf, o_buf, q4, k4, v4
+        del s_buf, p_buf, o_buf
+        # backward pass (not in the reference) at the same shape: nonzero FLOPs = 2.5 x the forward's (five products)
+        attn4 = RegularAttention(B4, L4, H4, d4, pat4, 16, 16, dev, dtype, scale=d4 ** -0.5)
+        g4 = torch.randn_like(q4)
+        _, pr = time_launches(lambda: attn4.backward_pass([q4, k4T, v4], g4), 10, 3)
+        ms = sum(pr) / len(pr)
+        extras["backward_cfg4"] = {"ms": round(ms, 3), "tflops_nnz": round(10 * d4 * nnz4 * B4 * H4 / ms / 1e9, 2)}
+        del attn4, g4, q4, k4, v4
     out["extras"] = extras
 
     if not args.no_cpu:
