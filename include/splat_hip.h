@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define SPLAT_VERSION 200 /* major*10000 + minor*100 + patch; 0.2.0 added the planned forward */
+#define SPLAT_VERSION 300 /* major*10000 + minor*100 + patch; 0.2.0 added the planned forward, 0.3.0 splat_spmm_t */
 
 /* element types of q/k/v/score/output buffers */
 #define SPLAT_F32 0
@@ -183,12 +183,16 @@ int splat_attention_fwd_planned(const void* q, int64_t q_sb, int64_t q_sh, int64
 /* ---- backward pass (the reference has none: r_attention.py:77-100 is forward only) ----
  * With S~ the compressed scores, P~ = softmax(S~), O = P~ . V:
  *   dP~ = splat_sddmm(x = dO, y = V viewed as [d, L])           dQ = splat_spmm(p = dS~, v = K)
- *   dS~ = splat_softmax_bwd(P~, dP~)                              dV = splat_spmm(P~ transposed, dO)
- *                                                                 dK = splat_spmm(dS~ transposed, Q)
- * where "transposed" is the compressed matrix in the layout of the ACSR of the transposed mask
- * (splat_acsr_build on mask^T, whose rows are affine for every pattern above), produced by
- * splat_compressed_transpose, and the last two products run with that ACSR.
+ *   dS~ = splat_softmax_bwd(P~, dP~)                              dV = splat_spmm_t(P~, dO)
+ *                                                                 dK = splat_spmm_t(dS~, Q)
+ * The transposed products also need the ACSR of the transposed mask (splat_acsr_build on mask^T, whose rows are
+ * affine for every pattern above): it says which rows a column meets.  splat_compressed_transpose stores a
+ * compressed matrix in that ACSR's layout, after which splat_spmm with that ACSR gives the same products.
  *
+ * splat_spmm_t: out[b, h, j, :] = sum over the rows i that keep column j of p[b, h, i, slot of j in row i] * x[b, h, i, :];
+ *   p [B*H, L, T] compressed (layout of `segs`), x [B, H, L, n_out] by strides with unit stride along the last
+ *   dimension, out [B*H, Lt, n_out] contiguous; segment k of `segs_t` must be the ACSR of the transpose of segment k
+ *   of `segs` (Lt rows).  fp32 accumulation.
  * splat_softmax_bwd: ds[r, s] = p[r, s] * (dp[r, s] - sum_s' p[r, s'] dp[r, s']) * scale over the live slots of
  *   each row; [BH, L, T] contiguous, one dtype; ds may alias dp; dead slots are not touched.
  * splat_compressed_transpose: dst[bh, j, t] = src[bh, i(j, t), s(i, j)]: segment k of `segs_t` must be the ACSR of
@@ -196,6 +200,10 @@ int splat_attention_fwd_planned(const void* q, int64_t q_sb, int64_t q_sh, int64
 int splat_softmax_bwd(const void* p, const void* dp, void* ds, const splat_acsr_seg* segs /* host */,
                       int32_t n_seg, int64_t BH, int32_t L, int32_t T, float scale, int32_t dtype,
                       void* stream);
+int splat_spmm_t(const void* p, const void* x, int64_t x_sb, int64_t x_sh, int64_t x_sl, void* out,
+                 const splat_acsr_seg* segs /* host */, const splat_acsr_seg* segs_t /* host */, int32_t n_seg,
+                 int32_t B, int32_t H, int32_t L, int32_t Lt, int32_t n_out, int32_t T, int32_t in_dtype,
+                 int32_t out_dtype, void* stream);
 int splat_compressed_transpose(const void* src, void* dst, const splat_acsr_seg* segs /* host */,
                                const splat_acsr_seg* segs_t /* host */, int32_t n_seg, int64_t BH,
                                int32_t L, int32_t T, int32_t Lt, int32_t Tt, int32_t dtype, void* stream);

@@ -1,5 +1,5 @@
-"""Backward pass (absent from the reference) against the oracle's dense gradients, and its two own kernels against
-their definitions on the compressed layout."""
+"""Backward pass (absent from the reference) against the oracle's dense gradients, and its own kernels against their
+definitions on the compressed layout."""
 import numpy as np
 import pytest
 import torch
@@ -7,7 +7,8 @@ import torch
 from oracle import splat_oracle as O
 import acsr_helpers as A
 from r_attention import RegularAttention, attention_with_grad
-from r_backward import compressed_transpose_launcher, softmax_backward_launcher, transposed_segments
+from r_backward import compressed_transpose_launcher, rspmm_t_launcher, softmax_backward_launcher, transposed_segments
+from r_spmm import rspmm_launcher
 
 pytestmark = pytest.mark.gpu
 
@@ -85,3 +86,49 @@ def test_compressed_transpose(dev, make, dense):
     compressed_transpose_launcher(src.to(dev), dst, segs, segs_t)
     assert src.shape[-1] == segs.T and want.shape[-1] == segs_t.T
     assert torch.equal(dst.cpu(), want)
+
+
+@pytest.mark.parametrize("dtype,n_out", [(torch.float32, 64), (torch.float32, 40), (torch.bfloat16, 128), (torch.float16, 24)])
+@pytest.mark.parametrize("make,dense", [
+    (lambda: [A.causal_windowed_pattern(300, 70)], lambda: [O.create_causal_windowed_mask(300, 70)]),
+    (lambda: [A.blocked_pattern(256, 64)], lambda: [O.create_blocked_mask(256, 64)]),
+    (lambda: [A.dilated_pattern(150, 16, 3)], lambda: [O.create_dilated_mask(150, 16, 3)]),
+    (lambda: A.strided_patterns(200, 16, 8), lambda: O.create_strided_segment_masks(200, 16, 8))],
+    ids=["causal window", "blocked", "dilated", "strided"])
+def test_transposed_product(dev, make, dense, dtype, n_out):
+    """out = (the compressed matrix as a dense one)^T . x, against that product in float64; and the same product from the
+    stored transpose (splat_compressed_transpose + splat_spmm)."""
+    masks, dms = make(), dense()
+    L = dms[0].shape[0]
+    segs = A.create_acsr_segments(masks, 16, dev)
+    segs_t = transposed_segments(masks, 16, dev)
+    g = torch.Generator().manual_seed(2)
+    full = torch.randn(2, 2, L, L, generator=g).to(dtype)
+    x = torch.randn(2, 2, L, n_out, generator=g).to(dtype)
+    src = torch.cat([O.compress(full, O.create_acsr(m, 16), first_col=O.row_extents(m)[0]) for m in dms], dim=-1)
+    live = torch.from_numpy(sum(np.asarray(m, dtype=np.int64) for m in dms) > 0)
+    want = (torch.where(live, full.double(), torch.zeros((), dtype=torch.float64)).transpose(2, 3) @ x.double())
+    out = torch.full((2, 2, L, n_out), 7.0, dtype=dtype).to(dev)
+    rspmm_t_launcher(src.to(dev), x.to(dev), out, segs, segs_t)
+    tol = {torch.float32: 2e-4, torch.float16: 6e-2, torch.bfloat16: 4e-1}[dtype]  # one rounding of sums of ~70 products
+    assert float((out.double().cpu() - want).abs().max()) <= tol
+    turned = torch.zeros(2, 2, L, segs_t.T, dtype=dtype).to(dev)
+    compressed_transpose_launcher(src.to(dev), turned, segs, segs_t)
+    out2 = torch.empty_like(out)
+    rspmm_launcher(turned, x.to(dev), out2, None, None, None, None, None, None, segs_t.T, None, None, 16, 16, segments=segs_t)
+    assert float((out.double() - out2.double()).abs().max().cpu()) <= tol
+
+
+def test_transposed_product_arguments_are_checked(dev):
+    segs = A.create_acsr_segments([A.causal_windowed_pattern(64, 8)], 16, dev)
+    segs_t = transposed_segments([A.causal_windowed_pattern(64, 8)], 16, dev)
+    p = torch.zeros(1, 1, 64, segs.T, device=dev)
+    x = torch.zeros(1, 1, 64, 32, device=dev)
+    out = torch.zeros(1, 1, 64, 32, device=dev)
+    from _splat_hip import SplatError
+    with pytest.raises(SplatError):
+        rspmm_t_launcher(p[..., :-1], x, out, segs, segs_t)
+    with pytest.raises(SplatError):
+        rspmm_t_launcher(p, x.transpose(2, 3), out, segs, segs_t)
+    with pytest.raises(SplatError):
+        rspmm_t_launcher(p, x[..., :16], out, segs, segs_t)

@@ -7,11 +7,13 @@ The reference stops at the forward (``r_attention.py:77-100``); this module give
     S~  = rsddmm(q, kT) * scale            P~ = rsoftmax(S~)
     dP~ = rsddmm(dO, v^T)                  dS~ = P~ o (dP~ - rowsum(P~ o dP~)) * scale     (splat_softmax_bwd)
     dQ  = rspmm(dS~, k)
-    dV  = rspmm(P~ in the layout of the transposed mask's ACSR, dO)
-    dK  = rspmm(dS~ in that layout, q)                                                     (splat_compressed_transpose)
+    dV  = P~^T . dO                        dK = dS~^T . q                                   (splat_spmm_t)
 
-The transposed mask must have affine rows as well, which holds for every closed-form pattern (band, blocked, dilated,
-strided); for arbitrary affine-row masks it need not, and the gradients with respect to k and v would then be wrong.
+The transposed products read the compressed matrices as they are and take the ACSR of the transposed mask to know
+which rows a column meets (``compressed_transpose_launcher`` can also store a matrix in that ACSR's layout, after which
+``rspmm_launcher`` gives the same products).  The transposed mask must have affine rows as well, which holds for every
+closed-form pattern (band, blocked, dilated, strided); for arbitrary affine-row masks it need not, and the gradients
+with respect to k and v would then be wrong.
 """
 from __future__ import annotations
 
@@ -87,6 +89,36 @@ def compressed_transpose_launcher(src: torch.Tensor, dst: torch.Tensor, segments
     return dst
 
 
+def rspmm_t_launcher(p: torch.Tensor, x: torch.Tensor, out: torch.Tensor, segments: ACSRSegments,
+                     segments_t: ACSRSegments) -> torch.Tensor:
+    """out[.., j, :] = sum over the rows i that keep column j of p[.., i, slot of j in row i] * x[.., i, :], i.e. the
+    product with the transposed compressed matrix: p [B, H, L, T] contiguous in the layout of ``segments``, x
+    [B, H, L, n] with unit stride along n, out [B, H, Lt, n] contiguous; ``segments_t`` the ACSR of the transposed
+    segment masks."""
+    for name, t in (("p", p), ("x", x), ("out", out)):
+        _hip.require_device_tensor(t, name)
+        if t.dim() != 4:
+            raise _hip.SplatError(f"{name} must be a 4-D tensor")
+    if not p.is_contiguous() or not out.is_contiguous():
+        raise _hip.SplatError("p and out must be contiguous")
+    if x.stride(3) != 1:
+        raise _hip.SplatError("x needs unit stride along its last dimension")
+    B, H, L, T = p.shape
+    Lt, n = out.shape[2], out.shape[3]
+    if tuple(x.shape) != (B, H, L, n) or tuple(out.shape[:2]) != (B, H) or x.dtype != p.dtype:
+        raise _hip.SplatError(f"shapes do not fit: p {tuple(p.shape)}, x {tuple(x.shape)}, out {tuple(out.shape)}")
+    if T != segments.T or len(segments) != len(segments_t):
+        raise _hip.SplatError("the segments do not fit p (trailing dimension, number of segments)")
+    dev = p.device
+    a, b = _hip.seg_array(segments.seg_args()), _hip.seg_array(segments_t.seg_args())
+    xs = x.stride()
+    with torch.cuda.device(dev):
+        rc = _hip.lib().splat_spmm_t(p.data_ptr(), x.data_ptr(), xs[0], xs[1], xs[2], out.data_ptr(), a, b, len(segments), B, H,
+                                     L, Lt, n, T, _hip.dtype_code(p.dtype), _hip.dtype_code(out.dtype), _hip.stream_ptr(dev))
+    _hip.check(rc, "splat_spmm_t")
+    return out
+
+
 def _sddmm(x, y, out, segs, scale):
     rsddmm_launcher(x, y, out, None, None, None, None, segs.T, None, None, None, None, 16, 16, scale=scale, segments=segs)
 
@@ -106,7 +138,7 @@ def attention_backward(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor, grad_
     if k.stride(3) != 1:
         k = k.contiguous()
     grad_out = grad_out.contiguous() if grad_out.stride(3) != 1 else grad_out
-    T, Tt = segments.T, segments_t.T
+    T = segments.T
     probs = torch.empty((B, H, L, T), dtype=dt, device=dev)
     _sddmm(q, kT, probs, segments, scale)
     rsoftmax_launcher(probs, probs, None, None, None, None, T, 0, None, None, 16, segments=segments)
@@ -115,11 +147,8 @@ def attention_backward(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor, grad_
     softmax_backward_launcher(probs, dprobs, dprobs, segments, scale)  # dprobs now holds dS~
     dq = torch.empty((B, H, L, d), dtype=dt, device=dev)
     _spmm(dprobs, k, dq, segments)
-    turned = torch.empty((B, H, L, Tt), dtype=dt, device=dev)
-    compressed_transpose_launcher(probs, turned, segments, segments_t)
     dv = torch.empty((B, H, L, d), dtype=dt, device=dev)
-    _spmm(turned, grad_out, dv, segments_t)
-    compressed_transpose_launcher(dprobs, turned, segments, segments_t)
+    rspmm_t_launcher(probs, grad_out, dv, segments, segments_t)
     dk = torch.empty((B, H, L, d), dtype=dt, device=dev)
-    _spmm(turned, q if q.stride(3) == 1 else q.contiguous(), dk, segments_t)
+    rspmm_t_launcher(dprobs, q if q.stride(3) == 1 else q.contiguous(), dk, segments, segments_t)
     return dq, dk, dv

@@ -191,6 +191,30 @@ __device__ __forceinline__ int win_slot(const RowWin& w, int j) {
     return (w.lin == 1) ? u : u / w.lin;
 }
 
+// The entries of one compressed row at the 8 consecutive positions jj..jj+7 of a dense walk, zero where the row has no
+// slot (`row` points at the row's first slot of the segment).  Two integer divisions per call: the first live position
+// and its slot; the following ones are `lin` positions and one slot further each.
+template <typename V, typename T>
+__device__ __forceinline__ V gather_affine8(const T* row, const RowWin& w, int jj) {
+    V v;
+    const int u0 = jj - w.lo;
+    int r = u0 % w.lin;
+    if (r < 0) r += w.lin;
+    int next = (r == 0) ? 0 : w.lin - r;  // offset of the first position congruent to the row's first column
+    int slot = (u0 + next) / w.lin;       // exact; negative before the row's first column
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const bool hit = (e == next);
+        const bool live = hit && (unsigned)(u0 + e) < (unsigned)w.cnt;
+        v[e] = live ? row[slot] : (T)0.f;
+        if (hit) {
+            next += w.lin;
+            ++slot;
+        }
+    }
+    return v;
+}
+
 // Width of a wavefront's rows in tile positions: the tiles before lo_min / from hi_max on hold nothing for it, the
 // tiles from lo_max on and up to hi_min need no mask.
 struct WaveSpan {

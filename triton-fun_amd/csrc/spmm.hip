@@ -26,6 +26,59 @@ struct SpmmParams {
     int row_stride;
 };
 
+// Write a wavefront's 32 x (32*DVT) block of accumulators to rows r0 + rs*(32*wave + k) of out[bh] ([rows, n_out],
+// columns col0..).  An accumulator register holds one row's value at column lane%32: stored directly, a wavefront
+// instruction writes 32 consecutive elements of two rows.  When rows of the output can take 16-byte stores (`wide`), each
+// 32 x 32 tile is instead converted, turned around in the wavefront's staging area `stg` (32 rows of 144 bytes at
+// least) and written as 16-byte pieces (8 or 4 per row).
+template <int DVT>
+__device__ __forceinline__ void store_block_rows(const f32x16 (&acc)[DVT], char* stg, void* out, int out_dtype, bool wide,
+                                                 int64_t bh, int n_rows, int n_out, int r0, int rs, int wave, int lane, int col0) {
+    const int lm = lane & 31, g = lane >> 5;
+    const int es_out = (out_dtype == SPLAT_F32) ? 4 : 2;
+    if (wide) {
+        const int row_b = 32 * es_out + 16;  // padded staging row
+        const int cpr = 32 * es_out / 16;     // 16-byte pieces per row
+#pragma unroll
+        for (int dt = 0; dt < DVT; ++dt) {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                char* dst = stg + acc_row(j, g) * row_b + lm * es_out;
+                if (out_dtype == SPLAT_BF16)
+                    *reinterpret_cast<bf16*>(dst) = (bf16)acc[dt][j];
+                else if (out_dtype == SPLAT_F16)
+                    *reinterpret_cast<f16*>(dst) = (f16)acc[dt][j];
+                else
+                    *reinterpret_cast<float*>(dst) = acc[dt][j];
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wavefront's LDS writes are visible to its own reads
+            for (int flat = lane; flat < 32 * cpr; flat += 64) {
+                const int row = flat / cpr, c = flat % cpr;
+                const int r = r0 + rs * (32 * wave + row);
+                const u32x4 val = *reinterpret_cast<const u32x4*>(stg + row * row_b + c * 16);
+                if (r < n_rows) {
+                    char* orow = reinterpret_cast<char*>(out) + ((bh * n_rows + r) * n_out + col0 + 32 * dt) * es_out;
+                    *reinterpret_cast<u32x4*>(orow + c * 16) = val;
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // reads done before the next tile overwrites the staging
+        }
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const int r = r0 + rs * (32 * wave + acc_row(j, g));
+        if (r < n_rows) {
+            const int64_t base = (bh * n_rows + r) * n_out;
+#pragma unroll
+            for (int dt = 0; dt < DVT; ++dt) {
+                const int c = col0 + 32 * dt + lm;
+                if (c < n_out) store_as(out, base + c, acc[dt][j], out_dtype);
+            }
+        }
+    }
+}
+
 template <typename T, int DVT>
 __global__ __launch_bounds__(256, 2) void spmm_kernel(const SpmmParams p) {
     constexpr int ES = sizeof(T);
@@ -39,6 +92,7 @@ __global__ __launch_bounds__(256, 2) void spmm_kernel(const SpmmParams p) {
     constexpr int P_ROW = kBN * ES + 16;    // bytes per row of the probability staging tile
     __shared__ __attribute__((aligned(16))) char s_v[V_ROW * kBN];
     __shared__ __attribute__((aligned(16))) char s_p[4][32 * P_ROW];
+    static_assert(P_ROW >= 32 * 4 + 16, "the staging area also holds a 32 x 32 fp32 tile of the output");
     __shared__ SegPlan s_plan[SPLAT_MAX_SEGMENTS];
     __shared__ SegPtrs s_seg[SPLAT_MAX_SEGMENTS];
     __shared__ PlanScratch<BM> s_ps;
@@ -137,8 +191,7 @@ __global__ __launch_bounds__(256, 2) void spmm_kernel(const SpmmParams p) {
                     v[e] = ((unsigned)(u + e) < (unsigned)w.cnt) ? x : (T)0.f;
                 }
             } else {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) v[e] = win_live(w, jj + e) ? wrow[c][win_slot(w, jj + e)] : (T)0.f;
+                v = gather_affine8<vec8>(wrow[c], w, jj);
             }
             return v;
         };
@@ -185,56 +238,9 @@ __global__ __launch_bounds__(256, 2) void spmm_kernel(const SpmmParams p) {
         }
     }
 
-    // ---- epilogue ----
-    // An accumulator register holds one row's value at column lm: stored directly, a wavefront instruction writes 32
-    // consecutive elements of two rows.  When rows of the output can take 16-byte stores, each 32 x 32 tile is instead
-    // converted, turned around in the wavefront's staging area and written as 16-byte pieces (8 or 4 per row).
     __syncthreads();  // every wavefront is done with the staging areas and the V tile
-    const int es_out = (p.out_dtype == SPLAT_F32) ? 4 : 2;
-    const bool wide = p.out_vec && (col0 + 32 * DVT <= p.n_out);
-    if (wide) {
-        char* stg = s_p[wave];
-        static_assert(32 * P_ROW >= 32 * (32 * 4 + 16), "staging area holds a 32 x 32 fp32 tile");
-        const int row_b = 32 * es_out + 16;  // padded staging row
-        const int cpr = 32 * es_out / 16;     // 16-byte pieces per row
-#pragma unroll
-        for (int dt = 0; dt < DVT; ++dt) {
-#pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                char* dst = stg + acc_row(j, g) * row_b + lm * es_out;
-                if (p.out_dtype == SPLAT_BF16)
-                    *reinterpret_cast<bf16*>(dst) = (bf16)acc[dt][j];
-                else if (p.out_dtype == SPLAT_F16)
-                    *reinterpret_cast<f16*>(dst) = (f16)acc[dt][j];
-                else
-                    *reinterpret_cast<float*>(dst) = acc[dt][j];
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wavefront's LDS writes are visible to its own reads
-            for (int flat = lane; flat < 32 * cpr; flat += 64) {
-                const int row = flat / cpr, c = flat % cpr;
-                const int r = r0 + rs * (32 * wave + row);
-                const u32x4 val = *reinterpret_cast<const u32x4*>(stg + row * row_b + c * 16);
-                if (r < L) {
-                    char* orow = reinterpret_cast<char*>(p.out) + (((int64_t)bh * L + r) * p.n_out + col0 + 32 * dt) * es_out;
-                    *reinterpret_cast<u32x4*>(orow + c * 16) = val;
-                }
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // reads done before the next tile overwrites the staging
-        }
-        return;
-    }
-#pragma unroll
-    for (int j = 0; j < 16; ++j) {
-        const int r = r0 + rs * (32 * wave + acc_row(j, g));
-        if (r < L) {
-            const int64_t base = ((int64_t)bh * L + r) * p.n_out;
-#pragma unroll
-            for (int dt = 0; dt < DVT; ++dt) {
-                const int c = col0 + 32 * dt + lm;
-                if (c < p.n_out) store_as(p.out, base + c, acc[dt][j], p.out_dtype);
-            }
-        }
-    }
+    store_block_rows<DVT>(acc, s_p[wave], p.out, p.out_dtype, p.out_vec && (col0 + 32 * DVT <= p.n_out), bh, L, p.n_out, r0, rs,
+                          wave, lane, col0);
 }
 
 template <typename T>
@@ -253,6 +259,206 @@ static int launch_spmm(SpmmParams p, hipStream_t st) {
     else
         spmm_kernel<T, 1><<<grid, 256, 0, st>>>(p);
     return check_launch("splat_spmm");
+}
+
+
+// ---- transposed product: out[bh, j, :] = sum over the rows i that keep column j of p[bh, i, slot of j in row i] * x[bh, i, :]
+// (the compressed matrix enters transposed without ever being stored that way; the backward pass needs P~^T.dO and
+// dS~^T.Q).  A workgroup owns 128 consecutive columns j of the mask = rows of the output; the rows i that meet them are
+// walked in dense tiles of 64, planned from the ACSR of the transposed mask.  Per tile, row i's stretch of columns
+// j0..j0+127 is read from its compressed row (consecutive slots for unit-step rows) into an LDS tile [i][j], zero where
+// row i does not keep the column, and read back as the A operand with the transposing LDS read, exactly as the x tile
+// [i][feature] is read as the B operand.
+struct SpmmTParams {
+    const void* p;   // [BH, L, T] compressed, rows of the mask
+    const void* x;   // [B, H, L, n_out] by strides, unit stride along the features
+    void* out;       // [BH, Lt, n_out] contiguous
+    int64_t x_sb, x_sh, x_sl;
+    int B, H, L, Lt, n_out, T;
+    int out_dtype, out_vec, x_vec;
+    int n_seg;
+    SegPtrs seg[SPLAT_MAX_SEGMENTS];    // the mask: which columns row i keeps, and where
+    SegPtrs seg_t[SPLAT_MAX_SEGMENTS];  // the transposed mask: which rows column j meets
+    int n_row_blocks, total, n_col_chunks;
+};
+
+template <typename T, int DVT>
+__global__ __launch_bounds__(256, 2) void spmm_t_kernel(const SpmmTParams p) {
+    constexpr int ES = sizeof(T);
+    constexpr int BM = 128;
+    constexpr int DVC = 32 * DVT;
+    constexpr int X_ROW = DVC * ES + 64;   // bytes per LDS row of the x tile
+    constexpr int PT_ROW = BM * ES + 64;   // bytes per LDS row of the probability tile
+    constexpr int EPC = 16 / ES;
+    constexpr int CR = DVC * ES / 16;
+    constexpr int NCHUNK = kBN * CR;
+    constexpr int CPT = NCHUNK / 256;
+    static_assert(NCHUNK % 256 == 0, "tile shape");
+
+    __shared__ __attribute__((aligned(16))) char s_x[X_ROW * kBN];
+    __shared__ __attribute__((aligned(16))) char s_pt[PT_ROW * kBN];
+    static_assert(PT_ROW * kBN >= 4 * 32 * (32 * 4 + 16), "the probability tile doubles as the output staging areas");
+    __shared__ SegPlan s_plan[SPLAT_MAX_SEGMENTS];
+    __shared__ SegPtrs s_seg[SPLAT_MAX_SEGMENTS];
+    __shared__ PlanScratch<BM> s_ps;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lm = lane & 31, g = lane >> 5;
+
+    const int logical = xcd_remap(blockIdx.x, gridDim.x);
+    if (logical >= p.total) return;
+    const int cchunk = logical % p.n_col_chunks;
+    const int rest = logical / p.n_col_chunks;
+    const int bh = rest / p.n_row_blocks;
+    const int rb = rest % p.n_row_blocks;
+    const int b = bh / p.H, h = bh % p.H;
+    const int j_first = rb * BM;  // first column of the mask (row of the output) of this workgroup
+    const int col0 = cchunk * DVC;
+
+    const T* xb = (const T*)p.x + b * p.x_sb + h * p.x_sh;
+    const T* pb = (const T*)p.p + (int64_t)bh * p.L * p.T;
+
+    if (tid == 0) {
+#pragma unroll
+        for (int k = 0; k < SPLAT_MAX_SEGMENTS; ++k) s_seg[k] = p.seg[k];
+    }
+    // dense walks over consecutive rows i: a row's stretch of 128 columns is then one contiguous run of its slots
+    plan_segments<BM>(p.seg_t, p.n_seg, j_first, 1, p.Lt, false, s_plan, &s_ps, tid);
+
+    f32x16 acc[DVT];
+#pragma unroll
+    for (int dt = 0; dt < DVT; ++dt)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[dt][j] = 0.f;
+
+    // this thread's part of the probability tile: row prow, pieces pq, pq + 4, pq + 8, pq + 12 of 8 columns each
+    const int prow = tid >> 2, pq = tid & 3;
+    const SegPlan cols_of_block = {j_first, 1, 0, 0};  // a row's window in columns relative to j_first, affine test
+
+    for (int sg = 0; sg < p.n_seg; ++sg) {
+        const SegPlan pl = s_plan[sg];
+        if (pl.n_tiles == 0) continue;
+        const SegPtrs src = s_seg[sg];
+
+        // the rows i this wavefront's 32 columns meet, in walk positions
+        const RowWin win = make_row_win(cached_row_map<BM>(&s_ps, sg, 32 * wave + lm), pl);
+        int lmin = win.cnt > 0 ? win.lo : 0x3fffffff;
+        int hmax = win.cnt > 0 ? win.lo + win.cnt : -0x3fffffff;
+        lmin = wave_min_i(lmin);
+        hmax = wave_max_i(hmax);
+
+        auto load_piece = [&](int i0, int k) {
+            const int idx = tid + 256 * k;
+            const int row = idx / CR, cc = idx % CR;
+            const int n = min(max(i0 + row, 0), p.L - 1);
+            const T* srow = xb + (int64_t)n * p.x_sl;
+            const int c = col0 + cc * EPC;
+            u32x4 val = {0u, 0u, 0u, 0u};
+            if (p.x_vec && c + EPC <= p.n_out) {
+                val = *reinterpret_cast<const u32x4*>(srow + c);
+            } else if (c < p.n_out) {
+                T tmp[EPC];
+#pragma unroll
+                for (int e = 0; e < EPC; ++e) tmp[e] = (c + e < p.n_out) ? srow[c + e] : (T)0.f;
+                __builtin_memcpy(&val, tmp, 16);
+            }
+            return val;
+        };
+        // the map of row i0 + prow of the mask; rows that do not exist are empty
+        auto load_map = [&](int i0) {
+            const int i = i0 + prow;
+            RowMap m = {0, 1, 0};
+            if (i >= 0 && i < p.L) m = load_row_map(src, i);
+            return m;
+        };
+        typedef T vec8 __attribute__((ext_vector_type(8)));
+        // piece pq + 4c of row i0 + prow: columns j_first + 8*(pq + 4c) .. + 7
+        auto load_probs = [&](const RowWin& w, int i0, int c) {
+            vec8 v;
+            const T* wrow = pb + (int64_t)min(max(i0 + prow, 0), p.L - 1) * p.T + src.slot_offset;
+            const int jj = 8 * (pq + 4 * c);
+            const int u = jj - w.lo;
+            if (w.lin == 1 && u >= 0 && u + 8 <= w.cnt) {
+                __builtin_memcpy(&v, wrow + u, 8 * ES);  // any alignment
+            } else if (w.lin == 1) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const T x = wrow[min(max(u + e, 0), max(w.cnt - 1, 0))];
+                    v[e] = ((unsigned)(u + e) < (unsigned)w.cnt) ? x : (T)0.f;
+                }
+            } else {
+                v = gather_affine8<vec8>(wrow, w, jj);
+            }
+            return v;
+        };
+
+        u32x4 xreg[CPT];
+#pragma unroll
+        for (int k = 0; k < CPT; ++k) xreg[k] = load_piece(pl.c0, k);
+        RowMap m_next = load_map(pl.c0 + kBN);  // requested two tiles ahead of its use, the probabilities one tile ahead
+        vec8 praw[4];
+        {
+            const RowWin w = make_row_win(load_map(pl.c0), cols_of_block);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) praw[c] = load_probs(w, pl.c0, c);
+        }
+
+        for (int tile = 0; tile < pl.n_tiles; ++tile) {
+            const int i0 = pl.c0 + tile * kBN;
+            const bool skip = (tile * kBN + kBN <= lmin) || (tile * kBN >= hmax);  // wavefront-uniform
+            __syncthreads();  // previous tile fully consumed
+#pragma unroll
+            for (int k = 0; k < CPT; ++k) {
+                const int idx = tid + 256 * k;
+                *reinterpret_cast<u32x4*>(s_x + (idx / CR) * X_ROW + (idx % CR) * 16) = xreg[k];
+            }
+#pragma unroll
+            for (int c = 0; c < 4; ++c) *reinterpret_cast<vec8*>(s_pt + prow * PT_ROW + (pq + 4 * c) * 8 * ES) = praw[c];
+            if (tile + 1 < pl.n_tiles) {
+#pragma unroll
+                for (int k = 0; k < CPT; ++k) xreg[k] = load_piece(i0 + kBN, k);
+                const RowWin w = make_row_win(m_next, cols_of_block);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) praw[c] = load_probs(w, i0 + kBN, c);
+                if (tile + 2 < pl.n_tiles) m_next = load_map(i0 + 2 * kBN);
+            }
+            __syncthreads();
+            if (skip) continue;
+            Frag<T> pf[kBN / 16];
+#pragma unroll
+            for (int t = 0; t < kBN / 16; ++t) pf[t] = lds_frag_cols<T>(s_pt, PT_ROW, 16 * t + 8 * g, 16 * t + 8 * g + 4, 32 * wave, lane);
+#pragma unroll
+            for (int t = 0; t < kBN / 16; ++t) {
+#pragma unroll
+                for (int dt = 0; dt < DVT; ++dt) {
+                    Frag<T> xf = lds_frag_cols<T>(s_x, X_ROW, 16 * t + 8 * g, 16 * t + 8 * g + 4, 32 * dt, lane);
+                    mma32(acc[dt], pf[t], xf);
+                }
+            }
+        }
+    }
+
+    __syncthreads();  // every wavefront is done with the tiles
+    store_block_rows<DVT>(acc, s_pt + wave * (32 * (32 * 4 + 16)), p.out, p.out_dtype, p.out_vec && (col0 + 32 * DVT <= p.n_out), bh,
+                          p.Lt, p.n_out, j_first, 1, wave, lane, col0);
+}
+
+template <typename T>
+static int launch_spmm_t(SpmmTParams p, hipStream_t st) {
+    p.n_row_blocks = (p.Lt + 127) / 128;
+    const int dvt = p.n_out > 64 ? 4 : (p.n_out > 32 ? 2 : 1);
+    p.n_col_chunks = (p.n_out + 32 * dvt - 1) / (32 * dvt);
+    const int64_t total = (int64_t)p.B * p.H * p.n_row_blocks * p.n_col_chunks;
+    if (total > 0x7ffffff0) return fail(SPLAT_E_SHAPE, "splat_spmm_t: problem too large for one launch");
+    p.total = (int)total;
+    const int grid = ((p.total + 7) / 8) * 8;
+    if (dvt == 4)
+        spmm_t_kernel<T, 4><<<grid, 256, 0, st>>>(p);
+    else if (dvt == 2)
+        spmm_t_kernel<T, 2><<<grid, 256, 0, st>>>(p);
+    else
+        spmm_t_kernel<T, 1><<<grid, 256, 0, st>>>(p);
+    return check_launch("splat_spmm_t");
 }
 
 }  // namespace splat
@@ -291,5 +497,39 @@ extern "C" int splat_spmm(const void* pp, const void* v, int64_t v_sb, int64_t v
         case SPLAT_F32: return launch_spmm<float>(p, st);
         case SPLAT_F16: return launch_spmm<f16>(p, st);
         default: return launch_spmm<bf16>(p, st);
+    }
+}
+
+extern "C" int splat_spmm_t(const void* pp, const void* x, int64_t x_sb, int64_t x_sh, int64_t x_sl, void* out,
+                            const splat_acsr_seg* segs, const splat_acsr_seg* segs_t, int32_t n_seg, int32_t B, int32_t H,
+                            int32_t L, int32_t Lt, int32_t n_out, int32_t T, int32_t in_dtype, int32_t out_dtype, void* stream) {
+    const char* who = "splat_spmm_t";
+    if (!pp || !x || !out || !segs || !segs_t) return fail(SPLAT_E_NULL, "%s: null pointer argument", who);
+    if (B <= 0 || H <= 0 || L <= 0 || Lt <= 0 || n_out <= 0 || T <= 0)
+        return fail(SPLAT_E_SHAPE, "%s: need B, H, L, Lt, n_out, T > 0 (got %d, %d, %d, %d, %d, %d)", who, B, H, L, Lt, n_out, T);
+    if (L > (1 << 23) || Lt > (1 << 23)) return fail(SPLAT_E_SHAPE, "%s: L and Lt are limited to 2^23", who);
+    if (out_dtype != SPLAT_F32 && out_dtype != SPLAT_F16 && out_dtype != SPLAT_BF16)
+        return fail(SPLAT_E_DTYPE, "%s: unknown out_dtype %d", who, out_dtype);
+    if (in_dtype != SPLAT_F32 && in_dtype != SPLAT_F16 && in_dtype != SPLAT_BF16)
+        return fail(SPLAT_E_DTYPE, "%s: unknown in_dtype %d", who, in_dtype);
+    if (x_sl < n_out) return fail(SPLAT_E_SHAPE, "%s: x row stride %lld < n_out %d", who, (long long)x_sl, n_out);
+    SpmmTParams p;
+    p.p = pp; p.x = x; p.out = out;
+    p.x_sb = x_sb; p.x_sh = x_sh; p.x_sl = x_sl;
+    p.B = B; p.H = H; p.L = L; p.Lt = Lt; p.n_out = n_out; p.T = T;
+    p.out_dtype = out_dtype;
+    p.n_seg = n_seg;
+    if (int rc = fill_segs(who, segs, n_seg, p.seg, T)) return rc;
+    if (int rc = fill_segs(who, segs_t, n_seg, p.seg_t, -1)) return rc;
+    const int es = in_dtype == SPLAT_F32 ? 4 : 2;
+    const int epc = 16 / es;
+    p.x_vec = ((reinterpret_cast<uintptr_t>(x) & 15) == 0 && x_sb % epc == 0 && x_sh % epc == 0 && x_sl % epc == 0) ? 1 : 0;
+    const int es_out = out_dtype == SPLAT_F32 ? 4 : 2;
+    p.out_vec = ((reinterpret_cast<uintptr_t>(out) & 15) == 0 && ((int64_t)n_out * es_out) % 16 == 0) ? 1 : 0;
+    hipStream_t st = (hipStream_t)stream;
+    switch (in_dtype) {
+        case SPLAT_F32: return launch_spmm_t<float>(p, st);
+        case SPLAT_F16: return launch_spmm_t<f16>(p, st);
+        default: return launch_spmm_t<bf16>(p, st);
     }
 }
