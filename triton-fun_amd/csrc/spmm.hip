@@ -264,11 +264,12 @@ static int launch_spmm(SpmmParams p, hipStream_t st) {
 
 // ---- transposed product: out[bh, j, :] = sum over the rows i that keep column j of p[bh, i, slot of j in row i] * x[bh, i, :]
 // (the compressed matrix enters transposed without ever being stored that way; the backward pass needs P~^T.dO and
-// dS~^T.Q).  A workgroup owns 128 consecutive columns j of the mask = rows of the output; the rows i that meet them are
-// walked in dense tiles of 64, planned from the ACSR of the transposed mask.  Per tile, row i's stretch of columns
-// j0..j0+127 is read from its compressed row (consecutive slots for unit-step rows) into an LDS tile [i][j], zero where
-// row i does not keep the column, and read back as the A operand with the transposing LDS read, exactly as the x tile
-// [i][feature] is read as the B operand.
+// dS~^T.Q).  A workgroup owns 128 columns j = first + rs*m of the mask = rows of the output (rs: the row stride of the
+// transposed mask's ACSR, 1 unless its rows alternate column phase); the rows i that meet them are walked in tiles of 64,
+// planned from that ACSR like any other row block.  Per tile, row i's entries at the block's 128 columns are read from
+// its compressed row (consecutive slots when the row's column step is rs and its phase the block's) into an LDS tile
+// [i][m], zero where row i does not keep the column, and read back as the A operand with the transposing LDS read,
+// exactly as the x tile [i][feature] is read as the B operand.
 struct SpmmTParams {
     const void* p;   // [BH, L, T] compressed, rows of the mask
     const void* x;   // [B, H, L, n_out] by strides, unit stride along the features
@@ -280,7 +281,42 @@ struct SpmmTParams {
     SegPtrs seg[SPLAT_MAX_SEGMENTS];    // the mask: which columns row i keeps, and where
     SegPtrs seg_t[SPLAT_MAX_SEGMENTS];  // the transposed mask: which rows column j meets
     int n_row_blocks, total, n_col_chunks;
+    int row_stride;  // of the transposed mask's ACSR
 };
+
+// Row i's entries seen from a block of columns first + rs*m, m = 0..127.
+struct BlockRow {
+    RowWin w;  // unit step (lin == 1): live iff 0 <= m - lo < cnt, slot m - lo; lin > 1 (rs == 1 only): affine test in
+               // columns as in dense plans; lin == 0: the row fits neither and is tested per entry from its map
+    RowMap m;
+};
+__device__ __forceinline__ BlockRow block_row(const RowMap& m, int first, int rs) {
+    BlockRow b;
+    b.m = m;
+    b.w.lo = 0, b.w.cnt = 0, b.w.lin = 1;
+    if (m.cnt <= 0) return b;
+    const int d0 = m.a - first;
+    if (rs == 1) {
+        b.w.lo = d0;
+        b.w.lin = (m.cnt > 1) ? m.lin : 1;
+        b.w.cnt = b.w.lin * (m.cnt - 1) + 1;
+    } else if ((m.cnt == 1 || m.lin == rs) && d0 % rs == 0) {
+        b.w.lo = d0 / rs;
+        b.w.cnt = m.cnt;
+    } else {
+        b.w.lin = 0;
+    }
+    return b;
+}
+// the general test: entry of the row at column j, or zero
+template <typename T>
+__device__ __forceinline__ T entry_at_column(const T* row, const RowMap& m, int j) {
+    const int u = j - m.a;
+    if (u < 0 || m.cnt <= 0) return (T)0.f;
+    if (u == 0) return row[0];
+    if (m.cnt == 1 || u % m.lin != 0 || u / m.lin >= m.cnt) return (T)0.f;
+    return row[u / m.lin];
+}
 
 template <typename T, int DVT>
 __global__ __launch_bounds__(256, 2) void spmm_t_kernel(const SpmmTParams p) {
@@ -312,7 +348,8 @@ __global__ __launch_bounds__(256, 2) void spmm_t_kernel(const SpmmTParams p) {
     const int bh = rest / p.n_row_blocks;
     const int rb = rest % p.n_row_blocks;
     const int b = bh / p.H, h = bh % p.H;
-    const int j_first = rb * BM;  // first column of the mask (row of the output) of this workgroup
+    const int rs = p.row_stride;
+    const int j_first = block_first_row(rb, BM, rs);  // first column of the mask (row of the output) of this workgroup
     const int col0 = cchunk * DVC;
 
     const T* xb = (const T*)p.x + b * p.x_sb + h * p.x_sh;
@@ -322,8 +359,7 @@ __global__ __launch_bounds__(256, 2) void spmm_t_kernel(const SpmmTParams p) {
 #pragma unroll
         for (int k = 0; k < SPLAT_MAX_SEGMENTS; ++k) s_seg[k] = p.seg[k];
     }
-    // dense walks over consecutive rows i: a row's stretch of 128 columns is then one contiguous run of its slots
-    plan_segments<BM>(p.seg_t, p.n_seg, j_first, 1, p.Lt, false, s_plan, &s_ps, tid);
+    plan_segments<BM>(p.seg_t, p.n_seg, j_first, rs, p.Lt, true, s_plan, &s_ps, tid);
 
     f32x16 acc[DVT];
 #pragma unroll
@@ -333,7 +369,6 @@ __global__ __launch_bounds__(256, 2) void spmm_t_kernel(const SpmmTParams p) {
 
     // this thread's part of the probability tile: row prow, pieces pq, pq + 4, pq + 8, pq + 12 of 8 columns each
     const int prow = tid >> 2, pq = tid & 3;
-    const SegPlan cols_of_block = {j_first, 1, 0, 0};  // a row's window in columns relative to j_first, affine test
 
     for (int sg = 0; sg < p.n_seg; ++sg) {
         const SegPlan pl = s_plan[sg];
@@ -347,10 +382,12 @@ __global__ __launch_bounds__(256, 2) void spmm_t_kernel(const SpmmTParams p) {
         lmin = wave_min_i(lmin);
         hmax = wave_max_i(hmax);
 
-        auto load_piece = [&](int i0, int k) {
+        // walk position -> row of the mask
+        auto row_at = [&](int pos) { return pl.c0 + pl.cs * pos; };
+        auto load_piece = [&](int pos0, int k) {
             const int idx = tid + 256 * k;
             const int row = idx / CR, cc = idx % CR;
-            const int n = min(max(i0 + row, 0), p.L - 1);
+            const int n = min(max(row_at(pos0 + row), 0), p.L - 1);
             const T* srow = xb + (int64_t)n * p.x_sl;
             const int c = col0 + cc * EPC;
             u32x4 val = {0u, 0u, 0u, 0u};
@@ -364,18 +401,19 @@ __global__ __launch_bounds__(256, 2) void spmm_t_kernel(const SpmmTParams p) {
             }
             return val;
         };
-        // the map of row i0 + prow of the mask; rows that do not exist are empty
-        auto load_map = [&](int i0) {
-            const int i = i0 + prow;
+        // the map of the row at walk position pos0 + prow; rows that do not exist are empty
+        auto load_map = [&](int pos0) {
+            const int i = row_at(pos0 + prow);
             RowMap m = {0, 1, 0};
             if (i >= 0 && i < p.L) m = load_row_map(src, i);
             return m;
         };
         typedef T vec8 __attribute__((ext_vector_type(8)));
-        // piece pq + 4c of row i0 + prow: columns j_first + 8*(pq + 4c) .. + 7
-        auto load_probs = [&](const RowWin& w, int i0, int c) {
+        // piece pq + 4c of that row: block columns 8*(pq + 4c) .. + 7
+        auto load_probs = [&](const BlockRow& br, int pos0, int c) {
             vec8 v;
-            const T* wrow = pb + (int64_t)min(max(i0 + prow, 0), p.L - 1) * p.T + src.slot_offset;
+            const RowWin& w = br.w;
+            const T* wrow = pb + (int64_t)min(max(row_at(pos0 + prow), 0), p.L - 1) * p.T + src.slot_offset;
             const int jj = 8 * (pq + 4 * c);
             const int u = jj - w.lo;
             if (w.lin == 1 && u >= 0 && u + 8 <= w.cnt) {
@@ -386,26 +424,29 @@ __global__ __launch_bounds__(256, 2) void spmm_t_kernel(const SpmmTParams p) {
                     const T x = wrow[min(max(u + e, 0), max(w.cnt - 1, 0))];
                     v[e] = ((unsigned)(u + e) < (unsigned)w.cnt) ? x : (T)0.f;
                 }
-            } else {
+            } else if (w.lin > 1) {
                 v = gather_affine8<vec8>(wrow, w, jj);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] = entry_at_column<T>(wrow, br.m, j_first + rs * (jj + e));
             }
             return v;
         };
 
         u32x4 xreg[CPT];
 #pragma unroll
-        for (int k = 0; k < CPT; ++k) xreg[k] = load_piece(pl.c0, k);
-        RowMap m_next = load_map(pl.c0 + kBN);  // requested two tiles ahead of its use, the probabilities one tile ahead
+        for (int k = 0; k < CPT; ++k) xreg[k] = load_piece(0, k);
+        RowMap m_next = load_map(kBN);  // requested two tiles ahead of its use, the probabilities one tile ahead
         vec8 praw[4];
         {
-            const RowWin w = make_row_win(load_map(pl.c0), cols_of_block);
+            const BlockRow br = block_row(load_map(0), j_first, rs);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) praw[c] = load_probs(w, pl.c0, c);
+            for (int c = 0; c < 4; ++c) praw[c] = load_probs(br, 0, c);
         }
 
         for (int tile = 0; tile < pl.n_tiles; ++tile) {
-            const int i0 = pl.c0 + tile * kBN;
-            const bool skip = (tile * kBN + kBN <= lmin) || (tile * kBN >= hmax);  // wavefront-uniform
+            const int pos0 = tile * kBN;
+            const bool skip = (pos0 + kBN <= lmin) || (pos0 >= hmax);  // wavefront-uniform
             __syncthreads();  // previous tile fully consumed
 #pragma unroll
             for (int k = 0; k < CPT; ++k) {
@@ -416,11 +457,11 @@ __global__ __launch_bounds__(256, 2) void spmm_t_kernel(const SpmmTParams p) {
             for (int c = 0; c < 4; ++c) *reinterpret_cast<vec8*>(s_pt + prow * PT_ROW + (pq + 4 * c) * 8 * ES) = praw[c];
             if (tile + 1 < pl.n_tiles) {
 #pragma unroll
-                for (int k = 0; k < CPT; ++k) xreg[k] = load_piece(i0 + kBN, k);
-                const RowWin w = make_row_win(m_next, cols_of_block);
+                for (int k = 0; k < CPT; ++k) xreg[k] = load_piece(pos0 + kBN, k);
+                const BlockRow br = block_row(m_next, j_first, rs);
 #pragma unroll
-                for (int c = 0; c < 4; ++c) praw[c] = load_probs(w, i0 + kBN, c);
-                if (tile + 2 < pl.n_tiles) m_next = load_map(i0 + 2 * kBN);
+                for (int c = 0; c < 4; ++c) praw[c] = load_probs(br, pos0 + kBN, c);
+                if (tile + 2 < pl.n_tiles) m_next = load_map(pos0 + 2 * kBN);
             }
             __syncthreads();
             if (skip) continue;
@@ -440,12 +481,12 @@ __global__ __launch_bounds__(256, 2) void spmm_t_kernel(const SpmmTParams p) {
 
     __syncthreads();  // every wavefront is done with the tiles
     store_block_rows<DVT>(acc, s_pt + wave * (32 * (32 * 4 + 16)), p.out, p.out_dtype, p.out_vec && (col0 + 32 * DVT <= p.n_out), bh,
-                          p.Lt, p.n_out, j_first, 1, wave, lane, col0);
+                          p.Lt, p.n_out, j_first, rs, wave, lane, col0);
 }
 
 template <typename T>
 static int launch_spmm_t(SpmmTParams p, hipStream_t st) {
-    p.n_row_blocks = (p.Lt + 127) / 128;
+    p.n_row_blocks = count_row_blocks(p.Lt, 128, p.row_stride);
     const int dvt = p.n_out > 64 ? 4 : (p.n_out > 32 ? 2 : 1);
     p.n_col_chunks = (p.n_out + 32 * dvt - 1) / (32 * dvt);
     const int64_t total = (int64_t)p.B * p.H * p.n_row_blocks * p.n_col_chunks;
@@ -521,6 +562,7 @@ extern "C" int splat_spmm_t(const void* pp, const void* x, int64_t x_sb, int64_t
     p.n_seg = n_seg;
     if (int rc = fill_segs(who, segs, n_seg, p.seg, T)) return rc;
     if (int rc = fill_segs(who, segs_t, n_seg, p.seg_t, -1)) return rc;
+    p.row_stride = common_row_stride(segs_t, n_seg);
     const int es = in_dtype == SPLAT_F32 ? 4 : 2;
     const int epc = 16 / es;
     p.x_vec = ((reinterpret_cast<uintptr_t>(x) & 15) == 0 && x_sb % epc == 0 && x_sh % epc == 0 && x_sl % epc == 0) ? 1 : 0;
