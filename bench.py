@@ -52,6 +52,20 @@ def time_launches(fn, steps: int, warmup: int):
     return wall_ms, per
 
 
+def time_cold_launches(fn, scratch, steps: int):
+    """Mean per-launch HIP-event duration in ms with a write of `scratch` (larger than L2 + MALL) before every launch,
+    so that no launch finds its operands in a cache."""
+    import torch
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for a, b in evs:
+        scratch.zero_()
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return sum(a.elapsed_time(b) for a, b in evs) / steps
+
+
 def make_inputs(seed: int, B: int, H: int, L: int, d: int, dtype):
     """Seeded q, k, v ~ N(0,1), drawn in fp32 on the host in that order, then cast."""
     import torch
@@ -186,18 +200,26 @@ def main() -> int:
                                                        (1, 1), 16)
         run_spmm = lambda: r_spmm.rspmm_launcher(p_buf, v4, o_buf, acsr[0], acsr[1], acsr[2], acsr[3], acsr[6], acsr[7],
                                                  T4, acsr[4], (1, 1, 1), 16, 16)
+        # the product with the transposed compressed matrix (backward pass only; the reference has no counterpart)
+        import r_backward
+        segs4 = A.create_acsr_segments([pat4], 16, dev)
+        segs4_t = r_backward.transposed_segments([pat4], 16, dev)
+        run_spmm_t = lambda: r_backward.rspmm_t_launcher(p_buf, v4, o_buf, segs4, segs4_t)
+        flush = torch.empty(512 << 20, dtype=torch.uint8, device=dev)  # > L2 + MALL: written before every "cold" launch
         for name, fn, byt, fl in (
                 ("sddmm_cfg4", run_sddmm, (2 * B4 * H4 * L4 * d4 + nnz4 * B4 * H4) * 2, 2 * d4 * nnz4 * B4 * H4),
                 ("softmax_cfg4", run_soft, 2 * nnz4 * B4 * H4 * 2, 0.0),
-                ("spmm_cfg4", run_spmm, (2 * B4 * H4 * L4 * d4 + nnz4 * B4 * H4) * 2, 2 * d4 * nnz4 * B4 * H4)):
+                ("spmm_cfg4", run_spmm, (2 * B4 * H4 * L4 * d4 + nnz4 * B4 * H4) * 2, 2 * d4 * nnz4 * B4 * H4),
+                ("spmm_t_cfg4", run_spmm_t, (2 * B4 * H4 * L4 * d4 + nnz4 * B4 * H4) * 2, 2 * d4 * nnz4 * B4 * H4)):
             _, pr = time_launches(fn, 40, 20)
             ms = sum(pr) / len(pr)
-            extras[name] = {"ms": round(ms, 4), "gbps_algorithmic": round(byt / ms / 1e6, 1),
+            extras[name] = {"ms": round(ms, 4), "ms_caches_flushed": round(time_cold_launches(fn, flush, 20), 4),
+                            "gbps_algorithmic": round(byt / ms / 1e6, 1),
                             "hbm_frac": round(byt / ms / 1e6 / HBM_PEAK_GBPS, 4)}
             if fl:
                 extras[name]["tflops_nnz"] = round(fl / ms / 1e9, 2)
         out["softmax_gbps"] = extras["softmax_cfg4"]["gbps_algorithmic"]
-        del s_buf, p_buf, o_buf
+        del s_buf, p_buf, o_buf, flush
         # backward pass (not in the reference) at the same shape: nonzero FLOPs = 2.5 x the forward's (five products)
         attn4 = RegularAttention(B4, L4, H4, d4, pat4, 16, 16, dev, dtype, scale=d4 ** -0.5)
         g4 = torch.randn_like(q4)
