@@ -10,6 +10,8 @@
 // with a uniform plan these are 8 consecutive compressed slots, one 16-byte store (any alignment).  Dead
 // positions are never stored.  The kernel is bound by the compressed output (HBM), not by MFMA: 2*d flops per
 // 2-4 output bytes.
+#include <algorithm>
+
 #include "acsr_plan.hpp"
 
 namespace splat {
@@ -28,6 +30,7 @@ struct SddmmParams {
     int n_row_blocks, total;
     int q_vec, k_vec;  // 16-byte loads are legal for q / k
     int row_stride;
+    int key_split;  // workgroups per row block: each takes a contiguous share of every segment's tiles
 };
 
 template <typename T>
@@ -99,8 +102,9 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
 
     const int logical = xcd_remap(blockIdx.x, gridDim.x);
     if (logical >= p.total) return;
-    const int bh = logical / p.n_row_blocks;
-    const int rb = logical % p.n_row_blocks;
+    const int ksp = logical % p.key_split;  // this workgroup's share of the row block's tiles
+    const int bh = (logical / p.key_split) / p.n_row_blocks;
+    const int rb = (logical / p.key_split) % p.n_row_blocks;
     const int b = bh / p.H, h = bh % p.H;
     const int rs = p.row_stride;
     const int r0 = block_first_row(rb, BM, rs);
@@ -167,7 +171,10 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
 
     for (int sg = 0; sg < p.n_seg; ++sg) {
         const SegPlan pl = s_plan[sg];
-        if (pl.n_tiles == 0) continue;
+        // output slots of different tiles are disjoint, so the tiles of a row block can be shared out freely
+        const int t_begin = (int)(((int64_t)pl.n_tiles * ksp) / p.key_split);
+        const int t_end = (int)(((int64_t)pl.n_tiles * (ksp + 1)) / p.key_split);
+        if (t_begin >= t_end) continue;
         const int off = s_off[sg];
         // this lane's own row (source of the wavefront's span) and the 2 block rows it writes out
         const RowWin mine = make_row_win(cached_row_map<BM>(&s_ps, sg, 32 * wave + lm), pl);
@@ -188,9 +195,9 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
 
         u32x4 kreg[CPT];
 #pragma unroll
-        for (int i = 0; i < CPT; ++i) kreg[i] = load_piece(pl, 0, 0, i);
+        for (int i = 0; i < CPT; ++i) kreg[i] = load_piece(pl, t_begin * kBN, 0, i);
 
-        for (int tile = 0; tile < pl.n_tiles; ++tile) {
+        for (int tile = t_begin; tile < t_end; ++tile) {
             const int j0 = tile * kBN;
             const bool skip = (j0 + kBN <= lmin) || (j0 >= hmax);  // wavefront-uniform
             f32x16 acc[NT];
@@ -212,7 +219,7 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
                     const bool last_ch = (ch + 1 == n_chunks);
                     const int nj0 = last_ch ? j0 + kBN : j0;
                     const int nkd0 = last_ch ? 0 : kd0 + DC;
-                    if (!(last_ch && tile + 1 == pl.n_tiles)) {
+                    if (!(last_ch && tile + 1 == t_end)) {
 #pragma unroll
                         for (int i = 0; i < CPT; ++i) kreg[i] = load_piece(pl, nj0, nkd0, i);
                     }
@@ -298,7 +305,12 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
 template <typename T>
 static int launch_sddmm(SddmmParams p, bool kt, hipStream_t st) {
     p.n_row_blocks = count_row_blocks(p.L, 128, p.row_stride);
-    p.total = p.B * p.H * p.n_row_blocks;
+    // Few row blocks (one head of a short sequence, the reference's own benchmark shape) would leave most of the 256
+    // compute units idle: share every row block's tiles out over several workgroups then.
+    const int64_t blocks = (int64_t)p.B * p.H * p.n_row_blocks;
+    if (blocks > 0x7ffffff0) return fail(SPLAT_E_SHAPE, "splat_sddmm: problem too large for one launch");
+    p.key_split = blocks >= 512 ? 1 : (int)std::min<int64_t>(32, (768 + blocks - 1) / blocks);
+    p.total = (int)(blocks * p.key_split);
     const int grid = ((p.total + 7) / 8) * 8;
     constexpr int DC = SddmmGeom<T>::DC, KSC = DC / 16;
     const int steps = (p.d + 15) / 16;
