@@ -59,6 +59,8 @@ extern "C" {
 #define SPLAT_MASK_DILATED 3         /* columns i - p0*p1/2 + p1*t, t in [0,p0): p0 = window, p1 = dilation */
 #define SPLAT_MASK_STRIDED_LOCAL 4   /* columns (i-p0, i]: p0 = local width */
 #define SPLAT_MASK_STRIDED_FAR 5     /* columns j <= i-p0 with j % p1 == p1-1: p0 = local width, p1 = stride */
+#define SPLAT_MASK_TRANSPOSED 8      /* flag: the transpose of the pattern it is or-ed onto (row j keeps the rows of the pattern
+                                        that keep column j); the backward pass needs the ACSR of the transposed mask */
 
 /* One affine segment of an ACSR: the five per-row arrays create_acsr returns
  * (acsr_helpers.py:148-152) plus where the segment's slots start in a compressed row. */

@@ -167,6 +167,24 @@ def test_closed_form_pattern_builder_equals_mask_scan(dev, case, BH):
     assert a.T == b.T and a.row_stride == b.row_stride
 
 
+@pytest.mark.parametrize("case", _pattern_cases(), ids=lambda c: f"{c[0]}-{c[1].s}-{c[1].p0}-{c[1].p1}")
+def test_transposed_patterns_in_closed_form(dev, case):
+    """The transposed patterns (the backward pass plans its transposed products from their ACSR): the generator's
+    transposed kind is the transpose of the rasterised pattern, and the closed-form builder on it equals the scan of
+    that transpose, every output array bit for bit."""
+    pat = case[1]
+    dev_t = torch.device(dev)
+    turned = pat.device_mask(dev_t).t().contiguous()
+    assert torch.equal(pat.transposed().device_mask(dev_t), turned)
+    assert pat.transposed().transposed() == pat
+    a = A.build_acsr(pat.transposed(), 16, dev_t)
+    b = A.build_acsr(turned, 16, dev_t)
+    for name in ("dTos_lin", "dTos_trans", "sTod_lin", "sTod_trans", "nnz", "span_start", "span_end"):
+        assert np.array_equal(bits(getattr(a, name)), bits(getattr(b, name))), name
+    assert torch.equal(a.row_first, b.row_first) and torch.equal(a.row_last, b.row_last)
+    assert a.T == b.T and a.row_stride == b.row_stride
+
+
 def test_pattern_builder_needs_no_mask_for_long_sequences(dev):
     """L = 2^20 rows (a 1 TiB mask): metadata in closed form, checked against the per-pattern formulas."""
     L, w = 1 << 20, 512

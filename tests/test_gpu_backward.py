@@ -132,3 +132,25 @@ def test_transposed_product_arguments_are_checked(dev):
         rspmm_t_launcher(p, x.transpose(2, 3), out, segs, segs_t)
     with pytest.raises(SplatError):
         rspmm_t_launcher(p, x[..., :16], out, segs, segs_t)
+
+
+def test_backward_of_a_long_sequence_by_properties(dev):
+    """L = 2^17 (no mask of that size exists anywhere: forward and transposed ACSR both come from the closed forms).
+    With every row of V equal to one vector the output does not depend on q and k, so dq = dk = 0; with dO = 1 the
+    columns of dV sum to the number of rows, because every row of the probabilities sums to 1."""
+    L, d, w = 1 << 17, 64, 256
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(1, 1, L, d, generator=g).to(dtype).to(dev)
+    k = torch.randn(1, 1, L, d, generator=g).to(dtype).to(dev)
+    v0 = torch.randn(d, generator=g).to(dtype)
+    v = v0.expand(1, 1, L, d).contiguous().to(dev)
+    attn = RegularAttention(1, L, 1, d, A.causal_windowed_pattern(L, w - 1), 16, 16, dev, dtype, scale=d ** -0.5)
+    go = torch.ones(1, 1, L, d, dtype=dtype, device=dev)
+    dq, dk, dv = attn.backward_pass([q, k.transpose(2, 3), v], go)
+    # dP~ is the same number in every slot of a row (exactly: the same dot product), so dS~ = P~ (dP~ - sum P~ dP~)
+    # is rounding noise of the 16-bit probabilities
+    assert float(dq.float().abs().max()) <= 0.05 and float(dk.float().abs().max()) <= 0.05
+    col_sums = dv.float().sum(dim=2)  # [1, 1, d]
+    assert float((col_sums / L - 1.0).abs().max()) <= 2e-3
+    assert torch.isfinite(dv.float()).all()

@@ -18,6 +18,7 @@ LIB_PATH = os.environ.get("SPLAT_HIP_LIB") or os.path.normpath(os.path.join(_HER
 SPLAT_F32, SPLAT_F16, SPLAT_BF16 = 0, 1, 2
 MAX_SEGMENTS = 4
 MASK_BLOCKED, MASK_WINDOWED, MASK_CAUSAL_WINDOWED, MASK_DILATED, MASK_STRIDED_LOCAL, MASK_STRIDED_FAR = range(6)
+MASK_TRANSPOSED = 8  # flag or-ed onto a pattern: its transpose
 
 _DTYPES = {torch.float32: SPLAT_F32, torch.float16: SPLAT_F16, torch.bfloat16: SPLAT_BF16}
 

@@ -73,6 +73,10 @@ class MaskPattern:
         _hip.check(rc, "splat_mask_generate")
         return out
 
+    def transposed(self) -> "MaskPattern":
+        """The transposed pattern (row j keeps the rows of this pattern that keep column j), itself closed-form."""
+        return MaskPattern(self.kind ^ _hip.MASK_TRANSPOSED, self.s, self.p0, self.p1)
+
 
 def blocked_pattern(s: int, p: int) -> MaskPattern:
     return MaskPattern(_hip.MASK_BLOCKED, s, p)

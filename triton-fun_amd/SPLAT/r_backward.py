@@ -29,12 +29,13 @@ from r_softmax import rsoftmax_launcher
 from r_spmm import rspmm_launcher
 
 
-def transposed_mask(mask, device: Any) -> torch.Tensor:
-    """mask^T as a contiguous uint8 device tensor (patterns are rasterised on the device)."""
+def transposed_mask(mask, device: Any):
+    """mask^T: the transposed pattern for a closed-form pattern (nothing is rasterised), else a contiguous uint8 device
+    tensor."""
     dev = _hip.resolve_device(device)
     if isinstance(mask, MaskPattern):
-        m = mask.device_mask(dev)
-    elif isinstance(mask, torch.Tensor):
+        return mask.transposed()
+    if isinstance(mask, torch.Tensor):
         m = mask.to(device=dev, dtype=torch.uint8)
     else:
         m = torch.from_numpy(np.ascontiguousarray(np.asarray(mask), dtype=np.uint8)).to(dev)

@@ -246,6 +246,12 @@ __global__ __launch_bounds__(256) void acsr_spans_kernel(const float* __restrict
 }
 
 __device__ __forceinline__ bool mask_pred(int pattern, int64_t i, int64_t j, int64_t p0, int64_t p1) {
+    if (pattern & SPLAT_MASK_TRANSPOSED) {  // entry (i, j) of the transposed pattern is entry (j, i) of the pattern
+        const int64_t t = i;
+        i = j;
+        j = t;
+        pattern &= ~SPLAT_MASK_TRANSPOSED;
+    }
     switch (pattern) {
         case SPLAT_MASK_BLOCKED: {
             if (i < p0) return j < p0;
@@ -309,6 +315,44 @@ __device__ __forceinline__ RowScan pattern_row(int pattern, int64_t i, int64_t s
             count = room < 0 ? 0 : room / p1 + 1;
             break;
         }
+        // ---- rows of the transposed patterns = columns of the patterns: which rows keep column i ----
+        case SPLAT_MASK_TRANSPOSED | SPLAT_MASK_BLOCKED: {
+            // row block b >= 1 keeps column blocks b - 1 and b, row block 0 keeps column block 0: column block c is kept
+            // by row blocks c and c + 1
+            const int64_t c = i / p0;
+            first = c * p0;
+            count = min((c + 2) * p0, s) - first;
+            break;
+        }
+        case SPLAT_MASK_TRANSPOSED | SPLAT_MASK_WINDOWED:
+            first = max((int64_t)0, i - p0);
+            count = min(s - 1, i + p0) - first + 1;
+            break;
+        case SPLAT_MASK_TRANSPOSED | SPLAT_MASK_CAUSAL_WINDOWED:
+            first = i;
+            count = min(s - 1, i + p0) - first + 1;
+            break;
+        case SPLAT_MASK_TRANSPOSED | SPLAT_MASK_STRIDED_LOCAL:
+            first = i;
+            count = min(s - 1, i + p0 - 1) - first + 1;
+            break;
+        case SPLAT_MASK_TRANSPOSED | SPLAT_MASK_DILATED: {
+            // row r keeps column r - h + t * p1, t in [0, p0), h = p0 * p1 / 2: column i is kept by rows i + h - t * p1,
+            // in ascending order base + u * p1, u in [0, p0)
+            const int64_t base = i + (p0 * p1) / 2 - (p0 - 1) * p1;
+            const int64_t u_lo = base < 0 ? (-base + p1 - 1) / p1 : 0;
+            const int64_t room = s - 1 - base;
+            const int64_t u_hi = room < 0 ? -1 : min(p0 - 1, room / p1);
+            step = p1;
+            first = base + u_lo * p1;
+            count = u_hi - u_lo + 1;
+            break;
+        }
+        case SPLAT_MASK_TRANSPOSED | SPLAT_MASK_STRIDED_FAR:
+            // only columns congruent to p1 - 1 are kept, by every row from i + p0 on
+            first = i + p0;
+            count = (i % p1 == p1 - 1) ? s - first : 0;
+            break;
     }
     RowScan r;
     r.init();
@@ -387,10 +431,11 @@ extern "C" int splat_acsr_build(const uint8_t* mask, int64_t rows, int64_t cols,
 
 static int check_pattern(const char* who, int64_t s, int32_t pattern, int64_t p0, int64_t p1) {
     if (s <= 0 || s > (1 << 23)) return fail(SPLAT_E_SHAPE, "%s: need 0 < s <= 2^23 (got %lld)", who, (long long)s);
-    if (pattern < SPLAT_MASK_BLOCKED || pattern > SPLAT_MASK_STRIDED_FAR)
+    const int base = pattern & ~SPLAT_MASK_TRANSPOSED;
+    if (pattern < 0 || base < SPLAT_MASK_BLOCKED || base > SPLAT_MASK_STRIDED_FAR)
         return fail(SPLAT_E_UNSUPPORTED, "%s: unknown pattern %d", who, pattern);
-    const bool needs_p1 = pattern == SPLAT_MASK_DILATED || pattern == SPLAT_MASK_STRIDED_FAR;
-    if (p0 < 0 || (pattern == SPLAT_MASK_BLOCKED && p0 <= 0) || (needs_p1 && p1 <= 0))
+    const bool needs_p1 = base == SPLAT_MASK_DILATED || base == SPLAT_MASK_STRIDED_FAR;
+    if (p0 < 0 || (base == SPLAT_MASK_BLOCKED && p0 <= 0) || (needs_p1 && p1 <= 0))
         return fail(SPLAT_E_SHAPE, "%s: bad pattern parameters p0=%lld p1=%lld", who, (long long)p0, (long long)p1);
     return 0;
 }
@@ -420,11 +465,14 @@ extern "C" int splat_mask_generate(uint8_t* mask, int64_t rows, int64_t cols, in
     if (!mask) return fail(SPLAT_E_NULL, "splat_mask_generate: null mask");
     if (rows <= 0 || cols <= 0 || ld < cols || rows > (1 << 23) || cols > (1 << 23))
         return fail(SPLAT_E_SHAPE, "splat_mask_generate: bad shape rows=%lld cols=%lld ld=%lld", (long long)rows, (long long)cols, (long long)ld);
-    if (pattern < SPLAT_MASK_BLOCKED || pattern > SPLAT_MASK_STRIDED_FAR)
-        return fail(SPLAT_E_UNSUPPORTED, "splat_mask_generate: unknown pattern %d", pattern);
-    const bool needs_p1 = pattern == SPLAT_MASK_DILATED || pattern == SPLAT_MASK_STRIDED_FAR;
-    if (p0 < 0 || (pattern == SPLAT_MASK_BLOCKED && p0 <= 0) || (needs_p1 && p1 <= 0))
-        return fail(SPLAT_E_SHAPE, "splat_mask_generate: bad pattern parameters p0=%lld p1=%lld", (long long)p0, (long long)p1);
+    {
+        const int base = pattern & ~SPLAT_MASK_TRANSPOSED;
+        if (pattern < 0 || base < SPLAT_MASK_BLOCKED || base > SPLAT_MASK_STRIDED_FAR)
+            return fail(SPLAT_E_UNSUPPORTED, "splat_mask_generate: unknown pattern %d", pattern);
+        const bool needs_p1 = base == SPLAT_MASK_DILATED || base == SPLAT_MASK_STRIDED_FAR;
+        if (p0 < 0 || (base == SPLAT_MASK_BLOCKED && p0 <= 0) || (needs_p1 && p1 <= 0))
+            return fail(SPLAT_E_SHAPE, "splat_mask_generate: bad pattern parameters p0=%lld p1=%lld", (long long)p0, (long long)p1);
+    }
     const int vec_ok = ((reinterpret_cast<uintptr_t>(mask) & 15) == 0 && (ld & 15) == 0) ? 1 : 0;
     const int64_t n = rows * ((cols + 15) >> 4);
     mask_generate_kernel<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(mask, (int)rows, (int)cols, ld, pattern, p0, p1, vec_ok);
