@@ -196,6 +196,12 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
         u32x4 kreg[CPT];
 #pragma unroll
         for (int i = 0; i < CPT; ++i) kreg[i] = load_piece(pl, t_begin * kBN, 0, i);
+        // Wait for them here: otherwise the compiler's wait for them sits at the top of the loop below, where on every
+        // later iteration it can only mean "everything outstanding", the previous tile's stores included.
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) asm volatile("" ::"v"(kreg[i]));
+#endif
 
         for (int tile = t_begin; tile < t_end; ++tile) {
             const int j0 = tile * kBN;
@@ -208,7 +214,7 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
 
             for (int ch = 0; ch < n_chunks; ++ch) {
                 const int kd0 = ch * DC;
-                __syncthreads();  // previous chunk fully consumed
+                lds_barrier();  // previous chunk fully consumed (the stores of the previous tile stay in flight)
 #pragma unroll
                 for (int i = 0; i < CPT; ++i) {
                     const int idx = tid + 256 * i;
@@ -224,7 +230,7 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
                         for (int i = 0; i < CPT; ++i) kreg[i] = load_piece(pl, nj0, nkd0, i);
                     }
                 }
-                __syncthreads();
+                lds_barrier();  // the chunk is in LDS (the loads just requested stay in flight)
                 if (skip) continue;
                 auto load_k = [&](int ks, int nt) {
                     if constexpr (KT)

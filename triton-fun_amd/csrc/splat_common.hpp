@@ -126,6 +126,16 @@ __device__ __forceinline__ RowMap load_row_map(const float* sTod_lin, const floa
     return m;
 }
 
+// Workgroup barrier that hands LDS contents over and nothing else: it waits for this wavefront's LDS traffic, not for
+// its global loads and stores.  __syncthreads() waits for both counters, which serialises a kernel whose loads of the
+// next tile or stores of the previous one are meant to stay in flight across the barrier.  (The empty statements keep
+// the compiler from moving memory accesses across the barrier.)
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 // Map a launch-order workgroup id onto a logical id so that logically consecutive ids run on the
 // same XCD (hardware deals consecutive workgroup ids round-robin over the 8 XCDs, each with its own
 // L2).  gridDim.x must be 8 * chunk; ids >= total are idle.
