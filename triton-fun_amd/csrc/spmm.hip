@@ -89,7 +89,10 @@ __global__ __launch_bounds__(256, 2) void spmm_kernel(const SpmmParams p) {
     constexpr int CR = DVC * ES / 16;       // 16-byte chunks per LDS row
     constexpr int NCHUNK = kBN * CR;        // chunks per tile
 
-    constexpr int P_ROW = kBN * ES + 16;    // bytes per row of the probability staging tile
+    // Row of the probability staging tile.  16-bit types: 8 positions of margin on either side of the 64, because a piece
+    // that straddles an end of its row's span is loaded from inside the span and written where it belongs.
+    constexpr int P_MARGIN = (ES == 2) ? 8 : 0;
+    constexpr int P_ROW = (kBN + 2 * P_MARGIN) * ES + 16;
     __shared__ __attribute__((aligned(16))) char s_v[V_ROW * kBN];
     __shared__ __attribute__((aligned(16))) char s_p[4][32 * P_ROW];
     static_assert(P_ROW >= 32 * 4 + 16, "the staging area also holds a 32 x 32 fp32 tile of the output");
@@ -143,10 +146,10 @@ __global__ __launch_bounds__(256, 2) void spmm_kernel(const SpmmParams p) {
             if (r >= L) wr[c].cnt = 0;
             wrow[c] = pb + (int64_t)min(r, L - 1) * p.T + off;
         }
-        int lmin = win.cnt > 0 ? win.lo : 0x3fffffff;
-        int hmax = win.cnt > 0 ? win.lo + win.cnt : -0x3fffffff;
-        lmin = wave_min_i(lmin);
-        hmax = wave_max_i(hmax);
+        // tiles before lmin / from hmax on hold nothing for this wavefront; tiles from lo_max on and up to hi_min lie
+        // inside every one of its rows' spans (never, if a row is empty or not unit-step)
+        const WaveSpan span = wave_span(win, __all(win.lin == 1) != 0);
+        const int lmin = span.lo_min, hmax = span.hi_max;
 
         // one 16-byte piece of the V tile at positions j0.. for this thread's slot i
         auto load_piece = [&](int j0, int i) {
@@ -174,28 +177,63 @@ __global__ __launch_bounds__(256, 2) void spmm_kernel(const SpmmParams p) {
         // A tile's probabilities: lane (row 8c + lane/8 of the wavefront's 32, piece lane%8) fetches 8 consecutive
         // positions, so one instruction reads 8 rows x 64 consecutive slots; the pieces are turned into A fragments
         // (lane = row) through a per-wavefront staging tile.  Requested one tile ahead, like V.
+        // 16-bit types, unit-step rows of at least 8 slots: a piece that straddles an end of the row's span is loaded as
+        // the 8 slots at that end (one vector load like any other, no branch) and lands in the staging tile `shift`
+        // positions off its own place, over zeros; where it overlaps the neighbouring piece both hold the same values.
         typedef T vec8 __attribute__((ext_vector_type(8)));
-        auto load_probs = [&](int j0, int c) {
+        struct Piece {
             vec8 v;
+            int shift;   // positions between the piece's own place and where v belongs
+            int state;   // 0: nothing live (zeros), 1: v is the whole piece, 2: zeros, then v at its shifted place
+        };
+        auto load_probs = [&](int j0, int c) {
+            Piece pc;
+            pc.shift = 0;
+            pc.state = 1;
             const RowWin& w = wr[c];
             const int jj = j0 + 8 * (lane & 7);
             const int u = jj - w.lo;
-            if (w.lin == 1 && u >= 0 && u + 8 <= w.cnt) {
-                __builtin_memcpy(&v, wrow[c] + u, 8 * ES);  // any alignment
+            if ((j0 >= span.lo_max) && (j0 + kBN <= span.hi_min)) {  // wavefront-uniform: the tile is inside every span
+                __builtin_memcpy(&pc.v, wrow[c] + u, 8 * ES);        // any alignment
+            } else if (ES == 2 && w.lin == 1 && w.cnt >= 8) {
+                const bool touches = (u + 8 > 0) && (u < w.cnt);
+                const int uc = min(max(u, 0), w.cnt - 8);
+                pc.shift = uc - u;
+                pc.state = touches ? (pc.shift == 0 ? 1 : 2) : 0;
+                if (touches) __builtin_memcpy(&pc.v, wrow[c] + uc, 8 * ES);  // any alignment
+            } else if (w.lin == 1 && u >= 0 && u + 8 <= w.cnt) {
+                __builtin_memcpy(&pc.v, wrow[c] + u, 8 * ES);  // any alignment
             } else if (w.lin == 1) {
                 // an end of the row's span (or outside it): range test per slot, loads from a clamped slot so that
                 // they need no branch
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const T x = wrow[c][min(max(u + e, 0), max(w.cnt - 1, 0))];
-                    v[e] = ((unsigned)(u + e) < (unsigned)w.cnt) ? x : (T)0.f;
+                    pc.v[e] = ((unsigned)(u + e) < (unsigned)w.cnt) ? x : (T)0.f;
                 }
             } else {
-                v = gather_affine8<vec8>(wrow[c], w, jj);
+                pc.v = gather_affine8<vec8>(wrow[c], w, jj);
             }
-            return v;
+            return pc;
         };
-        vec8 praw[4];
+        // the piece's place in the staging tile, and what goes there
+        auto stage_piece = [&](char* stg, const Piece& pc, int c) {
+            char* own = stg + (8 * c + (lane >> 3)) * P_ROW + (P_MARGIN + (lane & 7) * 8) * ES;
+            if constexpr (ES == 2) {
+                if (!__any(pc.state != 1)) {  // every piece of the instruction lies inside its row's span
+                    *reinterpret_cast<vec8*>(own) = pc.v;
+                } else {
+                    vec8 zero;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) zero[e] = (T)0.f;
+                    if (pc.state != 1) *reinterpret_cast<vec8*>(own) = zero;
+                    if (pc.state != 0) __builtin_memcpy(own + pc.shift * ES, &pc.v, 8 * ES);
+                }
+            } else {
+                *reinterpret_cast<vec8*>(own) = pc.v;
+            }
+        };
+        Piece praw[4];
 #pragma unroll
         for (int c = 0; c < 4; ++c) praw[c] = load_probs(0, c);
 
@@ -216,7 +254,7 @@ __global__ __launch_bounds__(256, 2) void spmm_kernel(const SpmmParams p) {
             char* stg = s_p[wave];
 #pragma unroll
             for (int c = 0; c < 4; ++c)
-                *reinterpret_cast<vec8*>(stg + (8 * c + (lane >> 3)) * P_ROW + (lane & 7) * 8 * ES) = praw[c];
+                stage_piece(stg, praw[c], c);
             if (tile + 1 < pl.n_tiles) {
 #pragma unroll
                 for (int c = 0; c < 4; ++c) praw[c] = load_probs(j0 + kBN, c);
@@ -225,7 +263,7 @@ __global__ __launch_bounds__(256, 2) void spmm_kernel(const SpmmParams p) {
             if (skip) continue;
             Frag<T> pf[kBN / 16];
 #pragma unroll
-            for (int t = 0; t < kBN / 16; ++t) pf[t] = lds_frag_rowmajor<T>(stg + lm * P_ROW + (16 * t + 8 * g) * ES);
+            for (int t = 0; t < kBN / 16; ++t) pf[t] = lds_frag_rowmajor<T>(stg + lm * P_ROW + (P_MARGIN + 16 * t + 8 * g) * ES);
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // fragments read before the next tile overwrites the staging
 #pragma unroll
             for (int t = 0; t < kBN / 16; ++t) {
