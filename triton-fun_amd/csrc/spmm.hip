@@ -320,6 +320,7 @@ struct SpmmTParams {
     SegPtrs seg_t[SPLAT_MAX_SEGMENTS];  // the transposed mask: which rows column j meets
     int n_row_blocks, total, n_col_chunks;
     int row_stride;  // of the transposed mask's ACSR
+    int64_t p_elems;  // elements of p
 };
 
 // Row i's entries seen from a block of columns first + rs*m, m = 0..127.
@@ -451,11 +452,27 @@ __global__ __launch_bounds__(256, 2) void spmm_t_kernel(const SpmmTParams p) {
         auto load_probs = [&](const BlockRow& br, int pos0, int c) {
             vec8 v;
             const RowWin& w = br.w;
-            const T* wrow = pb + (int64_t)min(max(row_at(pos0 + prow), 0), p.L - 1) * p.T + src.slot_offset;
+            const int i_row = min(max(row_at(pos0 + prow), 0), p.L - 1);
+            const T* wrow = pb + (int64_t)i_row * p.T + src.slot_offset;
             const int jj = 8 * (pq + 4 * c);
             const int u = jj - w.lo;
-            if (w.lin == 1 && u >= 0 && u + 8 <= w.cnt) {
+            // A piece that straddles an end of the row's span is loaded like any other, as 16 bytes from where its first
+            // position would be, and the positions outside the span are cleared afterwards: what lies there (dead
+            // slots, the neighbouring row) is readable memory unless the piece leaves the whole buffer.  (Assembling
+            // such a piece from element loads costs more than the loads: the compiler guards their registers with a
+            // wait for every load in flight.)
+            const int64_t e0 = ((int64_t)bh * p.L + i_row) * p.T + src.slot_offset + u;
+            const bool touches = (u + 8 > 0) && (u < w.cnt);
+            if (w.lin == 1 && touches && e0 >= 0 && e0 + 8 <= p.p_elems) {
                 __builtin_memcpy(&v, wrow + u, 8 * ES);  // any alignment
+                if (u < 0 || u + 8 > w.cnt) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if ((unsigned)(u + e) >= (unsigned)w.cnt) v[e] = (T)0.f;
+                }
+            } else if (w.lin == 1 && !touches) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] = (T)0.f;
             } else if (w.lin == 1) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
@@ -601,6 +618,7 @@ extern "C" int splat_spmm_t(const void* pp, const void* x, int64_t x_sb, int64_t
     if (int rc = fill_segs(who, segs, n_seg, p.seg, T)) return rc;
     if (int rc = fill_segs(who, segs_t, n_seg, p.seg_t, -1)) return rc;
     p.row_stride = common_row_stride(segs_t, n_seg);
+    p.p_elems = (int64_t)B * H * L * T;
     const int es = in_dtype == SPLAT_F32 ? 4 : 2;
     const int epc = 16 / es;
     p.x_vec = ((reinterpret_cast<uintptr_t>(x) & 15) == 0 && x_sb % epc == 0 && x_sh % epc == 0 && x_sl % epc == 0) ? 1 : 0;
