@@ -178,10 +178,10 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
         const int off = s_off[sg];
         // this lane's own row (source of the wavefront's span) and the 2 block rows it writes out
         const RowWin mine = make_row_win(cached_row_map<BM>(&s_ps, sg, 32 * wave + lm), pl);
-        int lmin = mine.cnt > 0 ? mine.lo : 0x3fffffff;
-        int hmax = mine.cnt > 0 ? mine.lo + mine.cnt : -0x3fffffff;
-        lmin = wave_min_i(lmin);
-        hmax = wave_max_i(hmax);
+        // tiles before lmin / from hmax on hold nothing for this wavefront; tiles from lo_max on and up to hi_min lie
+        // inside every one of its rows' spans (never, if a row is empty or the plan is not uniform)
+        const WaveSpan span = wave_span(mine, pl.uniform != 0);
+        const int lmin = span.lo_min, hmax = span.hi_max;
         RowWin wr[2];
         int64_t wbase[2];
 #pragma unroll
@@ -193,9 +193,28 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
             wbase[c] = out_bh + (int64_t)r * p.T + off;
         }
 
+        // Tiles whose keys all exist need none of load_piece's clamping and 64-bit index arithmetic: a wavefront-uniform
+        // base (the tile's first key) plus a per-lane byte offset that is fixed for the segment.
+        const bool k_fast = !KT && QREG && p.k_vec && (d % EPC == 0) && ((int64_t)pl.cs * kBN * p.k_sl * ES < ((int64_t)1 << 31));
+        uint32_t k_off[CPT];
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+            const int idx = tid + 256 * i;
+            k_off[i] = (uint32_t)(((int64_t)pl.cs * (idx / CR) * p.k_sl + (idx % CR) * EPC) * ES);
+        }
+        auto load_tile_piece = [&](int tile, int i) {
+            const int64_t key_first = pl.c0 + (int64_t)pl.cs * (tile * kBN), key_last = key_first + (int64_t)pl.cs * (kBN - 1);
+            if (k_fast && key_first >= 0 && key_last < p.n_keys) {  // wavefront-uniform
+                const char* base = reinterpret_cast<const char*>(kb + key_first * p.k_sl);
+                u32x4 val = {0u, 0u, 0u, 0u};
+                if (((tid + 256 * i) % CR) * EPC < d) val = *reinterpret_cast<const u32x4*>(base + k_off[i]);
+                return val;
+            }
+            return load_piece(pl, tile * kBN, 0, i);
+        };
         u32x4 kreg[CPT];
 #pragma unroll
-        for (int i = 0; i < CPT; ++i) kreg[i] = load_piece(pl, t_begin * kBN, 0, i);
+        for (int i = 0; i < CPT; ++i) kreg[i] = QREG ? load_tile_piece(t_begin, i) : load_piece(pl, t_begin * kBN, 0, i);
         // Wait for them here: otherwise the compiler's wait for them sits at the top of the loop below, where on every
         // later iteration it can only mean "everything outstanding", the previous tile's stores included.
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -227,7 +246,7 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
                     const int nkd0 = last_ch ? 0 : kd0 + DC;
                     if (!(last_ch && tile + 1 == t_end)) {
 #pragma unroll
-                        for (int i = 0; i < CPT; ++i) kreg[i] = load_piece(pl, nj0, nkd0, i);
+                        for (int i = 0; i < CPT; ++i) kreg[i] = QREG ? load_tile_piece(tile + 1, i) : load_piece(pl, nj0, nkd0, i);
                     }
                 }
                 lds_barrier();  // the chunk is in LDS (the loads just requested stay in flight)
@@ -277,33 +296,48 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
 #endif
             if (skip) continue;
 
+            // every position of the tile is a slot of every row of this wavefront: no tests, one vector store per piece
+            const bool full = (j0 >= span.lo_max) && (j0 + kBN <= span.hi_min);
+            auto write_tile = [&](auto zero) {
+                using TO = decltype(zero);
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                // ---- turn the half tile around: lane (query lm, half g) holds positions 8jq + 4g + {0..3} ----
+                for (int nt = 0; nt < NT; ++nt) {
+                    // ---- turn the half tile around: lane (query lm, half g) holds positions 8jq + 4g + {0..3} ----
 #pragma unroll
-                for (int jq = 0; jq < 4; ++jq) {
-                    f32x4 v4 = {acc[nt][4 * jq] * p.scale, acc[nt][4 * jq + 1] * p.scale, acc[nt][4 * jq + 2] * p.scale,
-                                acc[nt][4 * jq + 3] * p.scale};
-                    *reinterpret_cast<f32x4*>(stg + lm * S_ROW + (8 * jq + 4 * g) * 4) = v4;
+                    for (int jq = 0; jq < 4; ++jq) {
+                        f32x4 v4 = {acc[nt][4 * jq] * p.scale, acc[nt][4 * jq + 1] * p.scale, acc[nt][4 * jq + 2] * p.scale,
+                                    acc[nt][4 * jq + 3] * p.scale};
+                        *reinterpret_cast<f32x4*>(stg + lm * S_ROW + (8 * jq + 4 * g) * 4) = v4;
+                    }
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wavefront's LDS writes are visible to its own reads
+                    // ---- lane writes positions 8*(lane%4) .. +7 of block rows 32w + 16c + lane/4 ----
+#pragma unroll
+                    for (int c = 0; c < 2; ++c) {
+                        const char* src = stg + (16 * c + (lane >> 2)) * S_ROW + (lane & 3) * 32;
+                        const f32x4 a0 = *reinterpret_cast<const f32x4*>(src);
+                        const f32x4 a1 = *reinterpret_cast<const f32x4*>(src + 16);
+                        const float v[8] = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+                        const int jj = j0 + 32 * nt + 8 * (lane & 3);
+                        TO* const row_out = (TO*)p.out + wbase[c];
+                        if (full) {
+                            typedef TO v8 __attribute__((ext_vector_type(8)));
+                            v8 t;
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) t[e] = (TO)v[e];
+                            __builtin_memcpy(row_out + (jj - wr[c].lo), &t, 8 * sizeof(TO));
+                        } else {
+                            store_piece<TO>(row_out, wr[c], jj, v);
+                        }
+                    }
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // staging reads done before it is overwritten
                 }
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wavefront's LDS writes are visible to its own reads
-                // ---- lane writes positions 8*(lane%4) .. +7 of block rows 32w + 16c + lane/4 ----
-#pragma unroll
-                for (int c = 0; c < 2; ++c) {
-                    const char* src = stg + (16 * c + (lane >> 2)) * S_ROW + (lane & 3) * 32;
-                    const f32x4 a0 = *reinterpret_cast<const f32x4*>(src);
-                    const f32x4 a1 = *reinterpret_cast<const f32x4*>(src + 16);
-                    const float v[8] = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
-                    const int jj = j0 + 32 * nt + 8 * (lane & 3);
-                    if (p.out_dtype == SPLAT_BF16)
-                        store_piece<bf16>((bf16*)p.out + wbase[c], wr[c], jj, v);
-                    else if (p.out_dtype == SPLAT_F16)
-                        store_piece<f16>((f16*)p.out + wbase[c], wr[c], jj, v);
-                    else
-                        store_piece<float>((float*)p.out + wbase[c], wr[c], jj, v);
-                }
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // staging reads done before it is overwritten
-            }
+            };
+            if (p.out_dtype == SPLAT_BF16)
+                write_tile((bf16)0);
+            else if (p.out_dtype == SPLAT_F16)
+                write_tile((f16)0);
+            else
+                write_tile(0.0f);
         }
     }
 }
