@@ -180,3 +180,17 @@ def test_comparison_sweeps_run_and_agree_with_dense(dev):
     assert len(att) == 7 and max(r["max_abs_diff"] for r in att) <= 1e-2
     with pytest.raises(Exception, match="Not implemented!"):
         comparison.benchmark("Strided", 64, 16, 16, dev, verbose=False)
+
+
+def test_a_segment_that_is_empty_everywhere_is_dropped(dev):
+    """Strided pattern on a sequence shorter than its local window: the far segment has no column at all."""
+    segs = A.create_acsr_segments(A.strided_patterns(100, 128, 16), 16, dev)
+    assert len(segs) == 1 and segs.T == 100
+    q, k, _ = O.make_inputs(3, 1, 2, 100, 64, torch.float32)
+    out = torch.zeros(1, 2, 100, segs.T, device=dev)
+    r_sddmm.rsddmm_launcher(q.to(dev), k.to(dev).transpose(2, 3), out, None, None, None, None, segs.T, None, None, None, None,
+                            16, 16, segments=segs)
+    want = torch.tril(q @ k.transpose(2, 3))
+    got = out.cpu()
+    for r in (0, 37, 99):
+        assert float((got[0, 1, r, :r + 1] - want[0, 1, r, :r + 1]).abs().max()) <= 1e-4

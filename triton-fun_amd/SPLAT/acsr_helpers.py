@@ -281,8 +281,11 @@ class ACSRSegments:
     [offsets[k], offsets[k] + T_k); ``T`` is the total trailing dimension."""
 
     def __init__(self, tuples: Sequence[tuple], first_cols: Sequence[torch.Tensor | None]):
-        self.tuples = list(tuples)
-        self.first_cols = list(first_cols)
+        # a segment that is empty in every row (trailing dimension 0) owns no slots: it is dropped, unless it is all
+        # there is (its slot offset would equal the row length, which the kernels reject)
+        keep = [i for i, t in enumerate(tuples) if int(t[5]) > 0] or [0]
+        self.tuples = [tuples[i] for i in keep]
+        self.first_cols = [first_cols[i] for i in keep]
         self.offsets = []
         off = 0
         for t in self.tuples:
