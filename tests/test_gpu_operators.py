@@ -76,6 +76,57 @@ def test_sddmm_patterns(dev, dtype, layout, make, d):
     assert torch.all(got[..., ~lv] == SENTINEL)
 
 
+@pytest.mark.parametrize("in_dt,out_dt", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16),
+                                          (torch.float32, torch.bfloat16)])
+@pytest.mark.parametrize("make,d", [
+    (lambda: O.create_causal_windowed_mask(1024, 511), 64),    # T = 512: rows of whole 16-byte pieces, short rows on top
+    (lambda: O.create_causal_windowed_mask(1024, 399), 128),   # T = 400, not a multiple of 64: every row ends inside a line
+    (lambda: O.create_windowed_mask(1024, 197), 64),           # T = 395: odd row length, rows clipped at both borders
+    (lambda: O.create_dilated_mask(1024, 448, 2), 64),         # row-stride grouping, T = 448
+    (lambda: O.create_blocked_mask(1024, 250), 64)],           # T = 500
+    ids=["causal512", "causal400", "window395", "dilated448", "blocked500"])
+def test_sddmm_line_wise_output(dev, make, d, in_dt, out_dt):
+    """Launches with at least 512 row blocks, 16-bit output and T >= 384 collect each row's scores in an LDS ring and
+    store whole 64-slot lines: same values as the oracle in every live slot, dead slots untouched."""
+    mask = make()
+    L = mask.shape[0]
+    B, H = 8, 8  # 64 x 8 row blocks = 512
+    q, k, _ = O.make_inputs(21, B, H, L, d, in_dt)
+    acsr, acsr_np = acsr_pair(mask, 16, dev)
+    assert acsr[5] >= 384
+    scale = d ** -0.5
+    out = torch.full((B, H, L, acsr[5]), SENTINEL, dtype=out_dt, device=dev)
+    r_sddmm.rsddmm_launcher(q.to(dev), k.to(dev).transpose(2, 3), out, acsr[0], acsr[1], acsr[2], acsr[3], acsr[5], acsr[4],
+                            (1, 1), None, None, 16, 16, scale=scale)
+    want = O.sddmm(q, k.transpose(2, 3), acsr_np, scale)
+    got = out.float().cpu()
+    lv = live(acsr_np)
+    tol = TOL[out_dt] * max(1.0, float(want.abs().max()))
+    assert float((got - want)[..., lv].abs().max()) <= tol
+    assert torch.all(got[..., ~lv] == SENTINEL), "dead slots must not be written"
+
+
+def test_sddmm_line_wise_output_two_segments(dev):
+    """The same path with two segments per row (local window 400 + every 8th earlier column): the second segment's
+    slots start at offset 400 of a row of 478."""
+    L, d = 1024, 64
+    pats = A.strided_patterns(L, 400, 8)
+    dms = O.create_strided_segment_masks(L, 400, 8)
+    segs = A.create_acsr_segments(pats, 16, dev)
+    assert segs.T >= 384 and len(segs) == 2
+    B, H = 8, 8
+    q, k, _ = O.make_inputs(22, B, H, L, d, torch.bfloat16)
+    out = torch.full((B, H, L, segs.T), SENTINEL, dtype=torch.bfloat16, device=dev)
+    r_sddmm.rsddmm_launcher(q.to(dev), k.to(dev).transpose(2, 3), out, None, None, None, None, segs.T, None, None, None, None,
+                            16, 16, scale=d ** -0.5, segments=segs)
+    dense = (q.float() @ k.float().transpose(2, 3)) * d ** -0.5
+    want = torch.cat([O.compress(dense, O.create_acsr(m, 16), first_col=O.row_extents(m)[0], fill=SENTINEL) for m in dms], dim=-1)
+    got = out.float().cpu()
+    lv = want != SENTINEL
+    assert float((got - want)[lv].abs().max()) <= TOL[torch.bfloat16] * max(1.0, float(dense.abs().max()))
+    assert torch.all(got[~lv] == SENTINEL)
+
+
 # ---------------------------------------------------------------- softmax
 @pytest.mark.parametrize("n,p", REF_SMALL)
 def test_softmax_reference_cases(dev, n, p):

@@ -29,6 +29,7 @@ struct SddmmParams {
     SegPtrs seg[SPLAT_MAX_SEGMENTS];
     int n_row_blocks, total;
     int q_vec, k_vec;  // 16-byte loads are legal for q / k
+    int out_vec;       // 16-bit outputs: every row's segment starts on a 16-byte boundary
     int row_stride;
     int key_split;  // workgroups per row block: each takes a contiguous share of every segment's tiles
 };
@@ -92,7 +93,12 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
     constexpr int S_ROW = 32 * 4 + 16;                            // staging row: 32 floats + pad
 
     __shared__ __attribute__((aligned(16))) char s_k[K_ROW * K_ROWS];
-    __shared__ __attribute__((aligned(16))) char s_stage[4][32 * S_ROW];
+    // Per-wavefront staging: either the turn-around tile (32 rows of 32 floats) or, for 16-bit outputs of uniform plans,
+    // a ring of 128 slots per row in which a row's scores collect until a whole 128-byte line of it can be stored
+    // (+ 4 slots that mirror the ring's first 4, so that a read of 8 slots never wraps).
+    constexpr int R_SLOTS = 128, R_ROW = (R_SLOTS + 4) * 2 + 8;
+    constexpr int STG_BYTES = 32 * S_ROW > 32 * R_ROW ? 32 * S_ROW : 32 * R_ROW;
+    __shared__ __attribute__((aligned(16))) char s_stage[4][STG_BYTES];
     __shared__ SegPlan s_plan[SPLAT_MAX_SEGMENTS];
     __shared__ int s_off[SPLAT_MAX_SEGMENTS];
     __shared__ PlanScratch<BM> s_ps;
@@ -212,6 +218,27 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
             }
             return load_piece(pl, tile * kBN, 0, i);
         };
+        // ---- line-wise output (16-bit outputs, uniform plans, the whole row block in this workgroup) ----
+        // Scores go from the accumulators into the row's ring at (slot + lo%4) mod 128, four consecutive slots at a time,
+        // untested: a position outside the row's span lands on ring entries that are not waiting to be stored.  After each
+        // tile every row stores the 64-slot lines that have become complete (and, once its last position has passed,
+        // the rest), 8 lanes x 16 bytes per line: whole aligned lines instead of pieces that straddle them, which is
+        // what lets them bypass the L2's write combining (non-temporal stores).
+        // (rows of fewer than six lines gain less from whole lines than the line bookkeeping costs: config 2, T = 256)
+        const bool use_ring = pl.uniform && p.key_split == 1 && p.out_dtype != SPLAT_F32 && p.T >= 384;
+        int f_lo[4], f_cnt[4], f_done[4];
+        int64_t f_base[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int rr = 32 * wave + 8 * c + (lane >> 3);
+            const RowWin w = make_row_win(cached_row_map<BM>(&s_ps, sg, rr), pl);
+            const int r = r0 + rs * rr;
+            f_lo[c] = w.lo;
+            f_cnt[c] = (r < L) ? w.cnt : 0;
+            f_done[c] = 0;
+            f_base[c] = out_bh + (int64_t)r * p.T + off;
+        }
+        const int lo4 = mine.lo & ~3;
         u32x4 kreg[CPT];
 #pragma unroll
         for (int i = 0; i < CPT; ++i) kreg[i] = QREG ? load_tile_piece(t_begin, i) : load_piece(pl, t_begin * kBN, 0, i);
@@ -332,12 +359,66 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // staging reads done before it is overwritten
                 }
             };
-            if (p.out_dtype == SPLAT_BF16)
+            auto ring_tile = [&](auto zero) {
+                using TO = decltype(zero);
+                typedef TO v4 __attribute__((ext_vector_type(4)));
+                typedef TO v8 __attribute__((ext_vector_type(8)));
+                char* const ring_row = stg + lm * R_ROW;
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int jq = 0; jq < 4; ++jq) {
+                        v4 t;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) t[i] = (TO)(acc[nt][4 * jq + i] * p.scale);
+                        const int ri = (j0 + 32 * nt + 8 * jq + 4 * g - lo4) & (R_SLOTS - 1);
+                        *reinterpret_cast<v4*>(ring_row + ri * 2) = t;
+                        if (ri == 0) *reinterpret_cast<v4*>(ring_row + R_SLOTS * 2) = t;
+                    }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wavefront's LDS writes are visible to its own reads
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const int u_end = j0 + kBN - f_lo[c];
+                    const int final_slot = min(max(u_end, 0), f_cnt[c]);  // slots below it hold their scores
+#pragma unroll
+                    for (int rep = 0; rep < 2; ++rep) {
+                        const int ls = 64 * f_done[c];
+                        const bool line = (ls + 64 <= final_slot) || (u_end >= f_cnt[c] && ls < f_cnt[c]);
+                        if (line) {
+                            const int s0 = ls + 8 * (lane & 7);
+                            const int rix = (s0 + (f_lo[c] & 3)) & (R_SLOTS - 1);
+                            v8 val;
+                            __builtin_memcpy(&val, stg + (8 * c + (lane >> 3)) * R_ROW + rix * 2, 16);
+                            TO* const dst = (TO*)p.out + f_base[c] + s0;
+                            const int n = f_cnt[c] - s0;
+                            if (n >= 8) {
+                                if (p.out_vec) {
+                                    __builtin_nontemporal_store(val, reinterpret_cast<v8*>(dst));
+                                } else {
+                                    __builtin_memcpy(dst, &val, 16);
+                                }
+                            } else {
+#pragma unroll
+                                for (int e = 0; e < 8; ++e)
+                                    if (e < n) dst[e] = val[e];
+                            }
+                            f_done[c] += 1;
+                        }
+                    }
+                }
+            };
+            if (use_ring) {
+                if (p.out_dtype == SPLAT_BF16)
+                    ring_tile((bf16)0);
+                else
+                    ring_tile((f16)0);
+            } else if (p.out_dtype == SPLAT_BF16) {
                 write_tile((bf16)0);
-            else if (p.out_dtype == SPLAT_F16)
+            } else if (p.out_dtype == SPLAT_F16) {
                 write_tile((f16)0);
-            else
+            } else {
                 write_tile(0.0f);
+            }
         }
     }
 }
@@ -409,6 +490,9 @@ extern "C" int splat_sddmm(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_
     const bool kt = !(k_sd == 1);
     p.q_vec = (al(q) && mul(q_sb) && mul(q_sh) && mul(q_sl)) ? 1 : 0;
     p.k_vec = (al(kT) && mul(k_sb) && mul(k_sh) && mul(kt ? k_sd : k_sl)) ? 1 : 0;
+    p.out_vec = (al(out) && T % 8 == 0) ? 1 : 0;
+    for (int k = 0; k < n_seg; ++k)
+        if (segs[k].slot_offset % 8 != 0) p.out_vec = 0;
     hipStream_t st = (hipStream_t)stream;
     switch (in_dtype) {
         case SPLAT_F32: return launch_sddmm<float>(p, kt, st);
