@@ -60,7 +60,7 @@ __global__ __launch_bounds__(256) void softmax_bwd_kernel(const T* __restrict__ 
                 vecT o;
 #pragma unroll
                 for (int e = 0; e < EPC; ++e) o[e] = (T)((float)a[e] * ((float)b[e] - rs) * scale);
-                *reinterpret_cast<vecT*>(dsr + s) = o;
+                __builtin_nontemporal_store(o, reinterpret_cast<vecT*>(dsr + s));
             }
             for (int s = lo + lane; s < min(v_lo, hi); s += 64) dsr[s] = (T)((float)pr[s] * ((float)dpr[s] - rs) * scale);
             for (int s = v_hi + lane; s < hi; s += 64) dsr[s] = (T)((float)pr[s] * ((float)dpr[s] - rs) * scale);

@@ -135,7 +135,7 @@ __global__ __launch_bounds__(256) void softmax_rows_vec(const Tin* __restrict__ 
                     vout o;
 #pragma unroll
                     for (int e = 0; e < 8; ++e) o[e] = (Tout)(v[c][e] * inv);
-                    *reinterpret_cast<vout*>(yr + (ch << 3)) = o;
+                    __builtin_nontemporal_store(o, reinterpret_cast<vout*>(yr + (ch << 3)));
                 } else {
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
