@@ -604,7 +604,8 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
             const int row = flat / CPR, c = flat % CPR;
             const int r = r0 + rs * (wave * 32 + row);
             const u32x4 val = *reinterpret_cast<const u32x4*>(stg + row * OROW + c * 16);
-            if (r < L) *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(ob + (int64_t)r * p.o_sl) + c * 16) = val;
+            // non-temporal: whole aligned rows that this kernel never reads back, so they need not pass through the L2
+            if (r < L) __builtin_nontemporal_store(val, reinterpret_cast<u32x4*>(reinterpret_cast<char*>(ob + (int64_t)r * p.o_sl) + c * 16));
         }
     }
 }
