@@ -106,6 +106,30 @@ def test_sddmm_line_wise_output(dev, make, d, in_dt, out_dt):
     assert torch.all(got[..., ~lv] == SENTINEL), "dead slots must not be written"
 
 
+def test_sddmm_line_wise_output_of_short_rows_in_a_large_launch(dev):
+    """Rows of four lines (T = 256) take the line-wise path only in launches of at least 4096 row blocks: the 16-bit
+    output must be the rounding of what the piece-wise path writes in float32 (same accumulators), dead slots untouched."""
+    L, d, B, H = 1024, 64, 16, 32
+    pat = A.causal_windowed_pattern(L, 255)
+    acsr = A.create_acsr(pat, 16, dev)
+    T = acsr[5]
+    assert T == 256
+    g = torch.Generator().manual_seed(23)
+    q = torch.randn(B, H, L, d, generator=g).to(torch.bfloat16).to(dev)
+    k = torch.randn(B, H, L, d, generator=g).to(torch.bfloat16).to(dev)
+    outs = {}
+    for dt in (torch.float32, torch.bfloat16):
+        out = torch.full((B, H, L, T), SENTINEL, dtype=dt, device=dev)
+        r_sddmm.rsddmm_launcher(q, k.transpose(2, 3), out, acsr[0], acsr[1], acsr[2], acsr[3], T, acsr[4], (1, 1), None, None,
+                                16, 16, scale=d ** -0.5)
+        outs[dt] = out
+    live_slots = torch.arange(T, device=dev)[None, :] < acsr[4][:, None]
+    zero = torch.zeros((), dtype=torch.bfloat16, device=dev)
+    a, b = outs[torch.float32].to(torch.bfloat16), outs[torch.bfloat16]
+    assert torch.equal(torch.where(live_slots, a, zero), torch.where(live_slots, b, zero))
+    assert torch.all(b[..., ~live_slots] == SENTINEL)
+
+
 def test_sddmm_line_wise_output_two_segments(dev):
     """The same path with two segments per row (local window 400 + every 8th earlier column): the second segment's
     slots start at offset 400 of a row of 478."""

@@ -224,8 +224,9 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
         // tile every row stores the 64-slot lines that have become complete (and, once its last position has passed,
         // the rest), 8 lanes x 16 bytes per line: whole aligned lines instead of pieces that straddle them, which is
         // what lets them bypass the L2's write combining (non-temporal stores).
-        // (rows of fewer than six lines gain less from whole lines than the line bookkeeping costs: config 2, T = 256)
-        const bool use_ring = pl.uniform && p.key_split == 1 && p.out_dtype != SPLAT_F32 && p.T >= 384;
+        // (measured: rows of four or five lines gain 13 % in launches of 4096 row blocks and lose 5 % in one of 2048)
+        const bool use_ring = pl.uniform && p.key_split == 1 && p.out_dtype != SPLAT_F32 &&
+                              (p.T >= 384 || (p.T >= 256 && p.total >= 4096));
         int f_lo[4], f_cnt[4], f_done[4];
         int64_t f_base[4];
 #pragma unroll
