@@ -30,12 +30,41 @@ struct SpmmParams {
 // columns col0..).  An accumulator register holds one row's value at column lane%32: stored directly, a wavefront
 // instruction writes 32 consecutive elements of two rows.  When rows of the output can take 16-byte stores (`wide`), each
 // 32 x 32 tile is instead converted, turned around in the wavefront's staging area `stg` (32 rows of 144 bytes at
-// least) and written as 16-byte pieces (8 or 4 per row).
+// least) and written as 16-byte pieces (8 or 4 per row).  16-bit outputs with a staging area `rows_stg` of
+// 32 x (64*DVT + 16) bytes: the whole 32 x (32*DVT) block is turned around at once and leaves as whole rows of the block
+// (aligned runs of 64*DVT bytes, non-temporal) instead of one 64-byte piece of every row per 32-column tile.
 template <int DVT>
-__device__ __forceinline__ void store_block_rows(const f32x16 (&acc)[DVT], char* stg, void* out, int out_dtype, bool wide,
-                                                 int64_t bh, int n_rows, int n_out, int r0, int rs, int wave, int lane, int col0) {
+__device__ __forceinline__ void store_block_rows(const f32x16 (&acc)[DVT], char* stg, char* rows_stg, void* out, int out_dtype,
+                                                 bool wide, int64_t bh, int n_rows, int n_out, int r0, int rs, int wave, int lane,
+                                                 int col0) {
     const int lm = lane & 31, g = lane >> 5;
     const int es_out = (out_dtype == SPLAT_F32) ? 4 : 2;
+    if (wide && es_out == 2 && rows_stg != nullptr) {
+        constexpr int ROW_B = 64 * DVT + 16, CPR = 4 * DVT;  // padded staging row, 16-byte pieces per row
+#pragma unroll
+        for (int dt = 0; dt < DVT; ++dt)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                char* dst = rows_stg + acc_row(j, g) * ROW_B + (32 * dt + lm) * 2;
+                if (out_dtype == SPLAT_BF16)
+                    *reinterpret_cast<bf16*>(dst) = (bf16)acc[dt][j];
+                else
+                    *reinterpret_cast<f16*>(dst) = (f16)acc[dt][j];
+            }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wavefront's LDS writes are visible to its own reads
+#pragma unroll
+        for (int i = 0; i < 32 * CPR / 64; ++i) {
+            const int flat = i * 64 + lane;
+            const int row = flat / CPR, c = flat % CPR;
+            const int r = r0 + rs * (32 * wave + row);
+            const u32x4 val = *reinterpret_cast<const u32x4*>(rows_stg + row * ROW_B + c * 16);
+            if (r < n_rows) {
+                char* orow = reinterpret_cast<char*>(out) + ((bh * n_rows + r) * n_out + col0) * 2;
+                __builtin_nontemporal_store(val, reinterpret_cast<u32x4*>(orow + c * 16));
+            }
+        }
+        return;
+    }
     if (wide) {
         const int row_b = 32 * es_out + 16;  // padded staging row
         const int cpr = 32 * es_out / 16;     // 16-byte pieces per row
@@ -94,7 +123,8 @@ __global__ __launch_bounds__(256, 2) void spmm_kernel(const SpmmParams p) {
     constexpr int P_MARGIN = (ES == 2) ? 8 : 0;
     constexpr int P_ROW = (kBN + 2 * P_MARGIN) * ES + 16;
     __shared__ __attribute__((aligned(16))) char s_v[V_ROW * kBN];
-    __shared__ __attribute__((aligned(16))) char s_p[4][32 * P_ROW];
+    constexpr int SP_BYTES = 32 * P_ROW;
+    __shared__ __attribute__((aligned(16))) char s_p[4][SP_BYTES];
     static_assert(P_ROW >= 32 * 4 + 16, "the staging area also holds a 32 x 32 fp32 tile of the output");
     __shared__ SegPlan s_plan[SPLAT_MAX_SEGMENTS];
     __shared__ SegPtrs s_seg[SPLAT_MAX_SEGMENTS];
@@ -277,8 +307,15 @@ __global__ __launch_bounds__(256, 2) void spmm_kernel(const SpmmParams p) {
     }
 
     __syncthreads();  // every wavefront is done with the staging areas and the V tile
-    store_block_rows<DVT>(acc, s_p[wave], p.out, p.out_dtype, p.out_vec && (col0 + 32 * DVT <= p.n_out), bh, L, p.n_out, r0, rs,
-                          wave, lane, col0);
+    // whole-row staging: the wavefront's own area if it is large enough, else halves of the two tiles (all free now)
+    constexpr int ROWS_STG = 32 * (64 * DVT + 16);
+    char* rows_stg = nullptr;
+    if constexpr (ROWS_STG <= SP_BYTES)
+        rows_stg = s_p[wave];
+    else if constexpr (2 * ROWS_STG <= 4 * SP_BYTES && 2 * ROWS_STG <= V_ROW * kBN)
+        rows_stg = (wave < 2 ? &s_p[0][0] : s_v) + (wave & 1) * ROWS_STG;
+    store_block_rows<DVT>(acc, s_p[wave], rows_stg, p.out, p.out_dtype, p.out_vec && (col0 + 32 * DVT <= p.n_out), bh, L, p.n_out,
+                          r0, rs, wave, lane, col0);
 }
 
 template <typename T>
@@ -535,8 +572,11 @@ __global__ __launch_bounds__(256, 2) void spmm_t_kernel(const SpmmTParams p) {
     }
 
     __syncthreads();  // every wavefront is done with the tiles
-    store_block_rows<DVT>(acc, s_pt + wave * (32 * (32 * 4 + 16)), p.out, p.out_dtype, p.out_vec && (col0 + 32 * DVT <= p.n_out), bh,
-                          p.Lt, p.n_out, j_first, rs, wave, lane, col0);
+    constexpr int ROWS_STG = 32 * (64 * DVT + 16);
+    char* rows_stg = nullptr;
+    if constexpr (2 * ROWS_STG <= PT_ROW * kBN && 2 * ROWS_STG <= X_ROW * kBN) rows_stg = (wave < 2 ? s_pt : s_x) + (wave & 1) * ROWS_STG;
+    store_block_rows<DVT>(acc, s_pt + wave * (32 * (32 * 4 + 16)), rows_stg, p.out, p.out_dtype,
+                          p.out_vec && (col0 + 32 * DVT <= p.n_out), bh, p.Lt, p.n_out, j_first, rs, wave, lane, col0);
 }
 
 template <typename T>
