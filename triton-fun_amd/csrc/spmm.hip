@@ -30,27 +30,23 @@ struct SpmmParams {
 // columns col0..).  An accumulator register holds one row's value at column lane%32: stored directly, a wavefront
 // instruction writes 32 consecutive elements of two rows.  When rows of the output can take 16-byte stores (`wide`), each
 // 32 x 32 tile is instead converted, turned around in the wavefront's staging area `stg` (32 rows of 144 bytes at
-// least) and written as 16-byte pieces (8 or 4 per row).  16-bit outputs with a staging area `rows_stg` of
-// 32 x (64*DVT + 16) bytes: the whole 32 x (32*DVT) block is turned around at once and leaves as whole rows of the block
-// (aligned runs of 64*DVT bytes, non-temporal) instead of one 64-byte piece of every row per 32-column tile.
+// least) and written as 16-byte pieces (8 or 4 per row).  With a staging area `rows_stg` of at least
+// 32 x (32*DVT*element size + 16) bytes the whole 32 x (32*DVT) block is turned around at once and leaves as whole rows
+// of the block (aligned runs, non-temporal) instead of one 64- or 128-byte piece of every row per 32-column tile.
 template <int DVT>
-__device__ __forceinline__ void store_block_rows(const f32x16 (&acc)[DVT], char* stg, char* rows_stg, void* out, int out_dtype,
-                                                 bool wide, int64_t bh, int n_rows, int n_out, int r0, int rs, int wave, int lane,
-                                                 int col0) {
+__device__ __forceinline__ void store_block_rows(const f32x16 (&acc)[DVT], char* stg, char* rows_stg, int rows_stg_bytes, void* out,
+                                                 int out_dtype, bool wide, int64_t bh, int n_rows, int n_out, int r0, int rs,
+                                                 int wave, int lane, int col0) {
     const int lm = lane & 31, g = lane >> 5;
     const int es_out = (out_dtype == SPLAT_F32) ? 4 : 2;
-    if (wide && es_out == 2 && rows_stg != nullptr) {
-        constexpr int ROW_B = 64 * DVT + 16, CPR = 4 * DVT;  // padded staging row, 16-byte pieces per row
+    auto whole_rows = [&](auto zero) {
+        using TO = decltype(zero);
+        constexpr int ROW_B = 32 * DVT * (int)sizeof(TO) + 16, CPR = 2 * DVT * (int)sizeof(TO);  // staging row, pieces per row
 #pragma unroll
         for (int dt = 0; dt < DVT; ++dt)
 #pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                char* dst = rows_stg + acc_row(j, g) * ROW_B + (32 * dt + lm) * 2;
-                if (out_dtype == SPLAT_BF16)
-                    *reinterpret_cast<bf16*>(dst) = (bf16)acc[dt][j];
-                else
-                    *reinterpret_cast<f16*>(dst) = (f16)acc[dt][j];
-            }
+            for (int j = 0; j < 16; ++j)
+                *reinterpret_cast<TO*>(rows_stg + acc_row(j, g) * ROW_B + (32 * dt + lm) * sizeof(TO)) = (TO)acc[dt][j];
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wavefront's LDS writes are visible to its own reads
 #pragma unroll
         for (int i = 0; i < 32 * CPR / 64; ++i) {
@@ -59,10 +55,18 @@ __device__ __forceinline__ void store_block_rows(const f32x16 (&acc)[DVT], char*
             const int r = r0 + rs * (32 * wave + row);
             const u32x4 val = *reinterpret_cast<const u32x4*>(rows_stg + row * ROW_B + c * 16);
             if (r < n_rows) {
-                char* orow = reinterpret_cast<char*>(out) + ((bh * n_rows + r) * n_out + col0) * 2;
+                char* orow = reinterpret_cast<char*>(out) + ((bh * n_rows + r) * n_out + col0) * sizeof(TO);
                 __builtin_nontemporal_store(val, reinterpret_cast<u32x4*>(orow + c * 16));
             }
         }
+    };
+    if (wide && rows_stg != nullptr && 32 * (32 * DVT * es_out + 16) <= rows_stg_bytes) {
+        if (out_dtype == SPLAT_BF16)
+            whole_rows((bf16)0);
+        else if (out_dtype == SPLAT_F16)
+            whole_rows((f16)0);
+        else
+            whole_rows(0.0f);
         return;
     }
     if (wide) {
@@ -308,14 +312,10 @@ __global__ __launch_bounds__(256, 2) void spmm_kernel(const SpmmParams p) {
 
     __syncthreads();  // every wavefront is done with the staging areas and the V tile
     // whole-row staging: the wavefront's own area if it is large enough, else halves of the two tiles (all free now)
-    constexpr int ROWS_STG = 32 * (64 * DVT + 16);
-    char* rows_stg = nullptr;
-    if constexpr (ROWS_STG <= SP_BYTES)
-        rows_stg = s_p[wave];
-    else if constexpr (2 * ROWS_STG <= 4 * SP_BYTES && 2 * ROWS_STG <= V_ROW * kBN)
-        rows_stg = (wave < 2 ? &s_p[0][0] : s_v) + (wave & 1) * ROWS_STG;
-    store_block_rows<DVT>(acc, s_p[wave], rows_stg, p.out, p.out_dtype, p.out_vec && (col0 + 32 * DVT <= p.n_out), bh, L, p.n_out,
-                          r0, rs, wave, lane, col0);
+    constexpr int HALF = (2 * SP_BYTES < V_ROW * kBN / 2 ? 2 * SP_BYTES : V_ROW * kBN / 2) & ~15;  // per wavefront, two per tile
+    char* const rows_stg = (wave < 2 ? &s_p[0][0] : s_v) + (wave & 1) * HALF;
+    store_block_rows<DVT>(acc, s_p[wave], rows_stg, HALF, p.out, p.out_dtype, p.out_vec && (col0 + 32 * DVT <= p.n_out), bh, L,
+                          p.n_out, r0, rs, wave, lane, col0);
 }
 
 template <typename T>
@@ -572,10 +572,9 @@ __global__ __launch_bounds__(256, 2) void spmm_t_kernel(const SpmmTParams p) {
     }
 
     __syncthreads();  // every wavefront is done with the tiles
-    constexpr int ROWS_STG = 32 * (64 * DVT + 16);
-    char* rows_stg = nullptr;
-    if constexpr (2 * ROWS_STG <= PT_ROW * kBN && 2 * ROWS_STG <= X_ROW * kBN) rows_stg = (wave < 2 ? s_pt : s_x) + (wave & 1) * ROWS_STG;
-    store_block_rows<DVT>(acc, s_pt + wave * (32 * (32 * 4 + 16)), rows_stg, p.out, p.out_dtype,
+    constexpr int HALF = ((PT_ROW < X_ROW ? PT_ROW : X_ROW) * kBN / 2) & ~15;  // per wavefront, two per tile
+    char* const rows_stg = (wave < 2 ? s_pt : s_x) + (wave & 1) * HALF;
+    store_block_rows<DVT>(acc, s_pt + wave * (32 * (32 * 4 + 16)), rows_stg, HALF, p.out, p.out_dtype,
                           p.out_vec && (col0 + 32 * DVT <= p.n_out), bh, p.Lt, p.n_out, j_first, rs, wave, lane, col0);
 }
 
