@@ -26,7 +26,7 @@ MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes one fused launch moves at config 5, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
 # copy kernel of known size (profiles/attn_fwd_kernel_cfg5_hbm_traffic.md).
-FUSED_TRAFFIC_BYTES = 1.400e9
+FUSED_TRAFFIC_BYTES = 1.395e9
 
 
 def causal_window_nnz(L: int, w: int) -> int:
