@@ -130,6 +130,28 @@ def test_sddmm_line_wise_output_of_short_rows_in_a_large_launch(dev):
     assert torch.all(b[..., ~live_slots] == SENTINEL)
 
 
+def test_sddmm_line_wise_output_of_a_long_sequence(dev):
+    """L = 2^17 rows of 512 slots through the line-wise path: with q = 1 every score is the sum of its key's
+    components, so slot s of row r must hold the column sum of key r - 511 + s (rows above 511: key s)."""
+    L, d, w = 1 << 17, 64, 512
+    acsr = A.create_acsr(A.causal_windowed_pattern(L, w - 1), 16, dev)
+    T = acsr[5]
+    g = torch.Generator().manual_seed(24)
+    k = torch.randn(1, 1, L, d, generator=g).to(torch.bfloat16).to(dev)
+    q = torch.ones(1, 1, L, d, dtype=torch.bfloat16, device=dev)
+    out = torch.full((1, 1, L, T), SENTINEL, dtype=torch.bfloat16, device=dev)
+    r_sddmm.rsddmm_launcher(q, k.transpose(2, 3), out, acsr[0], acsr[1], acsr[2], acsr[3], T, acsr[4], (1, 1), None, None, 16, 16)
+    sums = k.float().sum(-1)[0, 0]                                     # [L]
+    rows = torch.arange(L, device=dev)[:, None]
+    slots = torch.arange(T, device=dev)[None, :]
+    first = torch.clamp(rows - (w - 1), min=0)
+    live = slots < torch.clamp(rows + 1, max=w)
+    want = sums[torch.clamp(first + slots, max=L - 1)]
+    got = out[0, 0].float()
+    assert float((got - want)[live].abs().max()) <= 2 ** -7 * float(sums.abs().max()) + 1e-3  # one bf16 rounding
+    assert torch.all(got[~live] == SENTINEL)
+
+
 def test_sddmm_line_wise_output_two_segments(dev):
     """The same path with two segments per row (local window 400 + every 8th earlier column): the second segment's
     slots start at offset 400 of a row of 478."""
