@@ -2,7 +2,7 @@
 """Benchmark of the ACSR sparse-attention forward on one MI355X.
 
 A step is one fused forward (RegularAttention.forward -> splat_attention_fwd_planned, the mask's plan built once in
-the untimed set-up like the ACSR arrays) over BASELINE config 5: B=4, H=16, L=16384, d=128,
+the untimed set-up like the ACSR arrays) over benchmark configuration 5: B=4, H=16, L=16384, d=128,
 bf16, causal window 512, scale 1/sqrt(d), seeded synthetic N(0,1) inputs already resident in HBM, K handed
 over as ``k.transpose(2, 3)`` (a view of row-major K; the K^T-contiguous layout is timed as an extra).
 Prints ONE JSON line.  `value` counts only nonzero (live) FLOPs: 4 * d * nnz * B * H.

@@ -1,5 +1,5 @@
 """Fused forward and the three-kernel composition against fp32 dense masked attention (the oracle), at
-BASELINE's configurations: small ones whole, large ones through a head subset plus size-independent
+the five benchmark configurations: small ones whole, large ones through a head subset plus size-independent
 properties at full size."""
 import numpy as np
 import pytest
@@ -159,7 +159,7 @@ def test_unit_projection_wrapper(dev):
 @pytest.mark.parametrize("L,d,w,dtype", [(32768, 128, 512, torch.bfloat16), (40003, 64, 300, torch.float16),
                                          (1 << 20, 128, 512, torch.bfloat16)])
 def test_long_sequences_by_properties(dev, L, d, w, dtype):
-    """Sequences longer than any BASELINE configuration, one of them not a multiple of any tile size, one of a million
+    """Sequences longer than any benchmark configuration, one of them not a multiple of any tile size, one of a million
     rows: the mask never exists (`MaskPattern`: metadata in closed form), so the checks are size-independent ones:
     V = 1 gives 1 everywhere, and a few rows are recomputed directly from their window."""
     g = torch.Generator().manual_seed(L)
