@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define SPLAT_VERSION 300 /* major*10000 + minor*100 + patch; 0.2.0 added the planned forward, 0.3.0 splat_spmm_t */
+#define SPLAT_VERSION 400 /* major*10000 + minor*100 + patch; 0.2.0 added the planned forward, 0.3.0 splat_spmm_t, 0.4.0 splat_attention_fwd_stats */
 
 /* element types of q/k/v/score/output buffers */
 #define SPLAT_F32 0
@@ -181,6 +181,22 @@ int splat_attention_fwd_planned(const void* q, int64_t q_sb, int64_t q_sh, int64
                                 int64_t o_sh, int64_t o_sl, const splat_acsr_seg* segs /* host */,
                                 int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t d, float scale,
                                 int32_t dtype, const void* plan, int64_t plan_bytes, void* stream);
+
+/* The fused forward that also hands out every row's softmax statistic: lse[(b*H + h)*L + r] = natural log of the
+ * sum over the row's live columns of exp(scale * score), float32, so that the row's probabilities are
+ * exp(scale * score - lse).  +inf for a row without live columns (its output row is zero).  That is what a
+ * caller needs to merge partial results over disjoint key ranges (sequence shards) or to recompute the
+ * probabilities in a backward pass without a second normalisation.  `plan` may be NULL (then as
+ * splat_attention_fwd) or the plan of splat_attention_plan.  `out` is bit-identical to the other two
+ * forwards'.  The reference has no counterpart: r_softmax.py:30-59 normalises in place and keeps neither the
+ * row maximum nor the row sum. */
+int splat_attention_fwd_stats(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT,
+                              int64_t k_sb, int64_t k_sh, int64_t k_sd, int64_t k_sl, const void* v,
+                              int64_t v_sb, int64_t v_sh, int64_t v_sl, void* out, int64_t o_sb,
+                              int64_t o_sh, int64_t o_sl, const splat_acsr_seg* segs /* host */,
+                              int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t d, float scale,
+                              int32_t dtype, const void* plan, int64_t plan_bytes, float* lse,
+                              void* stream);
 
 /* ---- backward pass (the reference has none: r_attention.py:77-100 is forward only) ----
  * With S~ the compressed scores, P~ = softmax(S~), O = P~ . V:

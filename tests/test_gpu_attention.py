@@ -257,6 +257,68 @@ def A_plan(attn, L, dev):
     return attention_plan(attn.segments, L, dev)
 
 
+def _masked_scores(q, k, mask, scale):
+    s = torch.einsum("bhqd,bhkd->bhqk", q.float(), k.float()) * scale
+    return s.masked_fill(torch.as_tensor(np.asarray(mask) == 0), float("-inf"))
+
+
+@pytest.mark.parametrize("case", _plan_cases(), ids=lambda c: c[0])
+def test_forward_with_stats(dev, case):
+    """splat_attention_fwd_stats: the output is bit-identical to the other forwards' and lse equals torch.logsumexp
+    of the masked, scaled fp32 scores (+inf on rows without live columns), with and without a plan."""
+    name, make, L, d, dtype = case
+    B, H = 2, 3
+    mask = make()
+    attn = RegularAttention(B, L, H, d, mask, 16, 16, dev, dtype, scale=d ** -0.5)
+    q, k, v = O.make_inputs(5 * L, B, H, L, d, dtype)
+    if isinstance(mask, np.ndarray):
+        dense = mask
+    else:
+        # the device's rasterisation of a pattern is checked bit for bit against the oracle's masks elsewhere
+        dense = sum(m.device_mask(dev).cpu().numpy() for m in (mask if isinstance(mask, list) else [mask]))
+    want = torch.logsumexp(_masked_scores(q, k, dense, d ** -0.5), dim=-1)
+    want = torch.where(torch.isinf(want), torch.full_like(want, float("inf")), want)   # empty rows: -inf -> +inf
+    qd, kd, vd = [t.to(dev) for t in (q, k, v)]
+    kT = kd.transpose(2, 3)
+    plain = torch.empty_like(qd)
+    attention_launcher(qd, kT, vd, plain, attn.segments, attn.scale)
+    for plan in (None, A_plan(attn, L, dev)):
+        out = torch.full_like(qd, 3)
+        lse = torch.full((B, H, L), -7.0, device=dev)
+        attention_launcher(qd, kT, vd, out, attn.segments, attn.scale, plan, lse)
+        assert torch.equal(out, plain)
+        got = lse.cpu()
+        assert torch.equal(torch.isinf(got), torch.isinf(want))
+        fin = torch.isfinite(want)
+        assert float((got[fin] - want[fin]).abs().max()) <= 2e-5 * max(1.0, float(want[fin].abs().max())), name
+    o2, l2 = attn.forward_with_stats([qd, kT, vd])
+    assert torch.equal(o2, plain) and torch.equal(l2.cpu(), got)
+    with pytest.raises(Exception, match="lse"):
+        attention_launcher(qd, kT, vd, out, attn.segments, attn.scale, None, lse[:, :, :-1])
+
+
+def test_partial_results_merge_through_lse(dev):
+    """The two segments of the strided pattern run as two separate launches, merged row by row with their lse, give
+    the two-segment launch's output and lse: what a caller that shards the keys does."""
+    L, d, B, H = 2048, 128, 1, 2
+    pats = A.strided_patterns(L, 128, 128)
+    q, k, v = [t.to(dev) for t in O.make_inputs(321, B, H, L, d, torch.bfloat16)]
+    kT = k.transpose(2, 3)
+    outs, lses = [], []
+    for m in ([pats[0]], [pats[1]], pats):
+        attn = RegularAttention(B, L, H, d, m, 16, 16, dev, torch.bfloat16, scale=d ** -0.5)
+        o, l = attn.forward_with_stats([q, kT, v])
+        outs.append(o.float().clone())
+        lses.append(l.clone())
+    assert torch.isinf(lses[1][:, :, :128]).all() and torch.isfinite(lses[0]).all()   # no far columns before row 128
+    tot = torch.logaddexp(lses[0], torch.where(torch.isinf(lses[1]), torch.full_like(lses[1], -float("inf")), lses[1]))
+    w0 = torch.exp(lses[0] - tot).unsqueeze(-1)
+    w1 = torch.where(torch.isinf(lses[1]), torch.zeros_like(tot), torch.exp(lses[1] - tot)).unsqueeze(-1)
+    merged = w0 * outs[0] + w1 * outs[1]
+    assert float((tot - lses[2]).abs().max()) <= 1e-4
+    assert float((merged - outs[2]).abs().max()) <= TOL[torch.bfloat16]
+
+
 def test_plan_arguments_are_checked(dev):
     import _splat_hip as hip
     L, d = 256, 64

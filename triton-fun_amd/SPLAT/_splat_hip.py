@@ -60,6 +60,9 @@ _SIGNATURES = {
     "splat_attention_fwd_planned": (ctypes.c_int, [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64,
                                                    _vp, _i64, _i64, _i64, ctypes.POINTER(AcsrSeg), _i32, _i32, _i32, _i32,
                                                    _i32, _f32, _i32, _vp, _i64, _vp]),
+    "splat_attention_fwd_stats": (ctypes.c_int, [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64,
+                                                 _vp, _i64, _i64, _i64, ctypes.POINTER(AcsrSeg), _i32, _i32, _i32, _i32,
+                                                 _i32, _f32, _i32, _vp, _i64, _vp, _vp]),
 }
 EXPORTS = tuple(_SIGNATURES)
 

@@ -45,11 +45,14 @@ def attention_plan(segments: ACSRSegments, L: int, device) -> torch.Tensor:
 
 
 def attention_launcher(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor, output: torch.Tensor,
-                       segments: ACSRSegments, scale: float = 1.0, plan: torch.Tensor | None = None) -> torch.Tensor:
+                       segments: ACSRSegments, scale: float = 1.0, plan: torch.Tensor | None = None,
+                       lse: torch.Tensor | None = None) -> torch.Tensor:
     """Fused forward: output[b, h, r, :] = softmax over the live columns of (scale * q.kT)[b, h, r, :] times v.
     q [B, H, L, d], kT [B, H, d, L] (unit stride along d or along L), v [B, H, L, d], output [B, H, L, d];
     d in {64, 128}; one dtype for all four.  ``plan`` (from ``attention_plan`` for the same segments and L) spares
-    every workgroup the derivation of its tiles from the ACSR arrays; the results are the same."""
+    every workgroup the derivation of its tiles from the ACSR arrays; the results are the same.  ``lse`` (float32
+    [B, H, L], contiguous), when given, receives every row's log of the sum of exp(scale * score) over its live
+    columns (+inf for a row without any), so that the row's probabilities are exp(scale * score - lse)."""
     for name, t in (("q", q), ("kT", kT), ("v", v), ("output", output)):
         _hip.require_device_tensor(t, name)
         if t.dim() != 4:
@@ -74,14 +77,24 @@ def attention_launcher(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor, outpu
     args = (q.data_ptr(), qs[0], qs[1], qs[2], kT.data_ptr(), ks[0], ks[1], ks[2], ks[3],
             v.data_ptr(), vs[0], vs[1], vs[2], output.data_ptr(), os_[0], os_[1], os_[2],
             arr, len(segments), B, H, L, d, float(scale), _hip.dtype_code(q.dtype))
+    if plan is not None:
+        _hip.require_device_tensor(plan, "plan")
+        if plan.device != dev:
+            raise _hip.SplatError(f"the plan lives on {plan.device}, the tensors on {dev}")
+    if lse is not None:
+        _hip.require_device_tensor(lse, "lse")
+        if lse.dtype != torch.float32 or tuple(lse.shape) != (B, H, L) or not lse.is_contiguous() or lse.device != dev:
+            raise _hip.SplatError(f"lse must be a contiguous float32 tensor of shape {(B, H, L)} on {dev}")
     with torch.cuda.device(dev):
-        if plan is None:
+        if lse is not None:
+            rc = _hip.lib().splat_attention_fwd_stats(*args, plan.data_ptr() if plan is not None else None,
+                                                      plan.numel() * plan.element_size() if plan is not None else 0,
+                                                      lse.data_ptr(), _hip.stream_ptr(dev))
+            _hip.check(rc, "splat_attention_fwd_stats")
+        elif plan is None:
             rc = _hip.lib().splat_attention_fwd(*args, _hip.stream_ptr(dev))
             _hip.check(rc, "splat_attention_fwd")
         else:
-            _hip.require_device_tensor(plan, "plan")
-            if plan.device != dev:
-                raise _hip.SplatError(f"the plan lives on {plan.device}, the tensors on {dev}")
             rc = _hip.lib().splat_attention_fwd_planned(*args, plan.data_ptr(), plan.numel() * plan.element_size(),
                                                         _hip.stream_ptr(dev))
             _hip.check(rc, "splat_attention_fwd_planned")
@@ -127,6 +140,7 @@ class RegularAttention(nn.Module):
         self._unfused_ready = False
         self._plan = None  # the fused kernel's plan of this mask, built on the first fused forward
         self._segments_t = None  # ACSR of the transposed mask(s), built on the first backward
+        self._lse = None  # the rows' softmax statistics, allocated by the first forward_with_stats
         self._BLOCK_HEIGHT = BLOCK_SIZE_Y
 
     # The two [B, H, L, T] intermediates and the reference's launch geometry exist only for the unfused path.
@@ -190,6 +204,21 @@ class RegularAttention(nn.Module):
                        self.nnzs, self.rspmm_grid_dim, self.BLOCK_SIZE_Y, self.BLOCK_SIZE_X, segments=multi)
         return self.rspmm_output
 
+    def forward_with_stats(self, x):
+        """``forward(x)`` through the fused kernel plus every row's softmax statistic: returns ``(output, lse)`` with
+        ``lse`` float32 [B, H, L] = log of the row's sum of exp(scale * score) over its live columns (+inf for a row
+        without any).  Partial results over disjoint sets of keys merge exactly with it:
+        ``out = sum_i exp(lse_i - logsumexp_i(lse_i)) * out_i``."""
+        q, k, v = x
+        if not (q.shape[-1] in (64, 128) and q.dtype == k.dtype == v.dtype == self._out_dtype):
+            raise _hip.SplatError("the softmax statistic comes from the fused kernel: d in {64, 128}, one dtype")
+        if self._plan is None:
+            self._plan = attention_plan(self.segments, self._shape[2], self._device)
+            torch.cuda.current_stream(self._device).synchronize()
+        if self._lse is None:
+            self._lse = torch.empty(self._shape[:3], dtype=torch.float32, device=self._device)
+        attention_launcher(q, k, v, self.rspmm_output, self.segments, self.scale, self._plan, self._lse)
+        return self.rspmm_output, self._lse
 
     def backward_pass(self, x, grad_out: torch.Tensor):
         """Gradients (dq, dk, dv), each [B, H, L, d], of ``forward(x)`` for x = [q, kT, v] and the upstream gradient

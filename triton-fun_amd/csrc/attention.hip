@@ -43,6 +43,7 @@ struct AttnParams {
     int total;
     int row_stride;
     const PlanRec* plan;  // plan table of this mask (PLANNED kernels), variant already selected
+    float* lse;           // optional [B*H, L]: log of every row's sum of exponentials (natural log, scaled scores)
 };
 
 constexpr float kRescaleThreshold = 8.0f;  // in log2 units: exponentials stay below 2^8 before the reference moves
@@ -586,6 +587,12 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
         char* stg = smem + wave * (32 * OROW);
         const float l_tot = l_run + __shfl_xor(l_run, 32);
         const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+        if (p.lse != nullptr && g == 0) {
+            // probabilities are exp(scale * score - lse); a row without live columns gets +inf (every probability 0)
+            const int my_row = r0 + rs * (wave * 32 + lm);
+            const float lse = l_tot > 0.f ? (m_ref * p.scale_log2e + __log2f(l_tot)) * 0.6931471805599453f : __builtin_inff();
+            if (my_row < L) p.lse[(int64_t)bh * L + my_row] = lse;
+        }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -683,7 +690,7 @@ static int attention_fwd_common(const char* who, const void* q, int64_t q_sb, in
                                 int64_t v_sh, int64_t v_sl, void* out, int64_t o_sb, int64_t o_sh, int64_t o_sl,
                                 const splat_acsr_seg* segs, int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t d,
                                 float scale, int32_t dtype, const void* plan, int64_t plan_bytes, bool planned,
-                                void* stream) {
+                                float* lse, void* stream) {
     if (!q || !kT || !v || !out || !segs) return fail(SPLAT_E_NULL, "%s: null pointer argument", who);
     if (B <= 0 || H <= 0 || L <= 0) return fail(SPLAT_E_SHAPE, "%s: need B, H, L > 0 (got %d, %d, %d)", who, B, H, L);
     if (L > (1 << 23)) return fail(SPLAT_E_SHAPE, "%s: L is limited to 2^23 (got %d)", who, L);
@@ -725,6 +732,7 @@ static int attention_fwd_common(const char* who, const void* q, int64_t q_sb, in
     if (int rc = fill_segs(who, segs, n_seg, p.seg, -1)) return rc;
     p.row_stride = common_row_stride(segs, n_seg);
     p.plan = nullptr;
+    p.lse = lse;
     if (planned) {
         if (!plan) return fail(SPLAT_E_NULL, "%s: null plan", who);
         if ((reinterpret_cast<uintptr_t>(plan) & 15) != 0) return fail(SPLAT_E_ALIGN, "%s: the plan must be 16-byte aligned", who);
@@ -747,7 +755,7 @@ extern "C" int splat_attention_fwd(const void* q, int64_t q_sb, int64_t q_sh, in
                                    const splat_acsr_seg* segs, int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t d,
                                    float scale, int32_t dtype, void* stream) {
     return attention_fwd_common("splat_attention_fwd", q, q_sb, q_sh, q_sl, kT, k_sb, k_sh, k_sd, k_sl, v, v_sb, v_sh, v_sl, out,
-                                o_sb, o_sh, o_sl, segs, n_seg, B, H, L, d, scale, dtype, nullptr, 0, false, stream);
+                                o_sb, o_sh, o_sl, segs, n_seg, B, H, L, d, scale, dtype, nullptr, 0, false, nullptr, stream);
 }
 
 extern "C" int splat_attention_fwd_planned(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT,
@@ -758,7 +766,20 @@ extern "C" int splat_attention_fwd_planned(const void* q, int64_t q_sb, int64_t 
                                            int64_t plan_bytes, void* stream) {
     return attention_fwd_common("splat_attention_fwd_planned", q, q_sb, q_sh, q_sl, kT, k_sb, k_sh, k_sd, k_sl, v, v_sb, v_sh,
                                 v_sl, out, o_sb, o_sh, o_sl, segs, n_seg, B, H, L, d, scale, dtype, plan, plan_bytes, true,
-                                stream);
+                                nullptr, stream);
+}
+
+extern "C" int splat_attention_fwd_stats(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT,
+                                         int64_t k_sb, int64_t k_sh, int64_t k_sd, int64_t k_sl, const void* v,
+                                         int64_t v_sb, int64_t v_sh, int64_t v_sl, void* out, int64_t o_sb, int64_t o_sh,
+                                         int64_t o_sl, const splat_acsr_seg* segs, int32_t n_seg, int32_t B, int32_t H,
+                                         int32_t L, int32_t d, float scale, int32_t dtype, const void* plan,
+                                         int64_t plan_bytes, float* lse, void* stream) {
+    const char* who = "splat_attention_fwd_stats";
+    if (!lse) return fail(SPLAT_E_NULL, "%s: null lse", who);
+    if ((reinterpret_cast<uintptr_t>(lse) & 3) != 0) return fail(SPLAT_E_ALIGN, "%s: lse must be 4-byte aligned", who);
+    return attention_fwd_common(who, q, q_sb, q_sh, q_sl, kT, k_sb, k_sh, k_sd, k_sl, v, v_sb, v_sh, v_sl, out, o_sb, o_sh,
+                                o_sl, segs, n_seg, B, H, L, d, scale, dtype, plan, plan_bytes, plan != nullptr, lse, stream);
 }
 
 extern "C" int64_t splat_attention_plan_bytes(const splat_acsr_seg* segs, int32_t n_seg, int32_t L) {
