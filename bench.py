@@ -226,6 +226,10 @@ def main() -> int:
         _, pr = time_launches(lambda: attn4.backward_pass([q4, k4T, v4], g4), 10, 3)
         ms = sum(pr) / len(pr)
         extras["backward_cfg4"] = {"ms": round(ms, 3), "tflops_nnz": round(10 * d4 * nnz4 * B4 * H4 / ms / 1e9, 2)}
+        _, lse4 = attn4.forward_with_stats([q4, k4T, v4])
+        _, pr = time_launches(lambda: attn4.backward_pass([q4, k4T, v4], g4, lse4), 10, 3)
+        ms = sum(pr) / len(pr)
+        extras["backward_cfg4_with_forward_lse"] = {"ms": round(ms, 3), "tflops_nnz": round(10 * d4 * nnz4 * B4 * H4 / ms / 1e9, 2)}
         del attn4, g4, q4, k4, v4
     out["extras"] = extras
 

@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define SPLAT_VERSION 400 /* major*10000 + minor*100 + patch; 0.2.0 added the planned forward, 0.3.0 splat_spmm_t, 0.4.0 splat_attention_fwd_stats */
+#define SPLAT_VERSION 400 /* major*10000 + minor*100 + patch; 0.2.0 added the planned forward, 0.3.0 splat_spmm_t, 0.4.0 splat_attention_fwd_stats, splat_sddmm_probs */
 
 /* element types of q/k/v/score/output buffers */
 #define SPLAT_F32 0
@@ -128,6 +128,16 @@ int splat_sddmm(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const v
                 const splat_acsr_seg* segs /* host */, int32_t n_seg, int32_t B, int32_t H,
                 int32_t L, int32_t n_keys, int32_t d, int32_t T, float scale, int32_t in_dtype,
                 int32_t out_dtype, void* stream);
+
+/* splat_sddmm whose stored value is exp(scale * score - lse[(b*H + h)*L + r]) instead of scale * score: the
+ * row's softmax probabilities when lse is the row statistic of splat_attention_fwd_stats, written in one pass
+ * (rsddmm_launcher followed by rsoftmax_launcher, r_attention.py:80-90, without the second pass over the
+ * compressed matrix).  Used by the backward pass, which has the statistic from the forward. */
+int splat_sddmm_probs(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT,
+                      int64_t k_sb, int64_t k_sh, int64_t k_sd, int64_t k_sl, void* out,
+                      const splat_acsr_seg* segs /* host */, int32_t n_seg, int32_t B, int32_t H,
+                      int32_t L, int32_t n_keys, int32_t d, int32_t T, float scale, int32_t in_dtype,
+                      int32_t out_dtype, const float* lse, void* stream);
 
 /* Row softmax over the live slots of compressed rows: y[bh,r,s] = exp(x[bh,r,s]-max_r)/sum_r.
  * Replaces rsoftmax_launcher / r_softmax_1d_kernel, r_softmax.py:16-59,126-150, applied to every

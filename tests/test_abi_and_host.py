@@ -23,7 +23,7 @@ def header_symbols():
 def test_library_exports_every_declared_symbol():
     syms = header_symbols()
     assert {"splat_acsr_build", "splat_mask_generate", "splat_sddmm", "splat_softmax", "splat_spmm",
-            "splat_attention_fwd", "splat_attention_plan_bytes", "splat_attention_plan", "splat_attention_fwd_planned", "splat_attention_fwd_stats",
+            "splat_attention_fwd", "splat_attention_plan_bytes", "splat_attention_plan", "splat_attention_fwd_planned", "splat_attention_fwd_stats", "splat_sddmm_probs",
             "splat_version", "splat_last_error"} <= set(syms)
     handle = ctypes.CDLL(hip.LIB_PATH)
     for s in syms:

@@ -50,6 +50,42 @@ def test_gradients_against_dense_attention(dev, case, dtype):
         assert float((g.float().cpu() - w).abs().max()) <= TOL[dtype], name
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", _cases(), ids=lambda c: c[0])
+def test_probabilities_in_one_pass_and_gradients_with_the_forward_statistic(dev, case, dtype):
+    """rsddmm_launcher(..., lse=) stores exp(scale * score - lse): with the statistic of the fused forward these are
+    the probabilities that rsddmm + rsoftmax give (live slots equal within the type's rounding, dead slots untouched),
+    and the backward pass that starts from them meets the oracle's gradients like the one that recomputes the softmax."""
+    from r_sddmm import rsddmm_launcher
+    from r_softmax import rsoftmax_launcher
+    _, make, dense, L = case
+    B, H, d = 2, 2, 64
+    scale = d ** -0.5
+    q, k, v = O.make_inputs(3 * L, B, H, L, d, dtype)
+    go = O.make_inputs(3 * L + 1, B, H, L, d, dtype)[0]
+    attn = RegularAttention(B, L, H, d, make(), 16, 16, dev, dtype, scale=scale)
+    qd, kd, vd = [t.to(dev) for t in (q, k, v)]
+    kT = kd.transpose(2, 3)
+    _, lse = attn.forward_with_stats([qd, kT, vd])
+    segs, T = attn.segments, attn.segments.T
+    two = torch.full((B, H, L, T), 5, dtype=dtype, device=dev)
+    rsddmm_launcher(qd, kT, two, None, None, None, None, T, None, None, None, None, 16, 16, scale=scale, segments=segs)
+    rsoftmax_launcher(two, two, None, None, None, None, T, 0, None, None, 16, segments=segs)
+    one = torch.full((B, H, L, T), 5, dtype=dtype, device=dev)
+    rsddmm_launcher(qd, kT, one, None, None, None, None, T, None, None, None, None, 16, 16, scale=scale, segments=segs,
+                    lse=lse)
+    eps = {torch.float32: 2e-6, torch.float16: 2e-3, torch.bfloat16: 1.6e-2}[dtype]   # a few ulps of values <= 1
+    assert float((one.float() - two.float()).abs().max()) <= eps
+    assert torch.equal(one == 5, two == 5)   # the sentinel survives in exactly the same (dead) slots
+    want = O.dense_masked_attention_grads(q, k.transpose(2, 3), v, np.asarray(dense()), scale, go)
+    got = attn.backward_pass([qd, kT, vd], go.to(dev), lse)
+    for name, g, w in zip(("dq", "dk", "dv"), got, want):
+        assert float((g.float().cpu() - w).abs().max()) <= TOL[dtype], name
+    with pytest.raises(Exception, match="lse"):
+        rsddmm_launcher(qd, kT, one, None, None, None, None, T, None, None, None, None, 16, 16, scale=scale, segments=segs,
+                        lse=lse[:, :1])
+
+
 def test_softmax_backward_on_compressed_rows(dev):
     L = 200
     acsr = O.create_acsr(O.create_causal_windowed_mask(L, 30), 16)

@@ -44,6 +44,8 @@ _SIGNATURES = {
     "splat_acsr_build_pattern": (ctypes.c_int, [_i32, _i64, _i64, _i64, _i32] + [_vp] * 10 + [_vp]),
     "splat_sddmm": (ctypes.c_int, [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, ctypes.POINTER(AcsrSeg), _i32,
                                    _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _i32, _vp]),
+    "splat_sddmm_probs": (ctypes.c_int, [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, ctypes.POINTER(AcsrSeg), _i32,
+                                         _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _i32, _vp, _vp]),
     "splat_softmax": (ctypes.c_int, [_vp, _vp, ctypes.POINTER(AcsrSeg), _i32, _i64, _i32, _i32, _i32, _i32, _vp]),
     "splat_spmm": (ctypes.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, ctypes.POINTER(AcsrSeg), _i32, _i32, _i32, _i32, _i32,
                                   _i32, _i32, _i32, _i32, _vp]),

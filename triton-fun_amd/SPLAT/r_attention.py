@@ -220,28 +220,34 @@ class RegularAttention(nn.Module):
         attention_launcher(q, k, v, self.rspmm_output, self.segments, self.scale, self._plan, self._lse)
         return self.rspmm_output, self._lse
 
-    def backward_pass(self, x, grad_out: torch.Tensor):
+    def backward_pass(self, x, grad_out: torch.Tensor, lse: torch.Tensor | None = None):
         """Gradients (dq, dk, dv), each [B, H, L, d], of ``forward(x)`` for x = [q, kT, v] and the upstream gradient
-        ``grad_out`` [B, H, L, d].  The ACSR of the transposed mask is built on first use; see ``r_backward``."""
+        ``grad_out`` [B, H, L, d].  The ACSR of the transposed mask is built on first use; see ``r_backward``.  ``lse``:
+        the rows' statistic of ``forward_with_stats`` for the same x, which spares the backward its softmax pass."""
         from r_backward import attention_backward, transposed_segments
         q, kT, v = x
         if self._segments_t is None:
             masks = self._mask if _is_segment_list(self._mask) else [self._mask]
             self._segments_t = transposed_segments(masks, self._BLOCK_HEIGHT, self._GPU_ID)
-        return attention_backward(q, kT, v, grad_out, self.segments, self._segments_t, self.scale)
+        return attention_backward(q, kT, v, grad_out, self.segments, self._segments_t, self.scale, lse)
 
 
 class _AttentionFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, attn):
-        ctx.save_for_backward(q, k, v)
         ctx.attn = attn
-        return attn([q, k.transpose(2, 3), v]).clone()  # the module's buffer is reused by the next call
+        if attn.fused and q.shape[-1] in (64, 128) and q.dtype == k.dtype == v.dtype == attn._out_dtype:
+            out, lse = attn.forward_with_stats([q, k.transpose(2, 3), v])
+            ctx.save_for_backward(q, k, v, lse.clone())
+        else:
+            out = attn([q, k.transpose(2, 3), v])
+            ctx.save_for_backward(q, k, v)
+        return out.clone()  # the module's buffers are reused by the next call
 
     @staticmethod
     def backward(ctx, grad_out):
-        q, k, v = ctx.saved_tensors
-        dq, dk, dv = ctx.attn.backward_pass([q, k.transpose(2, 3), v], grad_out)
+        q, k, v, *stat = ctx.saved_tensors
+        dq, dk, dv = ctx.attn.backward_pass([q, k.transpose(2, 3), v], grad_out, stat[0] if stat else None)
         return dq, dk, dv, None
 
 

@@ -4,7 +4,7 @@ The reference stops at the forward (``r_attention.py:77-100``); this module give
 ``out = softmax_over_live_columns(scale * q.kT) . v`` with respect to q, k and v.  Everything stays in the compressed
 [B, H, L, T] layout:
 
-    S~  = rsddmm(q, kT) * scale            P~ = rsoftmax(S~)
+    S~  = rsddmm(q, kT) * scale            P~ = rsoftmax(S~)      (or P~ = exp(S~ - lse) in one pass, given the forward's lse)
     dP~ = rsddmm(dO, v^T)                  dS~ = P~ o (dP~ - rowsum(P~ o dP~)) * scale     (splat_softmax_bwd)
     dQ  = rspmm(dS~, k)
     dV  = P~^T . dO                        dK = dS~^T . q                                   (splat_spmm_t)
@@ -120,8 +120,9 @@ def rspmm_t_launcher(p: torch.Tensor, x: torch.Tensor, out: torch.Tensor, segmen
     return out
 
 
-def _sddmm(x, y, out, segs, scale):
-    rsddmm_launcher(x, y, out, None, None, None, None, segs.T, None, None, None, None, 16, 16, scale=scale, segments=segs)
+def _sddmm(x, y, out, segs, scale, lse=None):
+    rsddmm_launcher(x, y, out, None, None, None, None, segs.T, None, None, None, None, 16, 16, scale=scale, segments=segs,
+                    lse=lse)
 
 
 def _spmm(p, v, out, segs):
@@ -129,10 +130,13 @@ def _spmm(p, v, out, segs):
 
 
 def attention_backward(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor, grad_out: torch.Tensor,
-                       segments: ACSRSegments, segments_t: ACSRSegments, scale: float = 1.0):
+                       segments: ACSRSegments, segments_t: ACSRSegments, scale: float = 1.0,
+                       lse: torch.Tensor | None = None):
     """(dq, dk, dv), each [B, H, L, d], for out = softmax_over_live_columns(scale * q.kT) . v and the upstream gradient
     ``grad_out`` [B, H, L, d].  q, v [B, H, L, d]; kT [B, H, d, L] (a view or a copy); one dtype throughout.  The
-    probabilities are recomputed (SDDMM + softmax), as the fused forward never materialises them."""
+    probabilities are recomputed, as the fused forward never materialises them: by SDDMM + softmax, or, with the rows'
+    statistic ``lse`` [B, H, L] of the forward (``RegularAttention.forward_with_stats``), by one SDDMM that stores
+    exp(scale * score - lse)."""
     B, H, L, d = q.shape
     dt, dev = q.dtype, q.device
     k = kT.transpose(2, 3)
@@ -141,8 +145,9 @@ def attention_backward(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor, grad_
     grad_out = grad_out.contiguous() if grad_out.stride(3) != 1 else grad_out
     T = segments.T
     probs = torch.empty((B, H, L, T), dtype=dt, device=dev)
-    _sddmm(q, kT, probs, segments, scale)
-    rsoftmax_launcher(probs, probs, None, None, None, None, T, 0, None, None, 16, segments=segments)
+    _sddmm(q, kT, probs, segments, scale, lse)
+    if lse is None:
+        rsoftmax_launcher(probs, probs, None, None, None, None, T, 0, None, None, 16, segments=segments)
     dprobs = torch.empty_like(probs)
     _sddmm(grad_out, v.transpose(2, 3), dprobs, segments, 1.0)
     softmax_backward_launcher(probs, dprobs, dprobs, segments, scale)  # dprobs now holds dS~

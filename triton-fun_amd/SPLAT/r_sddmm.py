@@ -68,11 +68,13 @@ def rsddmm_launcher(x: torch.Tensor, y: torch.Tensor, output: torch.Tensor,
                     trailing_dim: int, nnzs: torch.Tensor, grid_dim: tuple[int],
                     tb_map_x: torch.Tensor, tb_map_y: torch.Tensor,
                     BLOCK_SIZE_Y: int, BLOCK_SIZE_X: int, *, scale: float | None = None,
-                    segments: ACSRSegments | None = None):
+                    segments: ACSRSegments | None = None, lse: torch.Tensor | None = None):
     """x = Q [B, H, L, d]; y = K^T [B, H, d, L] (any strides with unit stride along d or along L, so
     ``k.transpose(2, 3)`` of a [B, H, L, d] tensor needs no copy); output [B, H, L, T] is written in place for
     the live slots only.  ``grid_dim`` / ``tb_map_*`` / ``BLOCK_SIZE_*`` describe the reference's launch
-    geometry and are accepted unchanged; the HIP kernel tiles by itself from the row maps.
+    geometry and are accepted unchanged; the HIP kernel tiles by itself from the row maps.  With ``lse`` (float32
+    [B, H, L], contiguous: every row's log of its sum of exp(scale * score), as the fused forward hands it out) the
+    stored value is exp(scale * score - lse[row]), the row's softmax probability, instead of the score.
     Returns (output, sTod_linear_transformations, sTod_translations, nnzs)."""
     for name, t in (("x", x), ("y", y), ("output", output)):
         _hip.require_device_tensor(t, name)
@@ -93,10 +95,18 @@ def rsddmm_launcher(x: torch.Tensor, y: torch.Tensor, output: torch.Tensor,
     qs, ks = _strides4(x, "x"), _strides4(y, "y")
     dev = x.device
     arr = _hip.seg_array(segs.seg_args())
+    args = (x.data_ptr(), qs[0], qs[1], qs[2], y.data_ptr(), ks[0], ks[1], ks[2], ks[3], output.data_ptr(), arr, len(segs),
+            B, H, L, n_keys, d, trailing_dim, 1.0 if scale is None else float(scale), _hip.dtype_code(x.dtype),
+            _hip.dtype_code(output.dtype))
+    if lse is not None:
+        _hip.require_device_tensor(lse, "lse")
+        if lse.dtype != torch.float32 or tuple(lse.shape) != (B, H, L) or not lse.is_contiguous() or lse.device != dev:
+            raise _hip.SplatError(f"lse must be a contiguous float32 tensor of shape {(B, H, L)} on {dev}")
     with torch.cuda.device(dev):
-        rc = _hip.lib().splat_sddmm(x.data_ptr(), qs[0], qs[1], qs[2], y.data_ptr(), ks[0], ks[1], ks[2], ks[3],
-                                    output.data_ptr(), arr, len(segs), B, H, L, n_keys, d, trailing_dim,
-                                    1.0 if scale is None else float(scale), _hip.dtype_code(x.dtype),
-                                    _hip.dtype_code(output.dtype), _hip.stream_ptr(dev))
-    _hip.check(rc, "splat_sddmm")
+        if lse is None:
+            rc = _hip.lib().splat_sddmm(*args, _hip.stream_ptr(dev))
+            _hip.check(rc, "splat_sddmm")
+        else:
+            rc = _hip.lib().splat_sddmm_probs(*args, lse.data_ptr(), _hip.stream_ptr(dev))
+            _hip.check(rc, "splat_sddmm_probs")
     return (output, sTod_linear_transformations, sTod_translations, nnzs)

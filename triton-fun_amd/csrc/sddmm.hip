@@ -11,6 +11,7 @@
 // positions are never stored.  The kernel is bound by the compressed output (HBM), not by MFMA: 2*d flops per
 // 2-4 output bytes.
 #include <algorithm>
+#include <type_traits>
 
 #include "acsr_plan.hpp"
 
@@ -24,6 +25,7 @@ struct SddmmParams {
     int64_t k_sb, k_sh, k_sd, k_sl;
     int B, H, L, n_keys, d, T;
     float scale;
+    const float* row_lse;  // optional [B*H, L]: the output is exp(scale * score - row_lse[row]) instead of scale * score
     int out_dtype;
     int n_seg;
     SegPtrs seg[SPLAT_MAX_SEGMENTS];
@@ -77,7 +79,7 @@ __device__ __forceinline__ void store_piece(TO* row_out, const RowWin& w, int jj
 
 // KSU: 0 = the contraction is longer than one LDS chunk (Q fragments are re-read per chunk); otherwise Q stays in
 // registers, and KSU > 0 says at compile time how many MFMA steps hold data (-1: known at run time only).
-template <typename T, bool KT, int KSU>
+template <typename T, bool KT, int KSU, bool PROBS>
 __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
     constexpr bool QREG = KSU != 0;
     constexpr int ES = sizeof(T);
@@ -128,6 +130,11 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
     // B-operand row of this lane: query row 32*wave + lm of the block
     const int q_row = min(r0 + rs * (32 * wave + lm), L - 1);
     const T* qr = qb + (int64_t)q_row * p.q_sl;
+    // with a row statistic: exp(scale * s - lse) = exp2(s * exp_mul - exp_sub), stored as it is
+    const float out_scale = PROBS ? 1.0f : p.scale;
+    const float exp_mul = p.scale * 1.4426950408889634f;
+    float exp_sub = 0.f;
+    if constexpr (PROBS) exp_sub = p.row_lse[(int64_t)bh * L + q_row] * 1.4426950408889634f;
     Frag<T> qf[KSC];
     if constexpr (QREG) {
 #pragma unroll
@@ -323,6 +330,12 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
             for (int i = 0; i < CPT; ++i) asm volatile("" ::"v"(kreg[i]));
 #endif
             if (skip) continue;
+            if constexpr (PROBS) {  // probabilities of a softmax whose row statistic is known
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) acc[nt][j] = fast_exp2(fmaf(acc[nt][j], exp_mul, -exp_sub));
+            }
 
             // every position of the tile is a slot of every row of this wavefront: no tests, one vector store per piece
             const bool full = (j0 >= span.lo_max) && (j0 + kBN <= span.hi_min);
@@ -333,8 +346,8 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
                     // ---- turn the half tile around: lane (query lm, half g) holds positions 8jq + 4g + {0..3} ----
 #pragma unroll
                     for (int jq = 0; jq < 4; ++jq) {
-                        f32x4 v4 = {acc[nt][4 * jq] * p.scale, acc[nt][4 * jq + 1] * p.scale, acc[nt][4 * jq + 2] * p.scale,
-                                    acc[nt][4 * jq + 3] * p.scale};
+                        f32x4 v4 = {acc[nt][4 * jq] * out_scale, acc[nt][4 * jq + 1] * out_scale, acc[nt][4 * jq + 2] * out_scale,
+                                    acc[nt][4 * jq + 3] * out_scale};
                         *reinterpret_cast<f32x4*>(stg + lm * S_ROW + (8 * jq + 4 * g) * 4) = v4;
                     }
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wavefront's LDS writes are visible to its own reads
@@ -371,7 +384,7 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
                     for (int jq = 0; jq < 4; ++jq) {
                         v4 t;
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) t[i] = (TO)(acc[nt][4 * jq + i] * p.scale);
+                        for (int i = 0; i < 4; ++i) t[i] = (TO)(acc[nt][4 * jq + i] * out_scale);
                         const int ri = (j0 + 32 * nt + 8 * jq + 4 * g - lo4) & (R_SLOTS - 1);
                         *reinterpret_cast<v4*>(ring_row + ri * 2) = t;
                         if (ri == 0) *reinterpret_cast<v4*>(ring_row + R_SLOTS * 2) = t;
@@ -425,53 +438,60 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
 }
 
 template <typename T>
-static int launch_sddmm(SddmmParams p, bool kt, hipStream_t st) {
+static int launch_sddmm(const char* who, SddmmParams p, bool kt, hipStream_t st) {
     p.n_row_blocks = count_row_blocks(p.L, 128, p.row_stride);
     // Few row blocks (one head of a short sequence, the reference's own benchmark shape) would leave most of the 256
     // compute units idle: share every row block's tiles out over several workgroups then.
     const int64_t blocks = (int64_t)p.B * p.H * p.n_row_blocks;
-    if (blocks > 0x7ffffff0) return fail(SPLAT_E_SHAPE, "splat_sddmm: problem too large for one launch");
+    if (blocks > 0x7ffffff0) return fail(SPLAT_E_SHAPE, "%s: problem too large for one launch", who);
     p.key_split = blocks >= 512 ? 1 : (int)std::min<int64_t>(32, (768 + blocks - 1) / blocks);
     p.total = (int)(blocks * p.key_split);
     const int grid = ((p.total + 7) / 8) * 8;
     constexpr int DC = SddmmGeom<T>::DC, KSC = DC / 16;
     const int steps = (p.d + 15) / 16;
-    if (kt) {
-        if (p.d <= DC)
-            sddmm_kernel<T, true, -1><<<grid, 256, 0, st>>>(p);
-        else
-            sddmm_kernel<T, true, 0><<<grid, 256, 0, st>>>(p);
-    } else {
-        if (p.d > DC)
-            sddmm_kernel<T, false, 0><<<grid, 256, 0, st>>>(p);
-        else if (steps == KSC)
-            sddmm_kernel<T, false, KSC><<<grid, 256, 0, st>>>(p);
-        else if (steps == KSC / 2)
-            sddmm_kernel<T, false, KSC / 2><<<grid, 256, 0, st>>>(p);
-        else
-            sddmm_kernel<T, false, -1><<<grid, 256, 0, st>>>(p);
-    }
-    return check_launch("splat_sddmm");
+    auto go = [&](auto probs_c) {
+        constexpr bool PROBS = decltype(probs_c)::value;
+        if (kt) {
+            if (p.d <= DC)
+                sddmm_kernel<T, true, -1, PROBS><<<grid, 256, 0, st>>>(p);
+            else
+                sddmm_kernel<T, true, 0, PROBS><<<grid, 256, 0, st>>>(p);
+        } else {
+            if (p.d > DC)
+                sddmm_kernel<T, false, 0, PROBS><<<grid, 256, 0, st>>>(p);
+            else if (steps == KSC)
+                sddmm_kernel<T, false, KSC, PROBS><<<grid, 256, 0, st>>>(p);
+            else if (steps == KSC / 2)
+                sddmm_kernel<T, false, KSC / 2, PROBS><<<grid, 256, 0, st>>>(p);
+            else
+                sddmm_kernel<T, false, -1, PROBS><<<grid, 256, 0, st>>>(p);
+        }
+    };
+    if (p.row_lse != nullptr)
+        go(std::true_type{});
+    else
+        go(std::false_type{});
+    return check_launch(who);
 }
 
 }  // namespace splat
 
 using namespace splat;
 
-extern "C" int splat_sddmm(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT, int64_t k_sb, int64_t k_sh,
-                           int64_t k_sd, int64_t k_sl, void* out, const splat_acsr_seg* segs, int32_t n_seg, int32_t B, int32_t H,
-                           int32_t L, int32_t n_keys, int32_t d, int32_t T, float scale, int32_t in_dtype, int32_t out_dtype,
-                           void* stream) {
-    if (!q || !kT || !out || !segs) return fail(SPLAT_E_NULL, "splat_sddmm: null pointer argument");
+static int sddmm_common(const char* who, const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT, int64_t k_sb,
+                        int64_t k_sh, int64_t k_sd, int64_t k_sl, void* out, const splat_acsr_seg* segs, int32_t n_seg, int32_t B,
+                        int32_t H, int32_t L, int32_t n_keys, int32_t d, int32_t T, float scale, int32_t in_dtype,
+                        int32_t out_dtype, const float* row_lse, void* stream) {
+    if (!q || !kT || !out || !segs) return fail(SPLAT_E_NULL, "%s: null pointer argument", who);
     if (B <= 0 || H <= 0 || L <= 0 || n_keys <= 0 || d <= 0 || T <= 0)
-        return fail(SPLAT_E_SHAPE, "splat_sddmm: need B, H, L, n_keys, d, T > 0 (got %d, %d, %d, %d, %d, %d)", B, H, L, n_keys, d, T);
-    if (L > (1 << 23) || n_keys > (1 << 23)) return fail(SPLAT_E_SHAPE, "splat_sddmm: L and n_keys are limited to 2^23");
+        return fail(SPLAT_E_SHAPE, "%s: need B, H, L, n_keys, d, T > 0 (got %d, %d, %d, %d, %d, %d)", who, B, H, L, n_keys, d, T);
+    if (L > (1 << 23) || n_keys > (1 << 23)) return fail(SPLAT_E_SHAPE, "%s: L and n_keys are limited to 2^23", who);
     if (out_dtype != SPLAT_F32 && out_dtype != SPLAT_F16 && out_dtype != SPLAT_BF16)
-        return fail(SPLAT_E_DTYPE, "splat_sddmm: unknown out_dtype %d", out_dtype);
+        return fail(SPLAT_E_DTYPE, "%s: unknown out_dtype %d", who, out_dtype);
     if (in_dtype != SPLAT_F32 && in_dtype != SPLAT_F16 && in_dtype != SPLAT_BF16)
-        return fail(SPLAT_E_DTYPE, "splat_sddmm: unknown in_dtype %d", in_dtype);
+        return fail(SPLAT_E_DTYPE, "%s: unknown in_dtype %d", who, in_dtype);
     if (k_sd != 1 && k_sl != 1)
-        return fail(SPLAT_E_ALIGN, "splat_sddmm: kT needs unit stride along d (k_sd == 1) or along keys (k_sl == 1); got k_sd=%lld k_sl=%lld",
+        return fail(SPLAT_E_ALIGN, "%s: kT needs unit stride along d (k_sd == 1) or along keys (k_sl == 1); got k_sd=%lld k_sl=%lld", who,
                     (long long)k_sd, (long long)k_sl);
     SddmmParams p;
     p.q = q; p.k = kT; p.out = out;
@@ -479,9 +499,10 @@ extern "C" int splat_sddmm(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_
     p.k_sb = k_sb; p.k_sh = k_sh; p.k_sd = k_sd; p.k_sl = k_sl;
     p.B = B; p.H = H; p.L = L; p.n_keys = n_keys; p.d = d; p.T = T;
     p.scale = scale;
+    p.row_lse = row_lse;
     p.out_dtype = out_dtype;
     p.n_seg = n_seg;
-    if (int rc = fill_segs("splat_sddmm", segs, n_seg, p.seg, T)) return rc;
+    if (int rc = fill_segs(who, segs, n_seg, p.seg, T)) return rc;
     p.row_stride = common_row_stride(segs, n_seg);
     const int es = in_dtype == SPLAT_F32 ? 4 : 2;
     const int epc = 16 / es;
@@ -496,8 +517,27 @@ extern "C" int splat_sddmm(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_
         if (segs[k].slot_offset % 8 != 0) p.out_vec = 0;
     hipStream_t st = (hipStream_t)stream;
     switch (in_dtype) {
-        case SPLAT_F32: return launch_sddmm<float>(p, kt, st);
-        case SPLAT_F16: return launch_sddmm<f16>(p, kt, st);
-        default: return launch_sddmm<bf16>(p, kt, st);
+        case SPLAT_F32: return launch_sddmm<float>(who, p, kt, st);
+        case SPLAT_F16: return launch_sddmm<f16>(who, p, kt, st);
+        default: return launch_sddmm<bf16>(who, p, kt, st);
     }
+}
+
+extern "C" int splat_sddmm(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT, int64_t k_sb, int64_t k_sh,
+                           int64_t k_sd, int64_t k_sl, void* out, const splat_acsr_seg* segs, int32_t n_seg, int32_t B, int32_t H,
+                           int32_t L, int32_t n_keys, int32_t d, int32_t T, float scale, int32_t in_dtype, int32_t out_dtype,
+                           void* stream) {
+    return sddmm_common("splat_sddmm", q, q_sb, q_sh, q_sl, kT, k_sb, k_sh, k_sd, k_sl, out, segs, n_seg, B, H, L, n_keys, d, T,
+                        scale, in_dtype, out_dtype, nullptr, stream);
+}
+
+extern "C" int splat_sddmm_probs(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT, int64_t k_sb,
+                                 int64_t k_sh, int64_t k_sd, int64_t k_sl, void* out, const splat_acsr_seg* segs, int32_t n_seg,
+                                 int32_t B, int32_t H, int32_t L, int32_t n_keys, int32_t d, int32_t T, float scale,
+                                 int32_t in_dtype, int32_t out_dtype, const float* lse, void* stream) {
+    const char* who = "splat_sddmm_probs";
+    if (!lse) return fail(SPLAT_E_NULL, "%s: null lse", who);
+    if ((reinterpret_cast<uintptr_t>(lse) & 3) != 0) return fail(SPLAT_E_ALIGN, "%s: lse must be 4-byte aligned", who);
+    return sddmm_common(who, q, q_sb, q_sh, q_sl, kT, k_sb, k_sh, k_sd, k_sl, out, segs, n_seg, B, H, L, n_keys, d, T, scale,
+                        in_dtype, out_dtype, lse, stream);
 }
