@@ -77,6 +77,39 @@ def test_config4_dilated(dev, fused, contig):
     assert float((got - want).abs().max()) <= TOL[torch.bfloat16]
 
 
+@pytest.mark.parametrize("cfg", [3, 4])
+def test_config3_and_config4_at_full_batch_and_heads(dev, cfg):
+    """Configs 3 (B=2, H=16, L=8192, d=64, strided, two segments) and 4 (B=2, H=32, L=8192, d=128, dilated 512/2) at
+    their full size, fused and unfused: the first and the last (batch, head) pair against the oracle, every pair through
+    V = 1 gives 1."""
+    if cfg == 3:
+        B, H, L, d = 2, 16, 8192, 64
+        pat = A.strided_patterns(L, 128, 128)
+        segs = O.create_strided_segment_masks(L, 128, 128)
+        dense = segs[0] | segs[1]
+    else:
+        B, H, L, d = 2, 32, 8192, 128
+        pat = A.dilated_pattern(L, 512, 2)
+        dense = O.create_dilated_mask(L, 512, 2)
+    scale = d ** -0.5
+    q, k, v = O.make_inputs(1000 + cfg, B, H, L, d, torch.bfloat16)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    kT = kd.transpose(2, 3)
+    wants = {}
+    for b, h in ((0, 0), (B - 1, H - 1)):
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        wants[(b, h)] = (sl, O.dense_masked_attention_chunked(q[sl], k[sl].transpose(2, 3), v[sl],
+                                                              lambda a, c: dense[a:c] != 0, scale))
+    for fused in (True, False):
+        attn = RegularAttention(B, L, H, d, pat, 16, 16, dev, torch.bfloat16, scale=scale, fused=fused)
+        got = attn([qd, kT, vd]).float().cpu()
+        for sl, want in wants.values():
+            assert float((got[sl] - want).abs().max()) <= TOL[torch.bfloat16], fused
+        ones = attn([qd, kT, torch.ones_like(vd)]).float()
+        assert float((ones - 1).abs().max()) <= TOL[torch.bfloat16], fused
+        del attn
+
+
 def test_config5_headline_full_size(dev):
     """B=4, H=16, L=16384, d=128, bf16, causal window 512, fused only: the full problem runs on the GPU;
     two (batch, head) pairs are checked against the oracle, the rest through properties that do not depend on
