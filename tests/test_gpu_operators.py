@@ -76,6 +76,37 @@ def test_sddmm_patterns(dev, dtype, layout, make, d):
     assert torch.all(got[..., ~lv] == SENTINEL)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("layout", ["view", "contig"])
+@pytest.mark.parametrize("make,d", [
+    (lambda: O.create_causal_windowed_mask(1024, 511), 64),   # whole-line output path of the 16-bit types
+    (lambda: O.create_windowed_mask(300, 20), 40), (lambda: O.create_dilated_mask(256, 32, 2), 128),
+    (lambda: O.create_blocked_mask(200, 33), 200), (lambda: O.create_causal_windowed_mask(130, 9), 10)])
+def test_sddmm_probabilities_from_a_row_statistic(dev, dtype, layout, make, d):
+    """rsddmm_launcher(..., lse=): exp(scale * score - lse[row]) in the live slots, nothing in the dead ones; with
+    lse = torch.logsumexp of the row's live scaled scores that is the oracle's compressed softmax of its SDDMM.  Head
+    widths the fused kernel does not take, contractions longer than one staging chunk, both K layouts."""
+    mask = make()
+    L = mask.shape[0]
+    q, k, _ = O.make_inputs(13, 2, 3, L, d, dtype)
+    acsr, acsr_np = acsr_pair(mask, 16, dev)
+    scale = d ** -0.5
+    scores = torch.einsum("bhqd,bhkd->bhqk", q.float(), k.float()) * scale
+    lse = torch.logsumexp(scores.masked_fill(torch.as_tensor(mask == 0), float("-inf")), dim=-1)
+    want = O.softmax_compressed(O.sddmm(q, k.transpose(2, 3), acsr_np, scale), live(acsr_np))
+    kT_dev = k.to(dev).transpose(2, 3)
+    if layout == "contig":
+        kT_dev = kT_dev.contiguous()
+    out = torch.full((2, 3, L, acsr[5]), SENTINEL, dtype=dtype, device=dev)
+    r_sddmm.rsddmm_launcher(q.to(dev), kT_dev, out, acsr[0], acsr[1], acsr[2], acsr[3], acsr[5], acsr[4], (1, 1),
+                            None, None, 16, 16, scale=scale, lse=lse.to(dev).contiguous())
+    got = out.float().cpu()
+    lv = live(acsr_np)
+    tol = {torch.float32: 2e-6, torch.float16: 1e-3, torch.bfloat16: 8e-3}[dtype]   # rounding of values <= 1
+    assert float((got - want)[..., lv].abs().max()) <= tol
+    assert torch.all(got[..., ~lv] == SENTINEL)
+
+
 @pytest.mark.parametrize("in_dt,out_dt", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16),
                                           (torch.float32, torch.bfloat16)])
 @pytest.mark.parametrize("make,d", [
