@@ -148,17 +148,52 @@ def test_config5_headline_full_size(dev):
 def test_fused_small_patterns(dev, dtype, d, make):
     mask = make()
     L = mask.shape[0]
-    if dtype != torch.float32 and L % 8:
-        contigs = (False,)  # K^T contiguous along keys needs 16-byte rows
-    elif dtype == torch.float32 and L % 4:
-        contigs = (False,)
-    else:
-        contigs = (False, True)
     q, k, v = O.make_inputs(L + d, 2, 2, L, d, dtype)
     want = O.dense_masked_attention(q, k.transpose(2, 3), v, mask, d ** -0.5)
-    for contig in contigs:
+    for contig in (False, True):  # K^T contiguous along the keys is the reference's layout, whatever L is
         got = run_module(mask, 2, 2, L, d, dtype, dev, q, k, v, d ** -0.5, True, contig)
         assert float((got - want).abs().max()) <= TOL[dtype], contig
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("L", [333, 1001])
+def test_fused_reference_k_layout_with_ragged_length(dev, dtype, L):
+    """The reference hands kT over as a contiguous [B, H, d, L] tensor (r_sddmm.py:230-231, r_attention.py:134-137).
+    With L not a multiple of the 16-byte piece the key rows of that layout are not piece-aligned; the default (fused)
+    forward must still take it."""
+    d = 64
+    mask = O.create_causal_windowed_mask(L, 77)
+    q, k, v = O.make_inputs(7 * L, 1, 3, L, d, dtype)
+    want = O.dense_masked_attention(q, k.transpose(2, 3), v, mask, d ** -0.5)
+    attn = RegularAttention(1, L, 3, d, mask, 16, 16, dev, dtype, scale=d ** -0.5)
+    assert attn.fused
+    kT = k.to(dev).transpose(2, 3).contiguous()
+    assert kT.stride(3) == 1 and L % 8 != 0
+    got = attn([q.to(dev), kT, v.to(dev)]).float().cpu()
+    assert float((got - want).abs().max()) <= TOL[dtype]
+
+
+def test_fused_views_that_are_not_piece_aligned(dev):
+    """q, v and the output as views whose storage offset or row stride is not a multiple of 16 bytes: the launcher
+    copies what the kernel cannot address piecewise and still writes the caller's output tensor."""
+    B, H, L, d = 1, 2, 200, 64
+    dtype = torch.float16
+    mask = O.create_windowed_mask(L, 20)
+    q, k, v = O.make_inputs(99, B, H, L, d, dtype)
+    want = O.dense_masked_attention(q, k.transpose(2, 3), v, mask, d ** -0.5)
+    segs = A.create_acsr_segments([mask], 16, dev)
+
+    def odd_view(t):  # same values, rows d + 3 elements apart, first element 3 elements into the storage
+        buf = torch.zeros(B, H, L, d + 3, dtype=dtype, device=dev).flatten()
+        buf = torch.cat([buf, buf.new_zeros(8)])
+        view = buf[3:3 + B * H * L * (d + 3)].view(B, H, L, d + 3)[..., :d]
+        view.copy_(t.to(dev))
+        return view
+    qv, vv, ov = odd_view(q), odd_view(v), odd_view(torch.zeros_like(q))
+    assert qv.data_ptr() % 16 != 0 and qv.stride(2) % 8 != 0
+    res = attention_launcher(qv, k.to(dev).transpose(2, 3), vv, ov, segs, d ** -0.5)
+    assert res is ov
+    assert float((ov.float().cpu() - want).abs().max()) <= TOL[dtype]
 
 
 def test_empty_and_single_column_rows(dev):

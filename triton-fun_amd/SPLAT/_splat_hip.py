@@ -120,9 +120,13 @@ def require_device_tensor(t: torch.Tensor, name: str) -> None:
         raise SplatError(f"{name} must be a tensor on a HIP device")
 
 
-def seg_array(segments: Sequence[tuple]) -> Any:
+def seg_array(segments: Sequence[tuple], rows: int, trailing_dim: int | None = None) -> Any:
     """segments: (dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnzs, first_col | None, slot_offset); the row-stride
-    hint is read from the attribute ``splat_row_stride`` of sTod_trans when the builder attached one."""
+    hint is read from the attribute ``splat_row_stride`` of sTod_trans when the builder attached one.
+
+    ``rows`` is the number of mask rows the launch will index the arrays with (the C ABI takes bare pointers, so this
+    is the only place where their length can be checked); ``trailing_dim``, when the launch has a compressed buffer,
+    the number of slots of its rows, which every segment's offset must lie inside."""
     if not 1 <= len(segments) <= MAX_SEGMENTS:
         raise SplatError(f"between 1 and {MAX_SEGMENTS} ACSR segments are supported (got {len(segments)})")
     arr = (AcsrSeg * len(segments))()
@@ -131,6 +135,15 @@ def seg_array(segments: Sequence[tuple]) -> Any:
             require_device_tensor(t, name)
             if t.dtype != torch.float32 or not t.is_contiguous():
                 raise SplatError(f"{name} must be a contiguous float32 tensor")
+            if t.numel() < rows:
+                raise SplatError(f"{name} of segment {i} has {t.numel()} entries, the launch has {rows} rows: the ACSR "
+                                 "was built for another mask")
+        if fc is not None:
+            require_device_tensor(fc, "first_col")
+            if fc.dtype != torch.int32 or not fc.is_contiguous() or fc.numel() < rows:
+                raise SplatError(f"first_col of segment {i} must be a contiguous int32 tensor with at least {rows} entries")
+        if trailing_dim is not None and not 0 <= int(off) < max(int(trailing_dim), 1):
+            raise SplatError(f"segment {i} starts at slot {off}, outside the compressed rows' {trailing_dim} slots")
         arr[i].dTos_lin, arr[i].dTos_trans = a.data_ptr(), b.data_ptr()
         arr[i].sTod_lin, arr[i].sTod_trans, arr[i].nnz = c.data_ptr(), d.data_ptr(), n.data_ptr()
         arr[i].first_col = fc.data_ptr() if fc is not None else None

@@ -17,6 +17,9 @@ from dataclasses import dataclass
 from math import ceil
 from typing import Any, Sequence, Type
 
+import hashlib
+import weakref
+
 import numpy as np
 import torch
 
@@ -154,50 +157,71 @@ class ACSR:
 
 
 class _MaskEntry:
-    __slots__ = ("key_obj", "mask", "builds")
+    __slots__ = ("key", "owner", "builds")
 
-    def __init__(self, key_obj, mask):
-        self.key_obj = key_obj  # keeps the caller's object alive so that its id() stays unique
-        self.mask = mask
+    def __init__(self, key, owner):
+        self.key = key
+        self.owner = owner  # weak reference to a tensor mask: while it lives, its storage address cannot be reused
         self.builds = {}
+
+    def alive(self) -> bool:
+        return self.owner is None or self.owner() is not None
 
 
 _MASK_CACHE: list[_MaskEntry] = []
 _MASK_CACHE_SIZE = 4
 
 
-def _cache_key(mask) -> tuple:
+def _host_mask_bytes(mask) -> np.ndarray:
+    arr = np.asarray(mask)
+    if arr.ndim != 2:
+        raise ValueError("mask must be a 2-D 0/1 array")
+    if arr.size and (arr.min() < 0 or arr.max() > 255):
+        raise ValueError("mask entries must fit in a byte")
+    return np.ascontiguousarray(arr, dtype=np.uint8)
+
+
+def _cache_key(mask, host_bytes: np.ndarray | None = None) -> tuple:
+    """What identifies a mask's contents.  Tensors: storage address, version counter (bumped by every in-place
+    edit), shape, strides, storage offset and dtype -- a transposed or offset view of the same storage is another
+    mask.  Patterns: the (frozen) descriptor.  Lists and arrays are mutable without a trace, so they are keyed on a
+    digest of their bytes, taken from the uint8 copy that the upload needs anyway."""
     if isinstance(mask, torch.Tensor):
-        return ("t", mask.data_ptr(), mask._version, tuple(mask.shape), str(mask.device))
+        return ("t", mask.data_ptr(), mask._version, tuple(mask.shape), tuple(mask.stride()), mask.storage_offset(),
+                str(mask.dtype), str(mask.device))
     if isinstance(mask, MaskPattern):
         return ("p", mask)
-    return ("o", id(mask))
+    b = _host_mask_bytes(mask) if host_bytes is None else host_bytes
+    return ("h", b.shape, hashlib.blake2b(b.data, digest_size=16).digest())
 
 
-def _mask_entry(mask, dev: torch.device) -> _MaskEntry:
-    """The uint8 [rows, cols] device copy of ``mask`` (shared by create_acsr and the three preambles,
-    which the reference hands the same mask object)."""
-    key = (_cache_key(mask), str(dev))
+def _mask_entry(mask, dev: torch.device) -> tuple[_MaskEntry, np.ndarray | None]:
+    """The cache entry of ``mask`` on ``dev`` (create_acsr and the three preambles are handed the same mask, as in the
+    reference, and share one build) and, for host masks, their uint8 bytes.  Only the small per-row results are kept:
+    no rows x cols copy of the mask outlives a build."""
+    host = None if isinstance(mask, (torch.Tensor, MaskPattern)) else _host_mask_bytes(mask)
+    key = (_cache_key(mask, host), str(dev))
+    _MASK_CACHE[:] = [e for e in _MASK_CACHE if e.alive()]
     for e in _MASK_CACHE:
-        if e.key_obj[0] == key:
-            return e
-    if isinstance(mask, MaskPattern):
-        dm = None  # never rasterised for the builder: its rows are known in closed form
-    elif isinstance(mask, torch.Tensor):
-        dm = mask.to(device=dev, dtype=torch.uint8).contiguous()
-    else:
-        arr = np.asarray(mask)
-        if arr.ndim != 2:
-            raise ValueError("mask must be a 2-D 0/1 array")
-        if arr.size and (arr.min() < 0 or arr.max() > 255):
-            raise ValueError("mask entries must fit in a byte")
-        dm = torch.from_numpy(np.ascontiguousarray(arr, dtype=np.uint8)).to(dev)
-    if dm is not None and dm.dim() != 2:
+        if e.key == key:
+            return e, host
+    if isinstance(mask, torch.Tensor) and mask.dim() != 2:
         raise ValueError("mask must be 2-D")
-    entry = _MaskEntry((key, mask), dm)
+    entry = _MaskEntry(key, weakref.ref(mask) if isinstance(mask, torch.Tensor) else None)
     _MASK_CACHE.append(entry)
     del _MASK_CACHE[:-_MASK_CACHE_SIZE]
-    return entry
+    return entry, host
+
+
+def _device_mask(mask, host: np.ndarray | None, dev: torch.device) -> torch.Tensor | None:
+    """uint8 [rows, cols] on ``dev`` with unit column stride; None for a MaskPattern (never rasterised for the builder:
+    its rows are known in closed form)."""
+    if isinstance(mask, MaskPattern):
+        return None
+    if isinstance(mask, torch.Tensor):
+        dm = mask.to(device=dev, dtype=torch.uint8)
+        return dm if dm.stride(1) == 1 else dm.contiguous()
+    return torch.from_numpy(host).to(dev)
 
 
 def mask_shape(mask) -> tuple[int, int]:
@@ -215,10 +239,10 @@ class AcsrBuild:
 
 
 def build_acsr(mask, BLOCK_HEIGHT: int, dev: torch.device) -> AcsrBuild:
-    entry = _mask_entry(mask, dev)
+    entry, host = _mask_entry(mask, dev)
     if BLOCK_HEIGHT in entry.builds:
         return entry.builds[BLOCK_HEIGHT]
-    dm = entry.mask
+    dm = _device_mask(mask, host, dev)
     rows, cols = mask_shape(mask) if dm is None else dm.shape
     n_blocks = ceil(rows / BLOCK_HEIGHT)
     f32 = dict(dtype=torch.float32, device=dev)
@@ -241,11 +265,11 @@ def build_acsr(mask, BLOCK_HEIGHT: int, dev: torch.device) -> AcsrBuild:
             rc = _hip.lib().splat_acsr_build(dm.data_ptr(), rows, cols, dm.stride(0), BLOCK_HEIGHT, *outs,
                                              _hip.stream_ptr(dev))
             _hip.check(rc, "splat_acsr_build")
-    host = summary.cpu()  # the one synchronisation: T is returned as a Python int, like the reference
-    assert int(host[1]) == 0, "Incorrect unpacking of affine-indices."
-    b.T = int(host[0])
+    found = summary.cpu()  # the one synchronisation: T is returned as a Python int, like the reference
+    assert int(found[1]) == 0, "Incorrect unpacking of affine-indices."
+    b.T = int(found[0])
     # rows whose columns step by n and start in phase with the row index (dilated windows): kernels group them by phase
-    b.row_stride = int(host[2]) if (int(host[2]) == int(host[3]) and int(host[3]) > 1 and int(host[4]) == 0) else 1
+    b.row_stride = int(found[2]) if (int(found[2]) == int(found[3]) and int(found[3]) > 1 and int(found[4]) == 0) else 1
     entry.builds[BLOCK_HEIGHT] = b
     return b
 
@@ -271,9 +295,12 @@ def create_acsr(mask, BLOCK_HEIGHT: int, GPU_ID: Any):
     hint for patterns whose rows alternate column phase."""
     dev = _hip.resolve_device(GPU_ID)
     b = build_acsr(mask, BLOCK_HEIGHT, dev)
-    b.sTod_trans.splat_first_col = b.row_first
-    b.sTod_trans.splat_row_stride = b.row_stride
-    return (b.dTos_lin, b.dTos_trans, b.sTod_lin, b.sTod_trans, b.nnz, b.T, b.span_start, b.span_end)
+    # every caller gets tensors of its own, as from the reference's create_acsr: a build shared through the cache must
+    # not change under one caller because another one wrote into its metadata
+    arrays = [t.clone() for t in (b.dTos_lin, b.dTos_trans, b.sTod_lin, b.sTod_trans, b.nnz, b.span_start, b.span_end)]
+    arrays[3].splat_first_col = b.row_first.clone()
+    arrays[3].splat_row_stride = b.row_stride
+    return (arrays[0], arrays[1], arrays[2], arrays[3], arrays[4], b.T, arrays[5], arrays[6])
 
 
 class ACSRSegments:

@@ -33,7 +33,7 @@ def attention_plan(segments: ACSRSegments, L: int, device) -> torch.Tensor:
     """The fused kernel's plan for these segments and ``L`` rows (which key tiles each 128-row block walks, every
     row's window): an opaque uint8 device tensor, built once per mask and handed to ``attention_launcher``."""
     dev = _hip.resolve_device(device)
-    arr = _hip.seg_array(segments.seg_args())
+    arr = _hip.seg_array(segments.seg_args(), L)
     nbytes = int(_hip.lib().splat_attention_plan_bytes(arr, len(segments), L))
     if nbytes <= 0:
         raise _hip.SplatError(f"no plan for {len(segments)} segments and L={L}")
@@ -63,17 +63,31 @@ def attention_launcher(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor, outpu
     if tuple(kT.shape) != (B, H, d, L) or tuple(v.shape) != (B, H, L, d) or tuple(output.shape) != (B, H, L, d):
         raise _hip.SplatError(f"expected kT {(B, H, d, L)}, v and output {(B, H, L, d)}; got {tuple(kT.shape)}, "
                               f"{tuple(v.shape)}, {tuple(output.shape)}")
-    if q.stride(3) != 1:
-        q = q.contiguous()
-    if v.stride(3) != 1:
-        v = v.contiguous()
-    if kT.stride(2) != 1 and kT.stride(3) != 1:
-        kT = kT.contiguous()
     if output.stride(3) != 1:
         raise _hip.SplatError("output needs unit stride along d")
+    # The kernel moves 16-byte pieces: base addresses and batch / head / row strides must be multiples of 16 bytes.
+    # Views that are not (odd storage offsets, row strides that are not a multiple of 8 or 4 elements) are copied.
+    epc = 16 // q.element_size()
+
+    def piecewise(t, strides):
+        return t.data_ptr() % 16 == 0 and all(t.stride(i) % epc == 0 for i in strides)
+    if q.stride(3) != 1 or not piecewise(q, (0, 1, 2)):
+        q = q.contiguous()
+    if v.stride(3) != 1 or not piecewise(v, (0, 1, 2)):
+        v = v.contiguous()
+    if kT.stride(2) == 1 and kT.stride(3) >= d and piecewise(kT, (0, 1, 3)):
+        pass  # rows of K contiguous: [.., L, d] memory seen as [.., d, L]
+    elif kT.stride(3) == 1 and L % epc == 0 and piecewise(kT, (0, 1, 2)):
+        pass  # K^T contiguous along the keys, the reference's layout, in whole 16-byte pieces
+    else:
+        # e.g. the reference's contiguous [B, H, d, L] with L not a multiple of the piece: rows of K made contiguous
+        kT = kT.transpose(2, 3).contiguous().transpose(2, 3)
+    target = output
+    if not piecewise(output, (0, 1, 2)):
+        output = torch.empty((B, H, L, d), dtype=target.dtype, device=target.device)
     qs, ks, vs, os_ = q.stride(), kT.stride(), v.stride(), output.stride()
     dev = q.device
-    arr = _hip.seg_array(segments.seg_args())
+    arr = _hip.seg_array(segments.seg_args(), L)
     args = (q.data_ptr(), qs[0], qs[1], qs[2], kT.data_ptr(), ks[0], ks[1], ks[2], ks[3],
             v.data_ptr(), vs[0], vs[1], vs[2], output.data_ptr(), os_[0], os_[1], os_[2],
             arr, len(segments), B, H, L, d, float(scale), _hip.dtype_code(q.dtype))
@@ -98,7 +112,9 @@ def attention_launcher(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor, outpu
             rc = _hip.lib().splat_attention_fwd_planned(*args, plan.data_ptr(), plan.numel() * plan.element_size(),
                                                         _hip.stream_ptr(dev))
             _hip.check(rc, "splat_attention_fwd_planned")
-    return output
+    if target is not output:
+        target.copy_(output)
+    return target
 
 
 class RegularAttention(nn.Module):
@@ -115,6 +131,10 @@ class RegularAttention(nn.Module):
         self.scale = 1.0 if scale is None else float(scale)
         self.fused = fused
 
+        for m in (mask if _is_segment_list(mask) else [mask]):
+            if tuple(mask_shape(m)) != (seq_length, seq_length):
+                raise _hip.SplatError(f"the mask is {tuple(mask_shape(m))}, the module attends over "
+                                      f"{(seq_length, seq_length)}: every kernel indexes the ACSR with the sequence's rows")
         if _is_segment_list(mask):
             self.segments = create_acsr_segments(mask, BLOCK_SIZE_Y, GPU_ID)
         else:

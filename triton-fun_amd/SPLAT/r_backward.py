@@ -59,7 +59,7 @@ def softmax_backward_launcher(p: torch.Tensor, dp: torch.Tensor, ds: torch.Tenso
     if T != segments.T:
         raise _hip.SplatError(f"trailing dimension {T} does not match the segments' {segments.T}")
     dev = p.device
-    arr = _hip.seg_array(segments.seg_args())
+    arr = _hip.seg_array(segments.seg_args(), L, T)
     with torch.cuda.device(dev):
         rc = _hip.lib().splat_softmax_bwd(p.data_ptr(), dp.data_ptr(), ds.data_ptr(), arr, len(segments), B * H, L, T,
                                           float(scale), _hip.dtype_code(p.dtype), _hip.stream_ptr(dev))
@@ -82,7 +82,7 @@ def compressed_transpose_launcher(src: torch.Tensor, dst: torch.Tensor, segments
     if T != segments.T or Tt != segments_t.T:
         raise _hip.SplatError("trailing dimensions do not match the segments")
     dev = src.device
-    a, b = _hip.seg_array(segments.seg_args()), _hip.seg_array(segments_t.seg_args())
+    a, b = _hip.seg_array(segments.seg_args(), L, T), _hip.seg_array(segments_t.seg_args(), Lt, Tt)
     with torch.cuda.device(dev):
         rc = _hip.lib().splat_compressed_transpose(src.data_ptr(), dst.data_ptr(), a, b, len(segments), B * H, L, T, Lt, Tt,
                                                    _hip.dtype_code(src.dtype), _hip.stream_ptr(dev))
@@ -111,7 +111,7 @@ def rspmm_t_launcher(p: torch.Tensor, x: torch.Tensor, out: torch.Tensor, segmen
     if T != segments.T or len(segments) != len(segments_t):
         raise _hip.SplatError("the segments do not fit p (trailing dimension, number of segments)")
     dev = p.device
-    a, b = _hip.seg_array(segments.seg_args()), _hip.seg_array(segments_t.seg_args())
+    a, b = _hip.seg_array(segments.seg_args(), L, T), _hip.seg_array(segments_t.seg_args(), Lt)
     xs = x.stride()
     with torch.cuda.device(dev):
         rc = _hip.lib().splat_spmm_t(p.data_ptr(), x.data_ptr(), xs[0], xs[1], xs[2], out.data_ptr(), a, b, len(segments), B, H,

@@ -2,7 +2,9 @@
 
 Mirrors the reference's ``SPLAT/r_sddmm.py``: ``gen_block_mappings`` / ``naive_block_mappings`` (:117-151),
 ``rsddmm_preamble`` (:154-169) and ``rsddmm_launcher`` (:171-184) keep their names, positional parameters
-and return tuples.  The Triton kernel (:15-115) is replaced by ``splat_sddmm`` (MFMA, gfx950).
+and return tuples.  The Triton kernel (:15-115) is replaced by ``splat_sddmm`` (MFMA, gfx950).  The module's
+self-check (``truth`` :186-188, ``is_correct`` :191-221, ``test`` :224-256) keeps its names, signatures and
+acceptance rule; the four nested Python loops of the checker are tensor operations on the device here.
 """
 from __future__ import annotations
 
@@ -94,7 +96,7 @@ def rsddmm_launcher(x: torch.Tensor, y: torch.Tensor, output: torch.Tensor,
         raise _hip.SplatError(f"output must be a contiguous [B, H, L, T] = {(B, H, L, trailing_dim)} tensor")
     qs, ks = _strides4(x, "x"), _strides4(y, "y")
     dev = x.device
-    arr = _hip.seg_array(segs.seg_args())
+    arr = _hip.seg_array(segs.seg_args(), L, trailing_dim)
     args = (x.data_ptr(), qs[0], qs[1], qs[2], y.data_ptr(), ks[0], ks[1], ks[2], ks[3], output.data_ptr(), arr, len(segs),
             B, H, L, n_keys, d, trailing_dim, 1.0 if scale is None else float(scale), _hip.dtype_code(x.dtype),
             _hip.dtype_code(output.dtype))
@@ -110,3 +112,64 @@ def rsddmm_launcher(x: torch.Tensor, y: torch.Tensor, output: torch.Tensor,
             rc = _hip.lib().splat_sddmm_probs(*args, lse.data_ptr(), _hip.stream_ptr(dev))
             _hip.check(rc, "splat_sddmm_probs")
     return (output, sTod_linear_transformations, sTod_translations, nnzs)
+
+
+def live_slot_columns(sTod_linear_transformations: torch.Tensor, sTod_translations: torch.Tensor, nnzs: torch.Tensor,
+                      trailing_dim: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """(columns int64 [rows, T], live bool [rows, T]): the dense column behind every compressed slot by the builder's
+    rule c = sTod_lin * (s + sTod_trans) (acsr_helpers.py:122-124; for unit steps the same as the reference checkers'
+    round(s * lin + trans), r_sddmm.py:210), and which slots are live (s < nnz).  Rows with one live column store
+    translation 0 whatever the column is; their column is taken from the builder's ``splat_first_col``."""
+    lin = sTod_linear_transformations.double()
+    trans = sTod_translations.double()
+    slots = torch.arange(trailing_dim, device=lin.device, dtype=torch.float64)
+    cols = torch.round(lin[:, None] * (slots[None, :] + trans[:, None])).long()
+    live = slots[None, :] < nnzs.double()[:, None]
+    first = getattr(sTod_translations, "splat_first_col", None)
+    if first is not None:
+        single = nnzs == 1
+        cols[single, 0] = first.long()[single]
+    return cols, live
+
+
+def truth(x: torch.Tensor, y: torch.Tensor, GPU_ID: Any) -> torch.Tensor:
+    """The dense product the sampled one is checked against."""
+    return torch.einsum('bnqd, bndk -> bnqk', x, y)
+
+
+def is_correct(out_torch: torch.Tensor, out_rsddmm: torch.Tensor,
+               sTod_linear_transofrmations: torch.Tensor, sTod_translations: torch.Tensor, nnzs: torch.Tensor,
+               batch_size: int, num_heads: int, mask) -> bool:
+    """Every live slot of ``out_rsddmm`` [B, H, L, T] must lie within 1e-3 of the dense product's entry at the slot's
+    column.  Prints the reference's verdict lines and returns the verdict."""
+    rows = len(mask) if not isinstance(mask, torch.Tensor) else mask.shape[0]
+    T = out_rsddmm.shape[-1]
+    cols, live = live_slot_columns(sTod_linear_transofrmations[:rows], sTod_translations[:rows], nnzs[:rows], T)
+    cols = cols.clamp_(0, out_torch.shape[-1] - 1).to(out_torch.device)
+    want = out_torch[:batch_size, :num_heads, :rows].double().gather(3, cols.expand(batch_size, num_heads, rows, T))
+    diff = (want - out_rsddmm[:batch_size, :num_heads, :rows].double().to(want.device)).abs()
+    bad = (diff > 1e-3) & live.to(diff.device)
+    if bool(bad.any()):
+        print(f'test case failed average mse: {float(diff[bad].sum())}')
+        return False
+    print('test case passed!')
+    return True
+
+
+def test(m: int, k: int, n: int, num_heads: int, batch_size: int, mask, GPU_ID: Any, BLOCK_SIZE_Y: int,
+         BLOCK_SIZE_X: int, out_dtype: torch.dtype) -> bool:
+    """[m, k] x [k, n] per (batch, head) on integer-valued inputs, sampled onto ``mask``; returns ``is_correct``'s verdict
+    (the reference drops it)."""
+    assert m == n, "We only need to consider the case when m=n."
+    left = torch.randint(0, 100, (batch_size, num_heads, m, k), dtype=out_dtype).to(GPU_ID)
+    right = torch.randint(0, 100, (batch_size, num_heads, k, n), dtype=out_dtype).to(GPU_ID)
+    (dTos_linear_transformations, dTos_translations, sTod_linear_transformations, sTod_translations, nnzs,
+     acsr_trailing_dimension, _, _) = create_acsr(mask, BLOCK_SIZE_X, GPU_ID)
+    output_tensor, grid_dim, tb_map_x, tb_map_y = rsddmm_preamble(mask, (batch_size, num_heads, m, acsr_trailing_dimension),
+                                                                  BLOCK_SIZE_X, BLOCK_SIZE_Y, GPU_ID, out_dtype)
+    rsddmm_output, sTod_linear_transformations, sTod_translations, nnzs = rsddmm_launcher(
+        left, right, output_tensor, dTos_linear_transformations, dTos_translations, sTod_linear_transformations,
+        sTod_translations, acsr_trailing_dimension, nnzs, grid_dim, tb_map_x, tb_map_y, BLOCK_SIZE_Y, BLOCK_SIZE_X)
+    torch_output = truth(left, right, GPU_ID)
+    return is_correct(torch_output, rsddmm_output, sTod_linear_transformations, sTod_translations, nnzs, batch_size,
+                      num_heads, mask)

@@ -1,7 +1,8 @@
 """R-SpMM: compressed probabilities (ACSR, row-major, row-compressed) times dense V.
 
 Mirrors the reference's ``SPLAT/r_spmm.py``: ``rspmm_preamble`` (:128-145) and ``rspmm_launcher``
-(:148-164).  The Triton kernel (:13-126) is replaced by ``splat_spmm`` (MFMA, gfx950).
+(:148-164).  The Triton kernel (:13-126) is replaced by ``splat_spmm`` (MFMA, gfx950).  The module's self-check
+(``is_correct`` :166-216, ``test`` :219-261) keeps its names, signatures and acceptance rule.
 """
 from __future__ import annotations
 
@@ -11,6 +12,7 @@ import torch
 
 import _splat_hip as _hip
 from acsr_helpers import ACSRSegments, build_acsr, create_acsr, create_blocked_mask, create_windowed_mask  # noqa: F401
+from r_sddmm import live_slot_columns
 
 
 def rspmm_preamble(mask, output_shape: tuple[int], BLOCK_SIZE_X: int, BLOCK_SIZE_Y: int, GPU_ID: Any,
@@ -52,10 +54,57 @@ def rspmm_launcher(x: torch.Tensor, y: torch.Tensor, output: torch.Tensor,
                                            sTod_linear_transformations, sTod_translations, nnzs, acsr_trailing_dim)
     vs = y.stride()
     dev = x.device
-    arr = _hip.seg_array(segs.seg_args())
+    arr = _hip.seg_array(segs.seg_args(), L, T)
     with torch.cuda.device(dev):
         rc = _hip.lib().splat_spmm(x.data_ptr(), y.data_ptr(), vs[0], vs[1], vs[2], output.data_ptr(), arr, len(segs),
                                    B, H, L, n_keys, n_out, T, _hip.dtype_code(x.dtype), _hip.dtype_code(output.dtype),
                                    _hip.stream_ptr(dev))
     _hip.check(rc, "splat_spmm")
     return (output, sTod_linear_transformations, sTod_translations, nnzs)
+
+
+def is_correct(left_tensor: torch.Tensor, right_tensor: torch.Tensor, out_rspmm: torch.Tensor,
+               sTod_linear_transofrmations: torch.Tensor, sTod_translations: torch.Tensor, nnzs: torch.Tensor,
+               num_heads: int, batch_size: int, mask) -> bool:
+    """``out_rspmm`` [B, H, L, n] against sum over the live slots s of left[.., r, s] * right[.., column of s, :], within
+    1e-3 per entry.  The reference evaluates that sum with a Python loop per entry (its ``dot_product``) and only at the
+    output columns whose index is a live mask column of the row; here every entry is checked, in float64 on the
+    device.  Prints the reference's verdict lines and returns the verdict."""
+    rows = len(mask) if not isinstance(mask, torch.Tensor) else mask.shape[0]
+    dev = left_tensor.device
+    T = left_tensor.shape[-1]
+    n_keys = right_tensor.shape[2]
+    cols, live = live_slot_columns(sTod_linear_transofrmations[:rows], sTod_translations[:rows], nnzs[:rows], T)
+    cols, live = cols.clamp_(0, n_keys - 1).to(dev), live.to(dev)
+    total, n_bad = 0.0, 0
+    for b in range(batch_size):
+        for h in range(num_heads):
+            p = torch.where(live, left_tensor[b, h, :rows].double(), torch.zeros((), dtype=torch.float64, device=dev))
+            dense = torch.zeros(rows, n_keys, dtype=torch.float64, device=dev).scatter_add_(1, cols, p)
+            diff = (dense @ right_tensor[b, h].double() - out_rspmm[b, h, :rows].double().to(dev)).abs()
+            bad = diff > 1e-3
+            n_bad += int(bad.sum())
+            total += float(diff[bad].sum())
+    if n_bad > 0:
+        print(f'test case failed average mse: {total}')
+        return False
+    print('test case passed!')
+    return True
+
+
+def test(m: int, k: int, n: int, num_heads: int, batch_size: int, mask, GPU_ID: Any, BLOCK_SIZE_Y: int,
+         BLOCK_SIZE_X: int, output_dtype: torch.dtype) -> bool:
+    """Compressed [m, T] times dense [k, n] per (batch, head) on integer-valued float32 inputs; returns ``is_correct``'s
+    verdict (the reference drops it)."""
+    assert m == n, "We only need to consider the case when m=n."
+    (dTos_linear_transformations, dTos_translations, sTod_linear_transformations, sTod_translations, nnzs, _,
+     span_loop_start, span_loop_end) = create_acsr(mask, BLOCK_SIZE_X, GPU_ID)
+    output_tensor, grid_dim, trailing_dim_acsr = rspmm_preamble(mask, (batch_size, num_heads, m, n), BLOCK_SIZE_X,
+                                                                BLOCK_SIZE_Y, GPU_ID, output_dtype)
+    left = torch.randint(0, 100, (batch_size, num_heads, m, trailing_dim_acsr), dtype=torch.float32).to(GPU_ID)
+    right = torch.randint(0, 100, (batch_size, num_heads, k, n), dtype=torch.float32).to(GPU_ID)
+    rspmm_output, sTod_linear_transformations, sTod_translations, nnzs = rspmm_launcher(
+        left, right, output_tensor, dTos_linear_transformations, dTos_translations, sTod_linear_transformations,
+        sTod_translations, span_loop_start, span_loop_end, trailing_dim_acsr, nnzs, grid_dim, BLOCK_SIZE_Y, BLOCK_SIZE_X)
+    return is_correct(left, right, rspmm_output, sTod_linear_transformations, sTod_translations, nnzs, num_heads,
+                      batch_size, mask)

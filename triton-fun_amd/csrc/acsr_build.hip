@@ -406,6 +406,7 @@ extern "C" int splat_acsr_build(const uint8_t* mask, int64_t rows, int64_t cols,
                                 float* dTos_lin, float* dTos_trans, float* sTod_lin, float* sTod_trans, float* nnz,
                                 float* span_start, float* span_end, int32_t* row_first, int32_t* row_last,
                                 int32_t* summary, void* stream) {
+    begin_launch();
     if (!mask || !dTos_lin || !dTos_trans || !sTod_lin || !sTod_trans || !nnz || !span_start || !span_end || !summary)
         return fail(SPLAT_E_NULL, "splat_acsr_build: null pointer argument");
     if (rows <= 0 || cols <= 0 || ld < cols || block_height <= 0)
@@ -444,6 +445,7 @@ extern "C" int splat_acsr_build_pattern(int32_t pattern, int64_t s, int64_t p0, 
                                         float* dTos_lin, float* dTos_trans, float* sTod_lin, float* sTod_trans, float* nnz,
                                         float* span_start, float* span_end, int32_t* row_first, int32_t* row_last,
                                         int32_t* summary, void* stream) {
+    begin_launch();
     const char* who = "splat_acsr_build_pattern";
     if (!dTos_lin || !dTos_trans || !sTod_lin || !sTod_trans || !nnz || !span_start || !span_end || !summary)
         return fail(SPLAT_E_NULL, "%s: null pointer argument", who);
@@ -462,6 +464,7 @@ extern "C" int splat_acsr_build_pattern(int32_t pattern, int64_t s, int64_t p0, 
 
 extern "C" int splat_mask_generate(uint8_t* mask, int64_t rows, int64_t cols, int64_t ld, int32_t pattern, int64_t p0,
                                    int64_t p1, void* stream) {
+    begin_launch();
     if (!mask) return fail(SPLAT_E_NULL, "splat_mask_generate: null mask");
     if (rows <= 0 || cols <= 0 || ld < cols || rows > (1 << 23) || cols > (1 << 23))
         return fail(SPLAT_E_SHAPE, "splat_mask_generate: bad shape rows=%lld cols=%lld ld=%lld", (long long)rows, (long long)cols, (long long)ld);

@@ -14,7 +14,7 @@ struct SegPtrs {
     const float* nnz;
     const int32_t* first_col;
     int slot_offset;
-    int pad_;
+    int max_cnt;  // slots the segment may own in a compressed row (T - slot_offset); INT32_MAX where no buffer has rows of T slots
 };
 
 // Per-workgroup plan of one segment.
@@ -26,8 +26,12 @@ struct SegPlan {
                   // 0: positions are dense columns and a row applies the full affine test
 };
 
+// A row's count is clamped to the slots its segment owns, so that metadata that disagrees with the buffer's trailing
+// dimension cannot send a kernel past the end of a compressed row.
 __device__ __forceinline__ RowMap load_row_map(const SegPtrs& s, int r) {
-    return load_row_map(s.sTod_lin, s.sTod_trans, s.nnz, s.first_col, r);
+    RowMap m = load_row_map(s.sTod_lin, s.sTod_trans, s.nnz, s.first_col, r);
+    m.cnt = min(m.cnt, s.max_cnt);
+    return m;
 }
 
 // LDS the planner needs: per-wavefront partial reductions, and the rows' integer maps for later reuse.
@@ -343,7 +347,8 @@ inline int fill_segs(const char* who, const splat_acsr_seg* segs, int n_seg, Seg
             return fail(SPLAT_E_NULL, "%s: segment %d lacks sTod_lin / sTod_trans / nnz", who, k);
         if (T >= 0 && (segs[k].slot_offset < 0 || segs[k].slot_offset >= T))
             return fail(SPLAT_E_SHAPE, "%s: segment %d slot_offset %d outside [0, T=%d)", who, k, segs[k].slot_offset, T);
-        out[k] = SegPtrs{segs[k].sTod_lin, segs[k].sTod_trans, segs[k].nnz, segs[k].first_col, segs[k].slot_offset, 0};
+        out[k] = SegPtrs{segs[k].sTod_lin, segs[k].sTod_trans, segs[k].nnz, segs[k].first_col, segs[k].slot_offset,
+                         T >= 0 ? T - segs[k].slot_offset : 0x7fffffff};
     }
     return 0;
 }

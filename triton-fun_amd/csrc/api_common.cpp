@@ -24,11 +24,33 @@ int fail(int code, const char* fmt, ...) {
     return code;
 }
 
+// An error left behind by another user of the runtime on this thread (it is sticky until someone reads it) must not
+// be reported as this library's: read it away before launching.
+void begin_launch() { (void)hipGetLastError(); }
+
 int check_launch(const char* what) {
     hipError_t e = hipGetLastError();
     if (e == hipSuccess) return 0;
     set_error("%s: launch failed: %s", what, hipGetErrorString(e));
     return (int)e;
+}
+
+int reserve_dynamic_lds(uint64_t* done, const void* kernel, size_t bytes, const char* who) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        set_error("%s: hipGetDevice: %s", who, hipGetErrorString(e));
+        return (int)e;
+    }
+    const uint64_t bit = 1ull << (dev & 63);
+    if (__atomic_load_n(done, __ATOMIC_ACQUIRE) & bit) return 0;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) {
+        set_error("%s: cannot reserve %zu bytes of LDS: %s", who, bytes, hipGetErrorString(e));
+        return (int)e;
+    }
+    __atomic_fetch_or(done, bit, __ATOMIC_RELEASE);
+    return 0;
 }
 
 }  // namespace splat

@@ -619,6 +619,7 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
 
 template <typename T, int D, bool KT, int BN, int NSTAGE, bool PLANNED>
 static int launch_attn(const AttnParams& p0, hipStream_t st) {
+    begin_launch();
     using G = TileGeom<T, D, KT, BN>;
     AttnParams p = p0;
     constexpr int BM = 128;
@@ -628,15 +629,8 @@ static int launch_attn(const AttnParams& p0, hipStream_t st) {
     const int grid = ((p.total + 7) / 8) * 8;
     const size_t lds = NSTAGE * (size_t)G::STAGE;
     auto kern = attn_fwd_kernel<T, D, KT, BN, NSTAGE, PLANNED>;
-    static thread_local bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) {
-            set_error("splat_attention_fwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-            return (int)e;
-        }
-        attr_set = true;
-    }
+    static uint64_t lds_reserved = 0;  // per instantiation: devices whose copy of this kernel has the limit raised
+    if (int rc = reserve_dynamic_lds(&lds_reserved, reinterpret_cast<const void*>(kern), lds, "splat_attention_fwd")) return rc;
     kern<<<grid, 256, lds, st>>>(p);
     return check_launch("splat_attention_fwd");
 }
@@ -790,6 +784,7 @@ extern "C" int64_t splat_attention_plan_bytes(const splat_acsr_seg* segs, int32_
 
 extern "C" int splat_attention_plan(const splat_acsr_seg* segs, int32_t n_seg, int32_t L, void* plan, int64_t plan_bytes,
                                     void* stream) {
+    begin_launch();
     const char* who = "splat_attention_plan";
     if (!segs || !plan) return fail(SPLAT_E_NULL, "%s: null pointer argument", who);
     if (L <= 0 || L > (1 << 23)) return fail(SPLAT_E_SHAPE, "%s: need 0 < L <= 2^23 (got %d)", who, L);

@@ -137,6 +137,7 @@ __global__ __launch_bounds__(256) void compressed_transpose_kernel(const Transpo
         const int jc = j0 + lane;  // the column this lane stands for in the "in" phase
         RowMap mj = {0, 1, 0};
         if (jc < p.Lt) mj = load_row_map(sg.t_sTod_lin, sg.t_sTod_trans, sg.t_nnz, sg.t_first_col, jc);
+        mj.cnt = min(mj.cnt, p.Tt - sg.t_off);  // never past the end of a compressed row, whatever the metadata says
         const int lo = wave_min_i(mj.cnt > 0 ? mj.a : 0x7fffffff);
         const int hi = wave_max_i(mj.cnt > 0 ? mj.a + mj.lin * (mj.cnt - 1) : -1);
         __syncthreads();  // the tile and the tables of the previous segment are done with
@@ -148,6 +149,7 @@ __global__ __launch_bounds__(256) void compressed_transpose_kernel(const Transpo
             if (wave == 0) {
                 RowMap mi = {0, 1, 0};
                 if (i0 + lane <= i_max) mi = load_row_map(sg.sTod_lin, sg.sTod_trans, sg.nnz, sg.first_col, i0 + lane);
+                mi.cnt = min(mi.cnt, p.T - sg.off);
                 mi_a[lane] = mi.a, mi_lin[lane] = mi.lin, mi_cnt[lane] = mi.cnt, mi_inv[lane] = 1.0f / (float)mi.lin;
             }
             __syncthreads();
@@ -185,6 +187,7 @@ using namespace splat;
 
 extern "C" int splat_softmax_bwd(const void* p, const void* dp, void* ds, const splat_acsr_seg* segs, int32_t n_seg, int64_t BH,
                                  int32_t L, int32_t T, float scale, int32_t dtype, void* stream) {
+    begin_launch();
     const char* who = "splat_softmax_bwd";
     if (!p || !dp || !ds || !segs) return fail(SPLAT_E_NULL, "%s: null pointer argument", who);
     if (n_seg < 1 || n_seg > SPLAT_MAX_SEGMENTS) return fail(SPLAT_E_SHAPE, "%s: n_seg must be 1..%d (got %d)", who, SPLAT_MAX_SEGMENTS, n_seg);
@@ -226,6 +229,7 @@ extern "C" int splat_softmax_bwd(const void* p, const void* dp, void* ds, const 
 extern "C" int splat_compressed_transpose(const void* src, void* dst, const splat_acsr_seg* segs, const splat_acsr_seg* segs_t,
                                           int32_t n_seg, int64_t BH, int32_t L, int32_t T, int32_t Lt, int32_t Tt, int32_t dtype,
                                           void* stream) {
+    begin_launch();
     const char* who = "splat_compressed_transpose";
     if (!src || !dst || !segs || !segs_t) return fail(SPLAT_E_NULL, "%s: null pointer argument", who);
     if (src == dst) return fail(SPLAT_E_UNSUPPORTED, "%s: not an in-place operation", who);

@@ -439,6 +439,7 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
 
 template <typename T>
 static int launch_sddmm(const char* who, SddmmParams p, bool kt, hipStream_t st) {
+    begin_launch();
     p.n_row_blocks = count_row_blocks(p.L, 128, p.row_stride);
     // Few row blocks (one head of a short sequence, the reference's own benchmark shape) would leave most of the 256
     // compute units idle: share every row block's tiles out over several workgroups then.

@@ -173,6 +173,7 @@ __global__ __launch_bounds__(256) void softmax_rows_any(const Tin* __restrict__ 
 
 template <typename Tin, typename Tout>
 static int launch_softmax(const void* x, void* y, const SoftmaxSegs& segs, int64_t n_rows, int L, int T, hipStream_t st) {
+    begin_launch();
     unsigned grid = (unsigned)((n_rows + 3) / 4);
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 31) == 0;
     const Tin* xi = (const Tin*)x;

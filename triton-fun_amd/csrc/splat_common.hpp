@@ -24,7 +24,12 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 // ---- host side error plumbing (defined in api_common.cpp) ---------------------------------
 void set_error(const char* fmt, ...);
 int fail(int code, const char* fmt, ...);
+void begin_launch();  // first statement of every function that launches and then calls check_launch
 int check_launch(const char* what);
+
+// Raise a kernel's dynamic LDS limit once per device (the attribute belongs to the device's copy of the kernel, so a
+// process that uses several GPUs needs it on each): `done` is a bit mask over device ordinals, one per kernel.
+int reserve_dynamic_lds(uint64_t* done, const void* kernel, size_t bytes, const char* who);
 
 constexpr int kWave = 64;
 

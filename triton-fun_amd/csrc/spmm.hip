@@ -320,6 +320,7 @@ __global__ __launch_bounds__(256, 2) void spmm_kernel(const SpmmParams p) {
 
 template <typename T>
 static int launch_spmm(SpmmParams p, hipStream_t st) {
+    begin_launch();
     p.n_row_blocks = count_row_blocks(p.L, 128, p.row_stride);
     const int dvt = p.n_out > 64 ? 4 : (p.n_out > 32 ? 2 : 1);
     p.n_col_chunks = (p.n_out + 32 * dvt - 1) / (32 * dvt);
@@ -580,6 +581,7 @@ __global__ __launch_bounds__(256, 2) void spmm_t_kernel(const SpmmTParams p) {
 
 template <typename T>
 static int launch_spmm_t(SpmmTParams p, hipStream_t st) {
+    begin_launch();
     p.n_row_blocks = count_row_blocks(p.Lt, 128, p.row_stride);
     const int dvt = p.n_out > 64 ? 4 : (p.n_out > 32 ? 2 : 1);
     p.n_col_chunks = (p.n_out + 32 * dvt - 1) / (32 * dvt);
