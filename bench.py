@@ -23,14 +23,49 @@ for _p in (ROOT, os.path.join(ROOT, "triton-fun_amd", "SPLAT")):
         sys.path.insert(0, _p)
 
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16
+FP32_MFMA_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes one fused launch moves at config 5, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
-# copy kernel of known size (profiles/attn_fwd_kernel_cfg5_hbm_traffic.md).
-FUSED_TRAFFIC_BYTES = 1.395e9
+# HBM bytes one fused launch moves at config 5 are not something this script can measure (hardware counters need
+# rocprofv3): the figure comes from the committed counter summary, which names the commit whose kernel it profiled.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "attn_fwd_kernel_cfg5_hbm_traffic.md")
+# The GPU's clock takes some tens of launches to settle under this kernel (the first launches of a process run at the
+# idle boost clock, the next ones slower, then the steady state): an untimed, declared phase ahead of --warmup.
+SETTLE_MIN_LAUNCHES = 100
+SETTLE_MIN_MS = 50.0
+
+
+def profiled_traffic():
+    """(bytes per launch, commit) from the lines `traffic_bytes_per_launch: X` / `kernel_commit: Y` of the committed
+    counter summary; (None, None) when it is missing or holds no such line."""
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return None, None
+    import re
+    b = re.search(r"traffic_bytes_per_launch:\s*([0-9.eE+]+)", text)
+    c = re.search(r"kernel_commit:\s*([0-9a-f]+)", text)
+    return (float(b.group(1)) if b else None), (c.group(1) if c else None)
+
+
+FUSED_KERNEL_NAME = "attn_fwd_kernel<bf16, D=128, KT=false, BN=64, NSTAGE=2, PLANNED=true>"
 
 
 def causal_window_nnz(L: int, w: int) -> int:
     return w * L - w * (w - 1) // 2
+
+
+def settle(fn):
+    """Untimed launches until the clock has settled: at least SETTLE_MIN_LAUNCHES and at least SETTLE_MIN_MS of
+    device time.  Returns the number of launches."""
+    import torch
+    n = 0
+    t0 = time.perf_counter()
+    while n < SETTLE_MIN_LAUNCHES or (time.perf_counter() - t0) * 1e3 < SETTLE_MIN_MS:
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+        n += 20
+    return n
 
 
 def time_launches(fn, steps: int, warmup: int):
@@ -79,6 +114,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50,
                     help="untimed launches before the timed ones (the GPU clock needs some tens of launches to settle)")
+    ap.add_argument("--no-settle", action="store_true",
+                    help="profiling runs: skip the clock-settle phase and the unsettled pass, so that a counter run sees "
+                         "only --warmup + --steps launches of the headline kernel")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host baseline")
     ap.add_argument("--no-extras", action="store_true", help="skip the unfused kernels and the ACSR build")
     ap.add_argument("--cpu-heads", type=int, default=16, help="(batch, head) pairs the host baseline computes")
@@ -122,12 +160,16 @@ def main() -> int:
     io_bytes = 4.0 * B * H * L * d * 2
 
     step = lambda: attn([qd, kT_view, vd])
+    # what the same --warmup / --steps give in a process that has just started (the clock has not settled)
+    cold_wall_ms, cold_per = (0.0, [0.0]) if args.no_settle else time_launches(step, args.steps, args.warmup)
+    settle_launches = 0 if args.no_settle else settle(step)
     wall_ms, per = time_launches(step, args.steps, args.warmup)
     ms_per_step = wall_ms / args.steps
     kern_ms = sum(per) / len(per)
     tflops = flops / (ms_per_step * 1e-3) / 1e12
     kern_tflops = flops / (kern_ms * 1e-3) / 1e12
 
+    traffic, traffic_commit = profiled_traffic()
     out = {
         "metric": "sparse-attn fwd ms + nnz-TFLOP/s (% MFMA peak) on 1 MI355X; softmax HBM GB/s",
         "value": round(tflops, 2),
@@ -135,7 +177,11 @@ def main() -> int:
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_launches": settle_launches,
         "ms_per_step": round(ms_per_step, 4),
+        "unsettled": {"ms_per_step": round(cold_wall_ms / args.steps, 4),
+                      "kernel_ms_avg": round(sum(cold_per) / len(cold_per), 4),
+                      "note": "the same warmup + steps run first, in the just-started process, before the settle phase"},
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -145,8 +191,9 @@ def main() -> int:
                                "scale 1/sqrt(d), K passed as k.transpose(2,3)",
                    "B": B, "H": H, "L": L, "d": d, "window": w, "nnz_per_head": nnz},
         "roofline": {"bound": "mfma", "achieved": round(kern_tflops, 2), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(kern_tflops / MFMA_PEAK_TFLOPS, 4), "traffic": FUSED_TRAFFIC_BYTES,
-                     "kernel": "attn_fwd_kernel<bf16, D=128, KT=false, BN=64, NSTAGE=2, PLANNED=true>", "kernel_ms_avg": round(kern_ms, 4),
+                     "frac": round(kern_tflops / MFMA_PEAK_TFLOPS, 4), "traffic": traffic,
+                     "traffic_source": {"profile": os.path.relpath(TRAFFIC_PROFILE, ROOT), "kernel_commit": traffic_commit},
+                     "kernel": FUSED_KERNEL_NAME, "kernel_ms_avg": round(kern_ms, 4),
                      "kernel_ms_min": round(per[0], 4), "algorithmic_flops": flops, "algorithmic_bytes": io_bytes,
                      "hbm_frac_at_algorithmic_bytes": round(io_bytes / (kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
         "fwd_ms": round(kern_ms, 4),
@@ -162,6 +209,29 @@ def main() -> int:
         torch.cuda.synchronize()
         del src, dst
     if not args.no_extras:
+        # the fused forward at the other four benchmark configurations
+        for name, (Bc, Hc, Lc, dc, dt, pat, mul) in {
+                "fused_cfg1": (1, 1, 512, 64, torch.float32, A.causal_windowed_pattern(512, 63), 1.0),
+                "fused_cfg2": (4, 16, 4096, 64, torch.float16, A.causal_windowed_pattern(4096, 255), 0.5),
+                "fused_cfg3": (2, 16, 8192, 64, torch.bfloat16, A.strided_patterns(8192, 128, 128), 1.0),
+                "fused_cfg4": (2, 32, 8192, 128, torch.bfloat16, A.dilated_pattern(8192, 512, 2), 1.0)}.items():
+            qc, kc, vc = (t.mul(mul).to(dt).to(dev) for t in make_inputs(1000 + int(name[-1]), Bc, Hc, Lc, dc, torch.float32))
+            at = RegularAttention(Bc, Lc, Hc, dc, pat, 16, 16, dev, dt, scale=dc ** -0.5)
+            nnz_c = sum(float(t[4].sum().item()) for t in at.segments.tuples)
+            fl = 4.0 * dc * nnz_c * Bc * Hc
+            byt = 4.0 * Bc * Hc * Lc * dc * qc.element_size()
+            kTc = kc.transpose(2, 3)
+            run = lambda: at([qc, kTc, vc])
+            for _ in range(60):
+                run()
+            _, pr = time_launches(run, 40, 10)
+            ms = sum(pr) / len(pr)
+            peak = FP32_MFMA_PEAK_TFLOPS if dt == torch.float32 else MFMA_PEAK_TFLOPS
+            extras[name] = {"ms": round(ms, 4), "ms_min": round(pr[0], 4), "tflops_nnz": round(fl / ms / 1e9, 2),
+                            "pct_mfma_peak": round(100 * fl / ms / 1e9 / peak, 2),
+                            "hbm_floor_ms": round(byt / HBM_PEAK_GBPS / 1e6, 4),
+                            "pct_of_hbm_floor_rate": round(100 * byt / HBM_PEAK_GBPS / 1e6 / ms, 2)}
+            del at, qc, kc, vc, kTc
         # the literal reference layout: K^T contiguous [B, H, d, L]
         kT_c = kT_view.contiguous()
         _, per_c = time_launches(lambda: attn([qd, kT_c, vd]), max(5, args.steps // 2), max(3, args.warmup // 2))

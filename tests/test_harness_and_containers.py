@@ -189,7 +189,7 @@ def test_a_trailing_dimension_smaller_than_the_rows_counts_stays_inside_the_buff
     assert acsr[5] == 16
     q, k, v = (t.to(dev) for t in O.make_inputs(3, 1, 1, L, d, torch.float16))
     SENT = 768.0
-    buf = torch.full((L + 4) * T_small, SENT, dtype=torch.float16, device=dev)
+    buf = torch.full(((L + 4) * T_small,), SENT, dtype=torch.float16, device=dev)
     s_buf = buf[:L * T_small].view(1, 1, L, T_small)
     r_sddmm.rsddmm_launcher(q, k.transpose(2, 3), s_buf, acsr[0], acsr[1], acsr[2], acsr[3], T_small, acsr[4], (1, 1), None,
                             None, 16, 16, scale=0.125)
@@ -200,8 +200,10 @@ def test_a_trailing_dimension_smaller_than_the_rows_counts_stays_inside_the_buff
     assert torch.all(buf[L * T_small:] == SENT)
     assert torch.isfinite(out.float()).all()
     # each row attended over its first T_small live columns
-    sums = s_buf.float().sum(-1)
+    live = torch.arange(T_small, device=dev)[None, :] < acsr[4].clamp(max=T_small)[:, None]
+    sums = torch.where(live, s_buf[0, 0].float(), torch.zeros((), device=dev)).sum(-1)
     assert torch.allclose(sums, torch.ones_like(sums), atol=1e-2)
+    assert torch.all(s_buf[0, 0][~live] == SENT)
 
 
 @pytest.mark.gpu
