@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define SPLAT_VERSION 400 /* major*10000 + minor*100 + patch; 0.2.0 added the planned forward, 0.3.0 splat_spmm_t, 0.4.0 splat_attention_fwd_stats, splat_sddmm_probs */
+#define SPLAT_VERSION 500 /* major*10000 + minor*100 + patch; 0.2.0 added the planned forward, 0.3.0 splat_spmm_t, 0.4.0 splat_attention_fwd_stats, splat_sddmm_probs, 0.5.0 splat_attention_fwd_noalloc */
 
 /* element types of q/k/v/score/output buffers */
 #define SPLAT_F32 0
@@ -207,6 +207,22 @@ int splat_attention_fwd_stats(const void* q, int64_t q_sb, int64_t q_sh, int64_t
                               int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t d, float scale,
                               int32_t dtype, const void* plan, int64_t plan_bytes, float* lse,
                               void* stream);
+
+/* The fused forward for callers that cannot allocate device memory or hold a plan buffer: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments and
+ * bit-identical results as splat_attention_fwd_planned, without the plan arguments: the plan is rebuilt by every call
+ * into a buffer of SPLAT_STATIC_PLAN_BYTES that is part of the library's device image (each GPU the library runs on
+ * holds one until the process ends), then the forward runs from it on the same stream.  The call allocates and frees
+ * nothing.  Masks whose plan is larger (splat_attention_plan_bytes; 4256 bytes per 128-row block and segment) are
+ * rejected with SPLAT_E_SHAPE.  All calls on one GPU share that one buffer: two calls whose work may overlap on a
+ * GPU (different streams, different threads) race; order them. */
+#define SPLAT_STATIC_PLAN_BYTES (4 << 20)
+int splat_attention_fwd_noalloc(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT,
+                                int64_t k_sb, int64_t k_sh, int64_t k_sd, int64_t k_sl, const void* v,
+                                int64_t v_sb, int64_t v_sh, int64_t v_sl, void* out, int64_t o_sb,
+                                int64_t o_sh, int64_t o_sl, const splat_acsr_seg* segs /* host */,
+                                int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t d, float scale,
+                                int32_t dtype, void* stream);
 
 /* ---- backward pass (the reference has none: r_attention.py:77-100 is forward only) ----
  * With S~ the compressed scores, P~ = softmax(S~), O = P~ . V:

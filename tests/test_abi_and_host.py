@@ -56,6 +56,26 @@ def test_null_and_shape_arguments_are_rejected_without_a_device():
     assert lib.splat_spmm(8, 8, 0, 0, 8, 8, seg, 1, 1, 1, 4, 4, 8, 4, 7, 0, None) == -3                    # bad dtype
 
 
+def test_the_allocation_free_forward_rejects_what_its_built_in_buffer_cannot_hold():
+    lib = hip.lib()
+    seg = (hip.AcsrSeg * 2)()
+    for i in range(2):
+        seg[i].sTod_lin = seg[i].sTod_trans = seg[i].nnz = 8
+        seg[i].row_stride_hint = 1
+    fwd = lambda n_seg, L: lib.splat_attention_fwd_noalloc(8, 0, 0, 64, 8, 0, 0, 1, 64, 8, 0, 0, 64, 8, 0, 0, 64, seg, n_seg, 1, 1, L,
+                                                           64, 1.0, 2, None)
+    L_big = 1 << 18
+    assert lib.splat_attention_plan_bytes(seg, 1, L_big) > hip.STATIC_PLAN_BYTES
+    assert fwd(1, L_big) == -2
+    msg = lib.splat_last_error()
+    assert b"splat_attention_fwd_noalloc" in msg and b"built-in buffer" in msg and str(hip.STATIC_PLAN_BYTES).encode() in msg
+    assert fwd(0, 128) == -2 and fwd(1, 0) == -2
+    assert lib.splat_attention_fwd_noalloc(8, 0, 0, 64, 8, 0, 0, 1, 64, 8, 0, 0, 64, 8, 0, 0, 64, None, 1, 1, 1, 128, 64, 1.0, 2,
+                                           None) == -1
+    header = open(HEADER).read()
+    assert int(eval(re.search(r"#define SPLAT_STATIC_PLAN_BYTES \((.*?)\)", header).group(1))) == hip.STATIC_PLAN_BYTES
+
+
 def test_plan_size_is_host_arithmetic():
     lib = hip.lib()
     seg = (hip.AcsrSeg * 2)()

@@ -19,6 +19,7 @@ SPLAT_F32, SPLAT_F16, SPLAT_BF16 = 0, 1, 2
 MAX_SEGMENTS = 4
 MASK_BLOCKED, MASK_WINDOWED, MASK_CAUSAL_WINDOWED, MASK_DILATED, MASK_STRIDED_LOCAL, MASK_STRIDED_FAR = range(6)
 MASK_TRANSPOSED = 8  # flag or-ed onto a pattern: its transpose
+STATIC_PLAN_BYTES = 4 << 20  # SPLAT_STATIC_PLAN_BYTES: the plan buffer built into the library for splat_attention_fwd_noalloc
 
 _DTYPES = {torch.float32: SPLAT_F32, torch.float16: SPLAT_F16, torch.bfloat16: SPLAT_BF16}
 
@@ -52,6 +53,9 @@ _SIGNATURES = {
     "splat_attention_fwd": (ctypes.c_int, [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _vp,
                                            _i64, _i64, _i64, ctypes.POINTER(AcsrSeg), _i32, _i32, _i32, _i32, _i32, _f32,
                                            _i32, _vp]),
+    "splat_attention_fwd_noalloc": (ctypes.c_int, [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _vp,
+                                                   _i64, _i64, _i64, ctypes.POINTER(AcsrSeg), _i32, _i32, _i32, _i32, _i32,
+                                                   _f32, _i32, _vp]),
     "splat_softmax_bwd": (ctypes.c_int, [_vp, _vp, _vp, ctypes.POINTER(AcsrSeg), _i32, _i64, _i32, _i32, _f32, _i32, _vp]),
     "splat_spmm_t": (ctypes.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, ctypes.POINTER(AcsrSeg), ctypes.POINTER(AcsrSeg), _i32, _i32,
                                    _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),

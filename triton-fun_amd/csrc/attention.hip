@@ -20,6 +20,8 @@
 // gathered rows of K/V) and validity is a per-row range test in j; otherwise tiles are dense columns
 // and validity is the full affine test (offset, step divisibility, count).  Each wavefront skips
 // tiles that lie outside all of its rows' spans and drops the mask on tiles inside all of them.
+#include <mutex>
+
 #include "tile_copy.hpp"
 
 namespace splat {
@@ -776,6 +778,31 @@ extern "C" int splat_attention_fwd_stats(const void* q, int64_t q_sb, int64_t q_
                                 o_sl, segs, n_seg, B, H, L, d, scale, dtype, plan, plan_bytes, plan != nullptr, lse, stream);
 }
 
+// ---- the forward for callers that cannot allocate: the plan lives in a file-scope device array ----------------
+constexpr int64_t kStaticPlanBytes = SPLAT_STATIC_PLAN_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticPlanBytes];
+// Host code must not use the array's name as an address: each device holds its own copy, whose address the runtime
+// hands out.  Resolved once per device, with that device current.
+static std::mutex g_scratch_lock;
+static void* g_scratch_ptr[64] = {};
+static int static_plan_buffer(const char* who, void** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail((int)e, "%s: hipGetDevice: %s", who, hipGetErrorString(e));
+    if (dev < 0 || dev >= 64) return fail(SPLAT_E_UNSUPPORTED, "%s: device ordinal %d is beyond the 64 this table holds", who, dev);
+    std::lock_guard<std::mutex> guard(g_scratch_lock);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr)
+            return fail(e != hipSuccess ? (int)e : SPLAT_E_NULL, "%s: cannot resolve the plan buffer on device %d: %s", who, dev,
+                        hipGetErrorString(e));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+
 extern "C" int64_t splat_attention_plan_bytes(const splat_acsr_seg* segs, int32_t n_seg, int32_t L) {
     if (!segs || n_seg < 1 || n_seg > SPLAT_MAX_SEGMENTS || L <= 0) return 0;
     const int n_rb = count_row_blocks(L, kPlanBM, common_row_stride(segs, n_seg));
@@ -801,4 +828,29 @@ extern "C" int splat_attention_plan(const splat_acsr_seg* segs, int32_t n_seg, i
     p.n_rb = count_row_blocks(L, kPlanBM, p.rs);
     attn_plan_kernel<<<dim3(p.n_rb, 2), 256, 0, (hipStream_t)stream>>>(p);
     return check_launch(who);
+}
+
+extern "C" int splat_attention_fwd_noalloc(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT,
+                                           int64_t k_sb, int64_t k_sh, int64_t k_sd, int64_t k_sl, const void* v,
+                                           int64_t v_sb, int64_t v_sh, int64_t v_sl, void* out, int64_t o_sb, int64_t o_sh,
+                                           int64_t o_sl, const splat_acsr_seg* segs, int32_t n_seg, int32_t B, int32_t H,
+                                           int32_t L, int32_t d, float scale, int32_t dtype, void* stream) {
+    const char* who = "splat_attention_fwd_noalloc";
+    if (!segs) return fail(SPLAT_E_NULL, "%s: null pointer argument", who);
+    if (L <= 0 || L > (1 << 23)) return fail(SPLAT_E_SHAPE, "%s: need 0 < L <= 2^23 (got %d)", who, L);
+    const int64_t need = splat_attention_plan_bytes(segs, n_seg, L);
+    if (need <= 0) return fail(SPLAT_E_SHAPE, "%s: no plan for n_seg=%d, L=%d", who, n_seg, L);
+    if (need > kStaticPlanBytes)
+        return fail(SPLAT_E_SHAPE,
+                    "%s: this mask's plan needs %lld bytes, the built-in buffer holds %lld (about %lld row blocks of 128 rows "
+                    "times segments); use splat_attention_plan + splat_attention_fwd_planned with a buffer of your own",
+                    who, (long long)need, (long long)kStaticPlanBytes,
+                    (long long)(kStaticPlanBytes / (2 * plan_variant_recs(1, 1) * (int64_t)sizeof(PlanRec))));
+    void* plan = nullptr;
+    if (int rc = static_plan_buffer(who, &plan)) return rc;
+    // the plan kernel rewrites every record this mask's forward reads, so nothing of an earlier call's plan is seen;
+    // the forward follows on the same stream
+    if (int rc = splat_attention_plan(segs, n_seg, L, plan, kStaticPlanBytes, stream)) return rc;
+    return attention_fwd_common(who, q, q_sb, q_sh, q_sl, kT, k_sb, k_sh, k_sd, k_sl, v, v_sb, v_sh, v_sl, out, o_sb, o_sh, o_sl,
+                                segs, n_seg, B, H, L, d, scale, dtype, plan, kStaticPlanBytes, true, nullptr, stream);
 }
