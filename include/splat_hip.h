@@ -224,6 +224,11 @@ int splat_attention_fwd_noalloc(const void* q, int64_t q_sb, int64_t q_sh, int64
                                 int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t d, float scale,
                                 int32_t dtype, void* stream);
 
+/* Measurement aid, no counterpart in the reference: copy `bytes` (a multiple of 16; both pointers 16-byte aligned) from
+ * src to dst with the access forms of the HBM-bound kernels here (16 bytes per lane, non-temporal, several requests
+ * in flight).  Its rate is the read + write streaming ceiling that bench.py quotes splat_softmax against. */
+int splat_stream_copy(const void* src, void* dst, int64_t bytes, void* stream);
+
 /* ---- backward pass (the reference has none: r_attention.py:77-100 is forward only) ----
  * With S~ the compressed scores, P~ = softmax(S~), O = P~ . V:
  *   dP~ = splat_sddmm(x = dO, y = V viewed as [d, L])           dQ = splat_spmm(p = dS~, v = K)

@@ -322,3 +322,18 @@ def test_a_segment_that_is_empty_everywhere_is_dropped(dev):
     got = out.cpu()
     for r in (0, 37, 99):
         assert float((got[0, 1, r, :r + 1] - want[0, 1, r, :r + 1]).abs().max()) <= 1e-4
+
+
+@pytest.mark.parametrize("n_bytes", [16, 4096 * 16, (4096 * 3 + 1000) * 16 + 48, 64 << 20])
+def test_stream_copy_copies(dev, n_bytes):
+    """splat_stream_copy, the streaming ceiling bench.py quotes the softmax against, is a faithful copy: whole chunks
+    and the tail that does not fill one, and nothing past the end."""
+    import _splat_hip as hip
+    g = torch.Generator().manual_seed(n_bytes % 1000)
+    src = torch.randint(0, 256, (n_bytes + 64,), dtype=torch.uint8, generator=g).to(dev)
+    dst = torch.full((n_bytes + 64,), 7, dtype=torch.uint8, device=dev)
+    hip.check(hip.lib().splat_stream_copy(src.data_ptr(), dst.data_ptr(), n_bytes, hip.stream_ptr(dev)), "splat_stream_copy")
+    assert torch.equal(dst[:n_bytes], src[:n_bytes])
+    assert torch.all(dst[n_bytes:] == 7)
+    assert hip.lib().splat_stream_copy(src.data_ptr(), dst.data_ptr(), 24, None) == -2
+    assert hip.lib().splat_stream_copy(src.data_ptr() + 8, dst.data_ptr(), 32, None) == -4

@@ -76,21 +76,25 @@ struct RowScan {
     }
 };
 
-__global__ void acsr_init_summary(int32_t* summary) {
-    if (threadIdx.x < 8) summary[threadIdx.x] = (threadIdx.x == 2) ? 0x7fffffff : 0;
+// The summary's starting values, written by the first workgroup of the rows kernel (no kernel of its own): the rows
+// kernels themselves never touch the summary otherwise, the span kernel that follows them reduces into it.
+__device__ __forceinline__ void init_summary(int32_t* summary) {
+    if (blockIdx.x == 0 && threadIdx.x < 8) summary[threadIdx.x] = (threadIdx.x == 2) ? 0x7fffffff : 0;
 }
+constexpr float kUnpackFailed = 0.0f;  // stored as a row's sTod_lin (a real step is >= 1) until the span kernel has counted it
 
 // What one row contributes once its scan is reduced: the closed-form 2x2 solve.  (The summary extrema are
 // reduced by the span kernel: per-row atomics on one address cost more than streaming the whole mask.)
 __device__ __forceinline__ void finish_row(const RowScan& s, int row, int cols, float* dTos_lin, float* dTos_trans,
                                            float* sTod_lin, float* sTod_trans, float* nnz_out, int32_t* row_first,
-                                           int32_t* row_last, int32_t* summary) {
+                                           int32_t* row_last) {
     const int nnz = (int)s.sum;
     double x0 = 1.0, x1 = 0.0;
     int step = 1;
+    bool failed = false;
     if (nnz > 1) {
         if (s.m1 == kInf || s.m2 == kInf) {
-            atomicAdd(&summary[1], 1);  // the reference asserts here (acsr_helpers.py:119)
+            failed = true;  // the reference asserts here (acsr_helpers.py:119); counted by the span kernel
         } else {
             step = s.m2 - s.m1;
             x0 = 1.0 / (double)step;
@@ -100,7 +104,7 @@ __device__ __forceinline__ void finish_row(const RowScan& s, int row, int cols, 
     }
     dTos_lin[row] = (float)x0;
     dTos_trans[row] = (float)x1;
-    sTod_lin[row] = (float)step;
+    sTod_lin[row] = failed ? kUnpackFailed : (float)step;
     sTod_trans[row] = (float)fabs(x1);
     nnz_out[row] = (float)nnz;
     if (row_first) row_first[row] = (s.first == kInf) ? cols : s.first;
@@ -122,6 +126,7 @@ __global__ __launch_bounds__(256) void acsr_rows_kernel(const uint8_t* __restric
                                                         float* __restrict__ sTod_trans, float* __restrict__ nnz_out,
                                                         int32_t* __restrict__ row_first,
                                                         int32_t* __restrict__ row_last, int32_t* __restrict__ summary) {
+    init_summary(summary);
     const int lane = threadIdx.x & 63;
     const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= rows) return;
@@ -137,7 +142,7 @@ __global__ __launch_bounds__(256) void acsr_rows_kernel(const uint8_t* __restric
     }
     for (int c = done + lane; c < cols; c += 64) s.byte(p[c], c);
     s.wave_reduce();
-    if (lane == 0) finish_row(s, row, cols, dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnz_out, row_first, row_last, summary);
+    if (lane == 0) finish_row(s, row, cols, dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnz_out, row_first, row_last);
 }
 
 // Long rows (>= 4 KiB, 16-byte aligned): one workgroup per row, so that the memory system sees a few thousand
@@ -148,6 +153,7 @@ __global__ __launch_bounds__(256) void acsr_rows_wide_kernel(const uint8_t* __re
                                                              float* __restrict__ sTod_trans, float* __restrict__ nnz_out,
                                                              int32_t* __restrict__ row_first,
                                                              int32_t* __restrict__ row_last, int32_t* __restrict__ summary) {
+    init_summary(summary);
     __shared__ uint32_t s_sum[4];
     __shared__ int s_m1[4], s_m2[4], s_first[4], s_last[4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -196,7 +202,7 @@ __global__ __launch_bounds__(256) void acsr_rows_wide_kernel(const uint8_t* __re
             t.first = min(t.first, s_first[w]);
             t.last = max(t.last, s_last[w]);
         }
-        finish_row(t, row, cols, dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnz_out, row_first, row_last, summary);
+        finish_row(t, row, cols, dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnz_out, row_first, row_last);
     }
 }
 
@@ -204,19 +210,24 @@ __global__ __launch_bounds__(256) void acsr_rows_wide_kernel(const uint8_t* __re
 // evaluated in double from the exact integers (a, lin, nnz) and rounded once to float32.  The same pass reduces
 // the summary: T = max nnz, smallest / largest column step over rows with nnz > 1, and how many rows with
 // nnz > 1 have a first column that is not congruent to the row index modulo their step.
-__global__ __launch_bounds__(256) void acsr_spans_kernel(const float* __restrict__ sTod_lin,
+__global__ __launch_bounds__(256) void acsr_spans_kernel(float* __restrict__ sTod_lin,
                                                          const float* __restrict__ sTod_trans,
                                                          const float* __restrict__ nnz, int rows, int cols,
                                                          int block_height, float* __restrict__ span_start,
                                                          float* __restrict__ span_end, int32_t* __restrict__ summary) {
     const int g = blockIdx.x * blockDim.x + threadIdx.x;
     const int n_blocks = (rows + block_height - 1) / block_height;
-    int t_max = 0, step_min = 0x7fffffff, step_max = 0, off_phase = 0;
+    int t_max = 0, step_min = 0x7fffffff, step_max = 0, off_phase = 0, failed = 0;
     if (g < n_blocks) {
         double lo = (double)cols, hi = -1.0;
         const int r1 = min(rows, (g + 1) * block_height);
         for (int r = g * block_height; r < r1; ++r) {
-            const float linf = sTod_lin[r];
+            float linf = sTod_lin[r];
+            if (linf == kUnpackFailed) {  // a row the reference would have asserted on: counted, then stored as (1, 0) like
+                ++failed;                 // the rows with at most one live column
+                linf = 1.0f;
+                sTod_lin[r] = linf;
+            }
             const int lin = (int)linf;
             const int a = (int)rintf(linf * sTod_trans[r]);
             const int cnt = (int)nnz[r];
@@ -237,7 +248,9 @@ __global__ __launch_bounds__(256) void acsr_spans_kernel(const float* __restrict
     step_min = wave_min_i(step_min);
     step_max = wave_max_i(step_max);
     off_phase = (int)wave_sum((float)off_phase);  // at most 64 * block_height per wavefront: exact in float
+    failed = (int)wave_sum((float)failed);
     if ((threadIdx.x & 63) == 0) {
+        if (failed) atomicAdd(&summary[1], failed);
         atomicMax(&summary[0], t_max);
         atomicMin(&summary[2], step_min);
         atomicMax(&summary[3], step_max);
@@ -370,10 +383,11 @@ __global__ __launch_bounds__(256) void acsr_rows_pattern_kernel(int pattern, int
                                                                 float* __restrict__ sTod_lin, float* __restrict__ sTod_trans,
                                                                 float* __restrict__ nnz_out, int32_t* __restrict__ row_first,
                                                                 int32_t* __restrict__ row_last, int32_t* __restrict__ summary) {
+    init_summary(summary);
     const int row = blockIdx.x * blockDim.x + threadIdx.x;
     if (row >= s) return;
     finish_row(pattern_row(pattern, row, s, p0, p1), row, s, dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnz_out, row_first,
-               row_last, summary);
+               row_last);
 }
 
 __global__ __launch_bounds__(256) void mask_generate_kernel(uint8_t* __restrict__ mask, int rows, int cols,
@@ -417,7 +431,6 @@ extern "C" int splat_acsr_build(const uint8_t* mask, int64_t rows, int64_t cols,
         return fail(SPLAT_E_SHAPE, "splat_acsr_build: rows and cols are limited to 2^23 (got %lld, %lld)", (long long)rows, (long long)cols);
     hipStream_t st = (hipStream_t)stream;
     const int vec_ok = ((reinterpret_cast<uintptr_t>(mask) & 15) == 0 && (ld & 15) == 0) ? 1 : 0;
-    acsr_init_summary<<<1, 64, 0, st>>>(summary);
     if (vec_ok && cols >= 4096)
         acsr_rows_wide_kernel<<<(unsigned)rows, 256, 0, st>>>(mask, (int)rows, (int)cols, ld, dTos_lin, dTos_trans, sTod_lin,
                                                               sTod_trans, nnz, row_first, row_last, summary);
@@ -453,7 +466,6 @@ extern "C" int splat_acsr_build_pattern(int32_t pattern, int64_t s, int64_t p0, 
     if (int rc = check_pattern(who, s, pattern, p0, p1)) return rc;
     if (p0 > (1 << 23) || p1 > (1 << 23)) return fail(SPLAT_E_SHAPE, "%s: pattern parameters are limited to 2^23", who);
     hipStream_t st = (hipStream_t)stream;
-    acsr_init_summary<<<1, 64, 0, st>>>(summary);
     acsr_rows_pattern_kernel<<<(unsigned)((s + 255) / 256), 256, 0, st>>>(pattern, (int)s, p0, p1, dTos_lin, dTos_trans, sTod_lin,
                                                                          sTod_trans, nnz, row_first, row_last, summary);
     const int n_blocks = (int)((s + block_height - 1) / block_height);

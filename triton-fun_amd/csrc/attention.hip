@@ -240,12 +240,17 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
     // FAST_DMA state for the segment being fetched: per-lane byte offsets inside a block, wavefront-uniform
     // running pointers to block `wave` of the next tile, and the byte distance between tile positions.
     uint32_t v_lane_off = 0, k_lane_off = 0;
+    bool lane_off_fits = true;  // the copy instruction takes a 32-bit per-lane offset: wider ones go the general way
     const char* v_next = nullptr;
     const char* k_next = nullptr;
     int64_t v_key = 0, k_key = 0;  // bytes from one tile position to the next (K^T layout: from one d row to the next)
     auto set_lane_offsets = [&](const SegPlan& pl) {
         if constexpr (FAST_DMA) {
             const int vr = lane / V_CPR, vpc = lane % V_CPR;
+            // the largest offsets of the segment: the last row of a block, with gathered rows pl.cs keys apart
+            const int64_t v_far = (int64_t)pl.cs * (V_RPI - 1) * p.v_sl * ES + G::V_ROWB;
+            const int64_t k_far = KT ? (int64_t)(K_RPI - 1) * p.k_sd * ES + G::K_ROWB : (int64_t)pl.cs * (K_RPI - 1) * p.k_sl * ES + G::K_ROWB;
+            lane_off_fits = v_far < ((int64_t)1 << 32) && k_far < ((int64_t)1 << 32);
             v_lane_off = (uint32_t)((int64_t)pl.cs * vr * p.v_sl * ES) + logical_chunk<G::V_ROWB, 2>(vr, vpc) * 16;
             v_key = (int64_t)p.v_sl * ES * pl.cs;
             v_next = reinterpret_cast<const char*>(vb) + (int64_t)pl.c0 * p.v_sl * ES + (int64_t)wave * V_RPI * v_key;
@@ -266,7 +271,7 @@ __global__ __launch_bounds__(256, sizeof(T) == 2 ? 2 : 1) void attn_fwd_kernel(c
     auto tile_is_fast = [&](const SegPlan& pl, int tile) {
         const int j0 = tile * BN;
         const int key_first = pl.c0 + pl.cs * j0, key_last = pl.c0 + pl.cs * (j0 + BN - 1);
-        bool fast = FAST_DMA && key_last < L;
+        bool fast = FAST_DMA && lane_off_fits && key_last < L;
         if constexpr (KT) fast = fast && (key_first + BN <= L);
         return fast;
     };
