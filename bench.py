@@ -117,6 +117,50 @@ def time_cold_launches(fn, scratch, steps: int):
     return sum(a.elapsed_time(b) for a, b in evs) / steps
 
 
+def sample_power_and_clock(fn, launches_per_batch: int = 50):
+    """Socket power (W) and graphics clock (MHz) as `amd-smi metric -p -c` reports them while `fn` is launched back to
+    back: two readings at least a second into the loop, averaged.  None when the tool is missing or prints no figures."""
+    import re
+    import shutil
+    import subprocess
+    import threading
+
+    import torch
+
+    tool = shutil.which("amd-smi")
+    if tool is None:
+        return None
+    readings, done = [], threading.Event()
+
+    def reader():
+        try:
+            time.sleep(1.0)
+            for _ in range(2):
+                txt = subprocess.run([tool, "metric", "-p", "-c"], capture_output=True, text=True, timeout=10).stdout
+                pw = re.search(r"SOCKET_POWER:\s*([0-9.]+)\s*W", txt)
+                ck = re.search(r"GFX_0:\s*\n\s*CLK:\s*([0-9.]+)\s*MHz", txt)
+                if pw and ck:
+                    readings.append((float(pw.group(1)), float(ck.group(1))))
+        except Exception:
+            pass
+        finally:
+            done.set()
+
+    th = threading.Thread(target=reader, daemon=True)
+    th.start()
+    t_end = time.perf_counter() + 30.0
+    while not done.is_set() and time.perf_counter() < t_end:
+        for _ in range(launches_per_batch):
+            fn()
+        torch.cuda.synchronize()
+    th.join(timeout=15.0)
+    if not readings:
+        return None
+    return {"socket_power_w": round(sum(r[0] for r in readings) / len(readings), 1),
+            "gfx_clk_mhz": round(sum(r[1] for r in readings) / len(readings), 1),
+            "source": "amd-smi metric -p -c, two readings during a sustained loop of the kernel"}
+
+
 def make_inputs(seed: int, B: int, H: int, L: int, d: int, dtype):
     """Seeded q, k, v ~ N(0,1), drawn in fp32 on the host in that order, then cast."""
     import torch
@@ -147,6 +191,7 @@ def main() -> int:
     import numpy as np
     import torch
 
+    import _splat_hip as hip
     import acsr_helpers as A
     import r_softmax
     import r_sddmm
@@ -217,6 +262,26 @@ def main() -> int:
         "acsr_setup_ms": round(setup_ms, 2),
     }
 
+    if not args.no_settle:
+        # What limits the clock: power and clock while the headline kernel runs back to back, and the rate of the bare
+        # matrix loop of the same tile shape (LDS reads + MFMAs only, random operands) under the same conditions.
+        out["roofline"]["sustained"] = sample_power_and_clock(step)
+        probe_data = torch.randn(32768, dtype=torch.float32).to(dtype).to(dev)
+        probe_wgs, probe_tiles = B * H * (L // 128), 40
+        probe_out = torch.empty(probe_wgs * 256, dtype=torch.float32, device=dev)
+        probe = lambda: hip.check(hip.lib().splat_mfma_lds_probe(probe_data.data_ptr(), probe_data.numel() * 2, probe_out.data_ptr(),
+                                                                 probe_out.numel() * 4, probe_wgs, probe_tiles, hip.stream_ptr(dev)),
+                                  "splat_mfma_lds_probe")
+        settle(probe)
+        probe_ms = min(time_batch(probe, 20, 5) for _ in range(3))
+        probe_tflops = probe_wgs * probe_tiles * 4 * 32 * 32768 / (probe_ms * 1e-3) / 1e12
+        out["roofline"]["mfma_lds_loop"] = {
+            "tflops": round(probe_tflops, 1), "frac_of_peak": round(probe_tflops / MFMA_PEAK_TFLOPS, 4),
+            "fused_frac_of_loop": round(kern_tflops / probe_tflops, 4), "sustained": sample_power_and_clock(probe, 10),
+            "note": "splat_mfma_lds_probe: the fused kernel's LDS reads and MFMAs per tile and nothing else, N(0,1) bf16 "
+                    "operands, same grid; its MFMAs are all counted, the fused figure counts nonzero FLOPs only"}
+        del probe_data, probe_out
+
     extras = {}
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
@@ -255,7 +320,6 @@ def main() -> int:
         # ACSR build on the config-5 mask (L*L bytes read once): create_acsr as a caller sees it (it ends with a read-back of
         # T, i.e. a stream synchronisation), and the builder's two kernels alone through the C ABI, each launch after a
         # 512 MiB write so that the freshly generated mask is not found in a cache
-        import _splat_hip as hip
         mask = A.causal_windowed_pattern(L, w - 1).device_mask(dev)
 
         def build():

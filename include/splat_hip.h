@@ -229,6 +229,16 @@ int splat_attention_fwd_noalloc(const void* q, int64_t q_sb, int64_t q_sh, int64
  * in flight).  Its rate is the read + write streaming ceiling that bench.py quotes splat_softmax against. */
 int splat_stream_copy(const void* src, void* dst, int64_t bytes, void* stream);
 
+/* Measurement aid, no counterpart in the reference: `workgroups` workgroups of 256 threads each run `tiles` times the
+ * LDS reads and MFMAs of one 64-key tile of the fused forward at d = 128 in bf16 (2 x 16 MFMAs of 32x32x16 per
+ * wavefront and tile, i.e. workgroups * tiles * 4 * 32 * 32768 floating-point operations per call), with no global
+ * loads, copies, exponentials or barriers in the loop.  The 64 KiB at `data` (16-byte aligned; give it random bf16
+ * values: the switching activity of the operands decides the clock a power-limited part reaches) fill the LDS; `out`
+ * receives one float per thread.  The rate of this loop is the matrix ceiling that bench.py quotes the fused forward
+ * against, beside the rated peak. */
+int splat_mfma_lds_probe(const void* data, int64_t data_bytes, void* out, int64_t out_bytes, int32_t workgroups,
+                         int32_t tiles, void* stream);
+
 /* ---- backward pass (the reference has none: r_attention.py:77-100 is forward only) ----
  * With S~ the compressed scores, P~ = softmax(S~), O = P~ . V:
  *   dP~ = splat_sddmm(x = dO, y = V viewed as [d, L])           dQ = splat_spmm(p = dS~, v = K)

@@ -337,3 +337,28 @@ def test_stream_copy_copies(dev, n_bytes):
     assert torch.all(dst[n_bytes:] == 7)
     assert hip.lib().splat_stream_copy(src.data_ptr(), dst.data_ptr(), 24, None) == -2
     assert hip.lib().splat_stream_copy(src.data_ptr() + 8, dst.data_ptr(), 32, None) == -4
+
+
+def test_mfma_lds_probe_runs_and_checks_its_arguments(dev):
+    """splat_mfma_lds_probe, the matrix loop bench.py quotes the fused forward against: every workgroup computes the same
+    figures from the same 64 KiB, zeros give zeros, two calls agree, and short buffers are refused."""
+    import _splat_hip as hip
+    data = torch.randn(32768, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16).to(dev)
+    wgs, tiles = 6, 3
+    out = torch.full((wgs * 256 + 8,), 7.0, dtype=torch.float32, device=dev)
+    call = lambda d, o, w=wgs, t=tiles: hip.lib().splat_mfma_lds_probe(d.data_ptr(), d.numel() * 2, o.data_ptr(), wgs * 256 * 4, w, t,
+                                                                     hip.stream_ptr(dev))
+    hip.check(call(data, out), "splat_mfma_lds_probe")
+    res = out[:wgs * 256].view(wgs, 256)
+    assert torch.isfinite(res).all() and float(res.abs().max()) > 0
+    assert torch.equal(res, res[0].expand_as(res))
+    assert torch.all(out[wgs * 256:] == 7.0)
+    again = torch.empty_like(out)
+    hip.check(call(data, again), "splat_mfma_lds_probe")
+    assert torch.equal(again[:wgs * 256], out[:wgs * 256])
+    hip.check(call(torch.zeros_like(data), again), "splat_mfma_lds_probe")
+    assert torch.all(again[:wgs * 256] == 0)
+    assert hip.lib().splat_mfma_lds_probe(data.data_ptr(), 65535, out.data_ptr(), wgs * 256 * 4, wgs, tiles, None) == -2
+    assert hip.lib().splat_mfma_lds_probe(data.data_ptr(), 65536, out.data_ptr(), wgs * 256 * 4 - 1, wgs, tiles, None) == -2
+    assert hip.lib().splat_mfma_lds_probe(data.data_ptr(), 65536, out.data_ptr(), wgs * 256 * 4, 0, tiles, None) == -2
+    assert hip.lib().splat_mfma_lds_probe(data.data_ptr() + 2, 65536, out.data_ptr(), wgs * 256 * 4, wgs, tiles, None) == -4
