@@ -180,6 +180,9 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the host baseline")
     ap.add_argument("--no-extras", action="store_true", help="skip the unfused kernels and the ACSR build")
     ap.add_argument("--cpu-heads", type=int, default=16, help="(batch, head) pairs the host baseline computes")
+    ap.add_argument("--zero-operands", action="store_true",
+                    help="power / clock studies only: q, k and v are all zeros (no switching in the multipliers), which says how "
+                         "much of the time is the power limit's; the line is marked and is not a result")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy, the known-size kernel that HBM counters are scaled by")
     args = ap.parse_args()
@@ -209,6 +212,8 @@ def main() -> int:
     scale = d ** -0.5
     q, k, v = make_inputs(1005, B, H, L, d, dtype)
     qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    if args.zero_operands:
+        qd.zero_(), kd.zero_(), vd.zero_()
     kT_view = kd.transpose(2, 3)
 
     t0 = time.perf_counter()
@@ -247,7 +252,8 @@ def main() -> int:
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
-        "data": "synthetic: seeded N(0,1) q/k/v (torch.Generator cpu seed 1005), resident in HBM",
+        "data": ("ALL-ZERO q/k/v (--zero-operands: a power study, not a result)" if args.zero_operands else
+                 "synthetic: seeded N(0,1) q/k/v (torch.Generator cpu seed 1005), resident in HBM"),
         "config": {"workload": "config 5: fused ACSR attention fwd, B=4 H=16 L=16384 d=128 bf16, causal window 512, "
                                "scale 1/sqrt(d), K passed as k.transpose(2,3)",
                    "B": B, "H": H, "L": L, "d": d, "window": w, "nnz_per_head": nnz},
@@ -267,6 +273,8 @@ def main() -> int:
         # matrix loop of the same tile shape (LDS reads + MFMAs only, random operands) under the same conditions.
         out["roofline"]["sustained"] = sample_power_and_clock(step)
         probe_data = torch.randn(32768, dtype=torch.float32).to(dtype).to(dev)
+        if args.zero_operands:
+            probe_data.zero_()
         probe_wgs, probe_tiles = B * H * (L // 128), 40
         probe_out = torch.empty(probe_wgs * 256, dtype=torch.float32, device=dev)
         probe = lambda: hip.check(hip.lib().splat_mfma_lds_probe(probe_data.data_ptr(), probe_data.numel() * 2, probe_out.data_ptr(),
