@@ -402,6 +402,20 @@ def main() -> int:
         extras["softmax_cfg4"]["frac_of_stream_copy"] = round(extras["softmax_cfg4"]["gbps_algorithmic"] /
                                                               extras["stream_copy_1GiB"]["gbps_read_plus_write"], 4)
         del src, dst
+        # the softmax on config 3's compressed rows: two segments, T = 191 slots, so rows begin anywhere inside a 16-byte chunk
+        pat3 = A.strided_patterns(8192, 128, 128)
+        segs3 = A.create_acsr_segments(pat3, 16, dev)
+        B3, H3, L3, T3 = 2, 16, 8192, segs3.T
+        live3 = int(sum(float(t[4].sum()) for t in segs3.tuples))
+        s3 = torch.randn(B3, H3, L3, T3, device=dev, dtype=dtype)
+        p3 = torch.empty_like(s3)
+        sg0 = segs3.tuples[0]
+        run_soft3 = lambda: r_softmax.rsoftmax_launcher(s3, p3, sg0[0], sg0[1], sg0[2], sg0[3], T3, 256, sg0[4], (1, 1), 16, segments=segs3)
+        ms = min(time_batch(run_soft3, 40, 10) for _ in range(3))
+        byt3 = 2 * live3 * B3 * H3 * 2
+        extras["softmax_cfg3"] = {"ms": round(ms, 4), "T": T3, "gbps_algorithmic": round(byt3 / ms / 1e6, 1),
+                                  "hbm_frac": round(byt3 / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+        del s3, p3
         del s_buf, p_buf, o_buf, flush
         # backward pass (not in the reference) at the same shape: nonzero FLOPs = 2.5 x the forward's (five products)
         attn4 = RegularAttention(B4, L4, H4, d4, pat4, 16, 16, dev, dtype, scale=d4 ** -0.5)

@@ -251,6 +251,37 @@ def test_softmax_patterns(dev, in_dt, out_dt, make):
         assert float((xd.float().cpu() - want)[..., lv].abs().max()) <= TOL[out_dt]
 
 
+@pytest.mark.parametrize("in_dt,out_dt", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float32), (torch.float32, torch.float32)])
+@pytest.mark.parametrize("L,w", [(3, 4), (40, 12), (300, 190), (260, 249), (1100, 1000), (2100, 2030), (2100, 2034)])
+def test_softmax_row_widths_that_are_not_multiples_of_eight(dev, in_dt, out_dt, L, w):
+    """Rows of T = w + 1 slots start anywhere inside an 8-element chunk (T = 191 is config 3's width): every live slot
+    matches the oracle, dead slots and the elements after the buffer keep what they held, also in place."""
+    mask = O.create_causal_windowed_mask(L, w)
+    acsr, acsr_np = acsr_pair(mask, 16, dev)
+    T = acsr[5]
+    assert T == min(L, w + 1) and (T % 8 != 0 or L < 8)
+    BH = (3, 1)
+    g = torch.Generator().manual_seed(T)
+    x = (torch.randn(*BH, L, T, generator=g) * 3).to(in_dt)
+    lv = live(acsr_np)
+    want = O.softmax_compressed(x.float(), lv)
+    n = x.numel()
+    buf = torch.full((n + 64,), SENTINEL, dtype=out_dt, device=dev)
+    out = buf[:n].view(*BH, L, T)
+    r_softmax.rsoftmax_launcher(x.to(dev), out, acsr[0], acsr[1], acsr[2], acsr[3], T, O.rsoftmax_pow2(T), acsr[4], (1, 1), 16)
+    got = out.float().cpu()
+    assert float((got - want)[..., lv].abs().max()) <= TOL[out_dt]
+    assert torch.all(got[..., ~lv] == SENTINEL)
+    assert torch.all(buf[n:] == SENTINEL)
+    if in_dt == out_dt:
+        inbuf = torch.full((n + 64,), SENTINEL, dtype=in_dt, device=dev)
+        xd = inbuf[:n].view(*BH, L, T)
+        xd.copy_(x)
+        r_softmax.rsoftmax_launcher(xd, xd, acsr[0], acsr[1], acsr[2], acsr[3], T, O.rsoftmax_pow2(T), acsr[4], (1, 1), 16)
+        assert float((xd.float().cpu() - want)[..., lv].abs().max()) <= TOL[out_dt]
+        assert torch.all(inbuf[n:] == SENTINEL)
+
+
 # ---------------------------------------------------------------- SpMM
 @pytest.mark.parametrize("n,p", REF_SMALL)
 def test_spmm_reference_cases(dev, n, p):

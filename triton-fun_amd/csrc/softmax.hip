@@ -3,8 +3,10 @@
 // One wavefront owns one row.  The row's live slots are read once with 16/32-byte loads (8 elements
 // per lane per step), kept in registers, reduced with wavefront shuffles (max, then sum of
 // exp2((x - max) * log2 e)) and written back once; dead slots (s >= nnz) are neither read as data nor
-// written.  HBM-bound: 2 * live slots * element size bytes per row.  Rows longer than 2048 slots, or
-// whose length is not a multiple of 8, take a three-pass kernel that re-reads the row from cache.
+// written.  HBM-bound: 2 * live slots * element size bytes per row.  Rows whose length is not a multiple of 8 start
+// at any element of an 8-element chunk: they are read as the aligned chunks that cover them (a chunk at a row's end
+// also holds its neighbour's first slots, which are discarded) and written whole where a chunk is all theirs, element by
+// element at the two ends.  Rows longer than 2048 slots take a three-pass kernel that re-reads the row from cache.
 #include "splat_common.hpp"
 
 namespace splat {
@@ -35,7 +37,7 @@ struct LiveRanges {
         for (int k = 0; k < SPLAT_MAX_SEGMENTS; ++k) v |= (k < n) && slot >= lo[k] && slot < hi[k];
         return v;
     }
-    // 8-bit liveness of slots [s0, s0+8)
+    // 8-bit liveness of slots [s0, s0+8); s0 may be negative (a chunk that begins before the row does)
     __device__ __forceinline__ uint32_t live8(int s0) const {
         uint32_t m = 0;
 #pragma unroll
@@ -60,7 +62,8 @@ constexpr float kNegBig = -1.0e30f;
 // LPR lanes share one row (64 / LPR rows per wavefront): rows shorter than 512 slots still fill every lane.  A wavefront
 // takes RIF such row groups at once and requests all of their chunks before it looks at any (bytes in flight per
 // wavefront are what a streaming kernel lives on).
-template <typename Tin, typename Tout, int NCH, int LPR, int RIF>
+// SHIFT: T is not a multiple of 8, so row r begins (r * T) % 8 elements into an aligned chunk.
+template <typename Tin, typename Tout, int NCH, int LPR, int RIF, bool SHIFT>
 __global__ __launch_bounds__(256) void softmax_rows_vec(const Tin* __restrict__ x, Tout* __restrict__ y, SoftmaxSegs segs,
                                                         int64_t n_rows, int L, int T) {
     typedef typename Vec8<Tin>::type vin;
@@ -69,37 +72,51 @@ __global__ __launch_bounds__(256) void softmax_rows_vec(const Tin* __restrict__ 
     const int lane = threadIdx.x & (LPR - 1);
     const int64_t row0 = (((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * RIF) * RPW + ((threadIdx.x & 63) / LPR);
     if (RPW == 1 && row0 >= n_rows) return;
-    const int nchunk = T >> 3;
+    const int64_t total = n_rows * (int64_t)T;
 
     // the loads do not wait for the rows' live counts: a chunk inside the row is fetched whole and the dead
     // slots in it are discarded afterwards
     vin raw[RIF][NCH];
     bool row_ok[RIF];
     int64_t row[RIF];
+    int shift[RIF], nchunk[RIF];  // elements of the first chunk that precede the row; chunks that cover the row
 #pragma unroll
     for (int i = 0; i < RIF; ++i) {
         const int64_t row_raw = row0 + (int64_t)i * RPW;
         row_ok[i] = row_raw < n_rows;
         row[i] = row_ok[i] ? row_raw : n_rows - 1;  // surplus lane groups shadow the last row and store nothing
-        const Tin* xr = x + row[i] * (int64_t)T;
+        const int64_t first = row[i] * (int64_t)T;
+        shift[i] = SHIFT ? (int)(first & 7) : 0;
+        nchunk[i] = (T + shift[i] + 7) >> 3;
+        const Tin* xr = x + (first - shift[i]);
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             const int ch = lane + LPR * c;
-            if (ch < nchunk) raw[i][c] = __builtin_nontemporal_load(reinterpret_cast<const vin*>(xr + (ch << 3)));
+            if (ch < nchunk[i]) {
+                if constexpr (!SHIFT) {
+                    raw[i][c] = __builtin_nontemporal_load(reinterpret_cast<const vin*>(xr + (ch << 3)));
+                } else if (first - shift[i] + (ch << 3) + 8 <= total) {
+                    // rows share the lines at their ends with their neighbours: through the cache, not around it
+                    raw[i][c] = *reinterpret_cast<const vin*>(xr + (ch << 3));
+                } else {  // the last chunk of the buffer ends beyond it: only the elements that exist
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) raw[i][c][e] = first - shift[i] + (ch << 3) + e < total ? xr[(ch << 3) + e] : (Tin)0.f;
+                }
+            }
         }
     }
 #pragma unroll
     for (int i = 0; i < RIF; ++i) {
         LiveRanges lr;
         lr.load(segs, (int)(row[i] % L), T);
-        Tout* yr = y + row[i] * (int64_t)T;
+        Tout* yr = y + (row[i] * (int64_t)T - shift[i]);  // chunk ch of the row = elements 8*ch .. 8*ch+7 from here
         float v[NCH][8];
         uint32_t live[NCH];
         float mx = kNegBig;
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             const int ch = lane + LPR * c;
-            live[c] = (ch < nchunk) ? lr.live8(ch << 3) : 0u;
+            live[c] = (ch < nchunk[i]) ? lr.live8((ch << 3) - shift[i]) : 0u;
             if (live[c]) {
                 const vin t = raw[i][c];
 #pragma unroll
@@ -135,7 +152,10 @@ __global__ __launch_bounds__(256) void softmax_rows_vec(const Tin* __restrict__ 
                     vout o;
 #pragma unroll
                     for (int e = 0; e < 8; ++e) o[e] = (Tout)(v[c][e] * inv);
-                    __builtin_nontemporal_store(o, reinterpret_cast<vout*>(yr + (ch << 3)));
+                    if constexpr (SHIFT)
+                        *reinterpret_cast<vout*>(yr + (ch << 3)) = o;
+                    else
+                        __builtin_nontemporal_store(o, reinterpret_cast<vout*>(yr + (ch << 3)));
                 } else {
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
@@ -178,21 +198,35 @@ static int launch_softmax(const void* x, void* y, const SoftmaxSegs& segs, int64
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 31) == 0;
     const Tin* xi = (const Tin*)x;
     Tout* yo = (Tout*)y;
-    if (aligned && (T & 7) == 0 && T <= 2048) {
+    if (aligned && (T & 7) != 0 && T <= 2032) {
+        // rows that start anywhere in a chunk: up to T/8 + 2 chunks cover one
+        const int chunks = T / 8 + 2;
+        auto groups = [&](int rows_per_wave) { return (unsigned)((n_rows + 4 * rows_per_wave - 1) / (4 * rows_per_wave)); };
+        if (chunks <= 16)
+            softmax_rows_vec<Tin, Tout, 1, 16, 1, true><<<groups(4), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+        else if (chunks <= 32)
+            softmax_rows_vec<Tin, Tout, 1, 32, 4, true><<<groups(2 * 4), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+        else if (chunks <= 64)
+            softmax_rows_vec<Tin, Tout, 1, 64, 4, true><<<groups(4), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+        else if (chunks <= 128)
+            softmax_rows_vec<Tin, Tout, 2, 64, 1, true><<<groups(1), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+        else
+            softmax_rows_vec<Tin, Tout, 4, 64, 1, true><<<groups(1), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+    } else if (aligned && (T & 7) == 0 && T <= 2048) {
         const int nch = (T / 8 + 63) / 64;
         // row groups in flight per wavefront: 4 where a row is 512 bytes or more (+7 % at T = 512, +4 % at T = 256 over
         // one group, measured), one for shorter rows (more was slower there)
         auto groups = [&](int rows_per_wave) { return (unsigned)((n_rows + 4 * rows_per_wave - 1) / (4 * rows_per_wave)); };
         if (T <= 128)
-            softmax_rows_vec<Tin, Tout, 1, 16, 1><<<groups(4), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+            softmax_rows_vec<Tin, Tout, 1, 16, 1, false><<<groups(4), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
         else if (T <= 256)
-            softmax_rows_vec<Tin, Tout, 1, 32, 4><<<groups(2 * 4), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+            softmax_rows_vec<Tin, Tout, 1, 32, 4, false><<<groups(2 * 4), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
         else if (nch <= 1)
-            softmax_rows_vec<Tin, Tout, 1, 64, 4><<<groups(4), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+            softmax_rows_vec<Tin, Tout, 1, 64, 4, false><<<groups(4), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
         else if (nch <= 2)
-            softmax_rows_vec<Tin, Tout, 2, 64, 1><<<groups(1), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+            softmax_rows_vec<Tin, Tout, 2, 64, 1, false><<<groups(1), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
         else
-            softmax_rows_vec<Tin, Tout, 4, 64, 1><<<groups(1), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+            softmax_rows_vec<Tin, Tout, 4, 64, 1, false><<<groups(1), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
     } else {
         softmax_rows_any<Tin, Tout><<<grid, 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
     }
