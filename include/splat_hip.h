@@ -267,6 +267,23 @@ int splat_compressed_transpose(const void* src, void* dst, const splat_acsr_seg*
                                const splat_acsr_seg* segs_t /* host */, int32_t n_seg, int64_t BH,
                                int32_t L, int32_t T, int32_t Lt, int32_t Tt, int32_t dtype, void* stream);
 
+/* The same backward pass in three launches of one kernel and without any compressed matrix in memory (no counterpart in
+ * the reference, which is forward only: r_attention.py:77-100).  q, k, v, out (the forward's output) and dout (the
+ * upstream gradient) are [B, H, L, d] views with unit stride along d (k is K itself, rows contiguous, not K^T);
+ * lse [B, H, L] is the row statistic of splat_attention_fwd_stats for the same inputs; delta [B, H, L] float32 is
+ * workspace (it receives rowsum(dout * out)); dq, dk, dv are contiguous [B, H, L, d].  segs / plan: the mask's ACSR and
+ * its splat_attention_plan; segs_t / plan_t: the same for the transposed mask (keys as rows).  16-bit dtypes, d = 64 or
+ * 128, scale > 0.  With P = exp(scale * q.k - lse) on the live columns:  dS = P * (dout.v - delta),
+ * dq = scale * dS k,  dk = scale * dS^T q,  dv = P^T dout. */
+int splat_attention_bwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* k, int64_t k_sb,
+                        int64_t k_sh, int64_t k_sl, const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sl,
+                        const void* out, int64_t o_sb, int64_t o_sh, int64_t o_sl, const void* dout, int64_t g_sb,
+                        int64_t g_sh, int64_t g_sl, const float* lse, float* delta, void* dq, void* dk, void* dv,
+                        const splat_acsr_seg* segs /* host */, int32_t n_seg, const void* plan, int64_t plan_bytes,
+                        const splat_acsr_seg* segs_t /* host */, int32_t n_seg_t, const void* plan_t,
+                        int64_t plan_t_bytes, int32_t B, int32_t H, int32_t L, int32_t d, float scale, int32_t dtype,
+                        void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -28,9 +28,13 @@ def _cases():
     ]
 
 
+@pytest.mark.parametrize("fused", [False, True], ids=["composed", "fused"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("case", _cases(), ids=lambda c: c[0])
-def test_gradients_against_dense_attention(dev, case, dtype):
+def test_gradients_against_dense_attention(dev, case, dtype, fused):
+    """Both backward passes (the operators composed over compressed matrices, and the fused kernel) against the oracle."""
+    if fused and dtype == torch.float32:
+        pytest.skip("the fused backward is built for 16-bit types; float32 takes the composed pass")
     _, make, dense, L = case
     B, H, d = 1, 2, 64
     scale = d ** -0.5
@@ -39,7 +43,7 @@ def test_gradients_against_dense_attention(dev, case, dtype):
     want = O.dense_masked_attention_grads(q, k.transpose(2, 3), v, np.asarray(dense()), scale, go)
     attn = RegularAttention(B, L, H, d, make(), 16, 16, dev, dtype, scale=scale)
     qd, kd, vd = [t.to(dev) for t in (q, k, v)]
-    got = attn.backward_pass([qd, kd.transpose(2, 3), vd], go.to(dev))
+    got = attn.backward_pass([qd, kd.transpose(2, 3), vd], go.to(dev), fused=fused)
     for name, g, w in zip(("dq", "dk", "dv"), got, want):
         assert float((g.float().cpu() - w).abs().max()) <= TOL[dtype], name
     # the same through autograd, K given as a contiguous [B, H, d, L] tensor underneath
@@ -78,12 +82,63 @@ def test_probabilities_in_one_pass_and_gradients_with_the_forward_statistic(dev,
     assert float((one.float() - two.float()).abs().max()) <= eps
     assert torch.equal(one == 5, two == 5)   # the sentinel survives in exactly the same (dead) slots
     want = O.dense_masked_attention_grads(q, k.transpose(2, 3), v, np.asarray(dense()), scale, go)
-    got = attn.backward_pass([qd, kT, vd], go.to(dev), lse)
+    got = attn.backward_pass([qd, kT, vd], go.to(dev), lse, fused=False)
     for name, g, w in zip(("dq", "dk", "dv"), got, want):
         assert float((g.float().cpu() - w).abs().max()) <= TOL[dtype], name
     with pytest.raises(Exception, match="lse"):
         rsddmm_launcher(qd, kT, one, None, None, None, None, T, None, None, None, None, 16, 16, scale=scale, segments=segs,
                         lse=lse[:, :1])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("name,make,dense,L", [
+    ("causal window over several row blocks and tiles", lambda: A.causal_windowed_pattern(700, 199), lambda: O.create_causal_windowed_mask(700, 199), 700),
+    ("two-sided window", lambda: A.windowed_pattern(513, 130), lambda: O.create_windowed_mask(513, 130), 513),
+    ("dilated, step 2", lambda: A.dilated_pattern(640, 96, 2), lambda: O.create_dilated_mask(640, 96, 2), 640),
+    ("blocked", lambda: A.blocked_pattern(512, 128), lambda: O.create_blocked_mask(512, 128), 512),
+    ("strided, two segments", lambda: A.strided_patterns(768, 64, 32), lambda: sum(O.create_strided_segment_masks(768, 64, 32)), 768),
+], ids=lambda x: x if isinstance(x, str) else None)
+def test_fused_backward(dev, name, make, dense, L, d, dtype):
+    """The fused backward kernel at both head dimensions over masks that need several row blocks, several tiles per block,
+    a last block that is not full and, for K, both memory layouts: against the oracle's dense gradients, and close to the
+    composed pass on the same inputs."""
+    B, H = 2, 2
+    scale = d ** -0.5
+    q, k, v = O.make_inputs(7 * L + d, B, H, L, d, dtype)
+    go = O.make_inputs(7 * L + d + 1, B, H, L, d, dtype)[0]
+    want = O.dense_masked_attention_grads(q, k.transpose(2, 3), v, np.asarray(dense()), scale, go)
+    attn = RegularAttention(B, L, H, d, make(), 16, 16, dev, dtype, scale=scale)
+    qd, kd, vd, god = [t.to(dev) for t in (q, k, v, go)]
+    out, lse = attn.forward_with_stats([qd, kd.transpose(2, 3), vd])
+    got = attn.backward_pass([qd, kd.transpose(2, 3), vd], god, lse.clone(), out.clone(), fused=True)
+    for nm, g, w in zip(("dq", "dk", "dv"), got, want):
+        assert torch.isfinite(g.float()).all(), nm
+        assert float((g.float().cpu() - w).abs().max()) <= TOL[dtype], nm
+    # K^T stored contiguously (the reference's layout) and no forward results handed in: the forward that backward_pass
+    # then runs walks dilated keys in another order, so its output and statistic may differ in their last bits
+    got2 = attn.backward_pass([qd, kd.transpose(2, 3).contiguous(), vd], god, fused=True)
+    for nm, a, b_ in zip(("dq", "dk", "dv"), got, got2):
+        assert float((a.float() - b_.float()).abs().max().cpu()) <= TOL[dtype] / 4, nm
+    composed = attn.backward_pass([qd, kd.transpose(2, 3), vd], god, lse, fused=False)
+    for nm, a, b_ in zip(("dq", "dk", "dv"), got, composed):
+        assert float((a.float() - b_.float()).abs().max().cpu()) <= 2 * TOL[dtype], nm
+
+
+def test_fused_backward_arguments_are_checked(dev):
+    from _splat_hip import SplatError
+    L, d = 128, 64
+    attn = RegularAttention(1, L, 1, d, A.causal_windowed_pattern(L, 15), 16, 16, dev, torch.float32, scale=0.125)
+    q = torch.zeros(1, 1, L, d, device=dev)
+    with pytest.raises(SplatError, match="16-bit"):
+        attn.backward_pass([q, q.transpose(2, 3), q], q, fused=True)
+    attn = RegularAttention(1, L, 1, d, A.causal_windowed_pattern(L, 15), 16, 16, dev, torch.bfloat16, scale=0.125)
+    qb = q.to(torch.bfloat16)
+    out, lse = attn.forward_with_stats([qb, qb.transpose(2, 3), qb])
+    with pytest.raises(SplatError, match="lse"):
+        attn.backward_pass([qb, qb.transpose(2, 3), qb], qb, lse[:, :, :-1], out, fused=True)
+    with pytest.raises(SplatError, match="out"):
+        attn.backward_pass([qb, qb.transpose(2, 3), qb], qb, lse, out[:, :, :-1], fused=True)
 
 
 def test_softmax_backward_on_compressed_rows(dev):

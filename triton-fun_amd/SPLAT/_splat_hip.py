@@ -71,6 +71,8 @@ _SIGNATURES = {
     "splat_attention_fwd_stats": (ctypes.c_int, [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64,
                                                  _vp, _i64, _i64, _i64, ctypes.POINTER(AcsrSeg), _i32, _i32, _i32, _i32,
                                                  _i32, _f32, _i32, _vp, _i64, _vp, _vp]),
+    "splat_attention_bwd": (ctypes.c_int, [_vp, _i64, _i64, _i64] * 5 + [_vp] * 5 +
+                            [ctypes.POINTER(AcsrSeg), _i32, _vp, _i64] * 2 + [_i32, _i32, _i32, _i32, _f32, _i32, _vp]),
 }
 EXPORTS = tuple(_SIGNATURES)
 

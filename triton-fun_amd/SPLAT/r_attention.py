@@ -160,6 +160,7 @@ class RegularAttention(nn.Module):
         self._unfused_ready = False
         self._plan = None  # the fused kernel's plan of this mask, built on the first fused forward
         self._segments_t = None  # ACSR of the transposed mask(s), built on the first backward
+        self._plan_t = None  # the fused backward's plan of the transposed mask
         self._lse = None  # the rows' softmax statistics, allocated by the first forward_with_stats
         self._BLOCK_HEIGHT = BLOCK_SIZE_Y
 
@@ -240,16 +241,35 @@ class RegularAttention(nn.Module):
         attention_launcher(q, k, v, self.rspmm_output, self.segments, self.scale, self._plan, self._lse)
         return self.rspmm_output, self._lse
 
-    def backward_pass(self, x, grad_out: torch.Tensor, lse: torch.Tensor | None = None):
+    def backward_pass(self, x, grad_out: torch.Tensor, lse: torch.Tensor | None = None, out: torch.Tensor | None = None,
+                      fused: bool | None = None):
         """Gradients (dq, dk, dv), each [B, H, L, d], of ``forward(x)`` for x = [q, kT, v] and the upstream gradient
-        ``grad_out`` [B, H, L, d].  The ACSR of the transposed mask is built on first use; see ``r_backward``.  ``lse``:
-        the rows' statistic of ``forward_with_stats`` for the same x, which spares the backward its softmax pass."""
-        from r_backward import attention_backward, transposed_segments
+        ``grad_out`` [B, H, L, d].  The ACSR of the transposed mask is built on first use; see ``r_backward``.  ``lse``
+        and ``out``: the rows' statistic and the output of ``forward_with_stats`` for the same x.  Where the fused
+        forward applies (16-bit dtype, d in {64, 128}) the gradients come from the fused backward kernel, which needs both
+        (a forward is run here when one is missing); otherwise, or with ``fused=False``, from the operators composed over
+        compressed matrices, which ``lse`` spares the softmax pass."""
+        from r_backward import attention_backward, attention_backward_fused, transposed_segments
         q, kT, v = x
         if self._segments_t is None:
             masks = self._mask if _is_segment_list(self._mask) else [self._mask]
             self._segments_t = transposed_segments(masks, self._BLOCK_HEIGHT, self._GPU_ID)
-        return attention_backward(q, kT, v, grad_out, self.segments, self._segments_t, self.scale, lse)
+        fusable = (self.fused and q.shape[-1] in (64, 128) and q.dtype in (torch.float16, torch.bfloat16) and
+                   q.dtype == kT.dtype == v.dtype == grad_out.dtype == self._out_dtype)
+        if fused is None:
+            fused = fusable
+        elif fused and not fusable:
+            raise _hip.SplatError("the fused backward needs a 16-bit dtype shared by all tensors and d in {64, 128}")
+        if not fused:
+            return attention_backward(q, kT, v, grad_out, self.segments, self._segments_t, self.scale, lse)
+        if lse is None or out is None:
+            out, lse = self.forward_with_stats(x)
+        if self._plan is None:
+            self._plan = attention_plan(self.segments, self._shape[2], self._device)
+        if self._plan_t is None:
+            self._plan_t = attention_plan(self._segments_t, self._shape[2], self._device)
+        return attention_backward_fused(q, kT, v, out, grad_out, lse, self.segments, self._segments_t, self._plan,
+                                        self._plan_t, self.scale)
 
 
 class _AttentionFunction(torch.autograd.Function):
@@ -258,16 +278,18 @@ class _AttentionFunction(torch.autograd.Function):
         ctx.attn = attn
         if attn.fused and q.shape[-1] in (64, 128) and q.dtype == k.dtype == v.dtype == attn._out_dtype:
             out, lse = attn.forward_with_stats([q, k.transpose(2, 3), v])
-            ctx.save_for_backward(q, k, v, lse.clone())
-        else:
-            out = attn([q, k.transpose(2, 3), v])
-            ctx.save_for_backward(q, k, v)
-        return out.clone()  # the module's buffers are reused by the next call
+            out = out.clone()  # the module's buffers are reused by the next call
+            ctx.save_for_backward(q, k, v, lse.clone(), out)
+            return out
+        out = attn([q, k.transpose(2, 3), v])
+        ctx.save_for_backward(q, k, v)
+        return out.clone()
 
     @staticmethod
     def backward(ctx, grad_out):
         q, k, v, *stat = ctx.saved_tensors
-        dq, dk, dv = ctx.attn.backward_pass([q, k.transpose(2, 3), v], grad_out, stat[0] if stat else None)
+        dq, dk, dv = ctx.attn.backward_pass([q, k.transpose(2, 3), v], grad_out, stat[0] if stat else None,
+                                            stat[1] if stat else None)
         return dq, dk, dv, None
 
 

@@ -158,3 +158,45 @@ def attention_backward(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor, grad_
     dk = torch.empty((B, H, L, d), dtype=dt, device=dev)
     rspmm_t_launcher(dprobs, q if q.stride(3) == 1 else q.contiguous(), dk, segments, segments_t)
     return dq, dk, dv
+
+
+def attention_backward_fused(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor, out: torch.Tensor, grad_out: torch.Tensor,
+                             lse: torch.Tensor, segments: ACSRSegments, segments_t: ACSRSegments, plan: torch.Tensor,
+                             plan_t: torch.Tensor, scale: float = 1.0):
+    """(dq, dk, dv) as ``attention_backward`` gives them, from three launches of one kernel and without a compressed
+    matrix: ``out`` and ``lse`` are the output and the row statistic of the fused forward for the same inputs
+    (``RegularAttention.forward_with_stats``), ``plan`` / ``plan_t`` the fused kernel's plans (``attention_plan``) of the
+    mask's segments and of the transposed mask's.  16-bit dtypes, d in {64, 128}; operands whose rows are not contiguous
+    16-byte pieces (K^T-contiguous keys among them) are copied first."""
+    B, H, L, d = q.shape
+    dt, dev = q.dtype, q.device
+    if dt not in (torch.float16, torch.bfloat16) or d not in (64, 128):
+        raise _hip.SplatError("the fused backward takes fp16 / bf16 tensors with d in {64, 128}")
+    k = kT.transpose(2, 3)
+
+    def rows(t, name):
+        _hip.require_device_tensor(t, name)
+        if t.dtype != dt or tuple(t.shape) != (B, H, L, d):
+            raise _hip.SplatError(f"{name} must be a {dt} tensor of shape {(B, H, L, d)}, got {t.dtype} {tuple(t.shape)}")
+        if t.stride(3) != 1 or t.data_ptr() % 16 != 0 or any(t.stride(i) % 8 != 0 for i in (0, 1, 2)):
+            t = t.contiguous()
+        return t
+    q, k, v, out, grad_out = rows(q, "q"), rows(k, "k"), rows(v, "v"), rows(out, "out"), rows(grad_out, "grad_out")
+    _hip.require_device_tensor(lse, "lse")
+    if lse.dtype != torch.float32 or tuple(lse.shape) != (B, H, L) or not lse.is_contiguous():
+        raise _hip.SplatError(f"lse must be a contiguous float32 tensor of shape {(B, H, L)}")
+    delta = torch.empty((B, H, L), dtype=torch.float32, device=dev)
+    dq, dk, dv = (torch.empty((B, H, L, d), dtype=dt, device=dev) for _ in range(3))
+    arr = _hip.seg_array(segments.seg_args(), L)
+    arr_t = _hip.seg_array(segments_t.seg_args(), L)
+    args = []
+    for t in (q, k, v, out, grad_out):
+        args += [t.data_ptr(), t.stride(0), t.stride(1), t.stride(2)]
+    args += [lse.data_ptr(), delta.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+             arr, len(segments), plan.data_ptr(), plan.numel() * plan.element_size(),
+             arr_t, len(segments_t), plan_t.data_ptr(), plan_t.numel() * plan_t.element_size(),
+             B, H, L, d, float(scale), _hip.dtype_code(dt)]
+    with torch.cuda.device(dev):
+        rc = _hip.lib().splat_attention_bwd(*args, _hip.stream_ptr(dev))
+    _hip.check(rc, "splat_attention_bwd")
+    return dq, dk, dv

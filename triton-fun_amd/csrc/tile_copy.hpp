@@ -40,12 +40,21 @@ template <int ROWB>
 __device__ __forceinline__ constexpr int swz64(int row) {
     return ROWB >= 256 ? (row & 3) : ((row >> 1) & 1);
 }
+// Swizzle for tiles that are read both ways: the 64-byte block index is rotated as for the transposing read, and the
+// chunk inside the block by the next two row bits, so that the 16 rows a row-wise 16-byte read touches at once land on
+// 16 different chunk positions of the 256-byte bank space (rows 16 apart share their pattern; rows 8 apart differ in
+// the second bit of the chunk position).  The map is its own inverse.
+template <int ROWB>
+__device__ __forceinline__ constexpr int dual_chunk(int row, int c) {
+    return (((c >> 2) ^ swz64<ROWB>(row)) << 2) | ((c & 3) ^ ((row >> 2) & 3));
+}
 // logical 16-byte chunk held at physical chunk position pc of `row`; MODE 0: none, 1: chunk XOR (b128 row reads),
-// 2: 64-byte block XOR (transposing reads)
+// 2: 64-byte block XOR (transposing reads), 3: both kinds of read (dual_chunk)
 template <int ROWB, int MODE>
 __device__ __forceinline__ int logical_chunk(int row, int pc) {
     if constexpr (MODE == 1) return pc ^ swz<ROWB>(row);
     if constexpr (MODE == 2) return (((pc >> 2) ^ swz64<ROWB>(row)) << 2) | (pc & 3);
+    if constexpr (MODE == 3) return dual_chunk<ROWB>(row, pc);
     return pc;
 }
 
@@ -76,6 +85,13 @@ __device__ __forceinline__ void dma16_uniform(const void* base, uint32_t lane_of
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
                  : "s"(lds_address(lds_block)), "v"(lane_off), "s"(base)
+                 : "memory", "m0");
+}
+// One wavefront-wide 256-byte copy: lane i's 4 bytes from its own address land at lds_block + 4*i.
+__device__ __forceinline__ void dma4(const void* src, char* lds_block) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
+                 :
+                 : "s"(lds_address(lds_block)), "v"(src)
                  : "memory", "m0");
 }
 __device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
