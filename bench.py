@@ -417,16 +417,25 @@ def main() -> int:
                                   "hbm_frac": round(byt3 / ms / 1e6 / HBM_PEAK_GBPS, 4)}
         del s3, p3
         del s_buf, p_buf, o_buf, flush
-        # backward pass (not in the reference) at the same shape: nonzero FLOPs = 2.5 x the forward's (five products)
+        # backward pass (not in the reference) at the same shape: nonzero FLOPs = 2.5 x the forward's (five products).  The
+        # fused kernel takes the forward's output and row statistic; the composed pass (operators over compressed matrices)
+        # is timed with and without the statistic.
         attn4 = RegularAttention(B4, L4, H4, d4, pat4, 16, 16, dev, dtype, scale=d4 ** -0.5)
         g4 = torch.randn_like(q4)
-        _, pr = time_launches(lambda: attn4.backward_pass([q4, k4T, v4], g4), 10, 3)
-        ms = sum(pr) / len(pr)
-        extras["backward_cfg4"] = {"ms": round(ms, 3), "tflops_nnz": round(10 * d4 * nnz4 * B4 * H4 / ms / 1e9, 2)}
-        _, lse4 = attn4.forward_with_stats([q4, k4T, v4])
-        _, pr = time_launches(lambda: attn4.backward_pass([q4, k4T, v4], g4, lse4), 10, 3)
-        ms = sum(pr) / len(pr)
-        extras["backward_cfg4_with_forward_lse"] = {"ms": round(ms, 3), "tflops_nnz": round(10 * d4 * nnz4 * B4 * H4 / ms / 1e9, 2)}
+        x4 = [q4, k4T, v4]
+        out4, lse4 = attn4.forward_with_stats(x4)
+        out4, lse4 = out4.clone(), lse4.clone()
+        fl4 = 10 * d4 * nnz4 * B4 * H4
+        ms_f = min(time_batch(lambda: attn4.backward_pass(x4, g4, lse4, out4, fused=True), 10, 3) for _ in range(3))
+        _, pr = time_launches(lambda: attn4.backward_pass(x4, g4, lse4, fused=False), 10, 3)
+        ms_c = sum(pr) / len(pr)
+        _, pr = time_launches(lambda: attn4.backward_pass(x4, g4, fused=False), 10, 3)
+        ms_c0 = sum(pr) / len(pr)
+        extras["backward_cfg4"] = {"ms": round(ms_f, 4), "tflops_nnz": round(fl4 / ms_f / 1e9, 2),
+                                   "x_fused_forward": round(ms_f / extras["fused_cfg4"]["ms"], 2),
+                                   "kernel": "splat_attention_bwd: row sums + three launches of attn_bwd_kernel, no compressed matrix",
+                                   "composed_ms_with_forward_lse": round(ms_c, 3), "composed_ms": round(ms_c0, 3)}
+        del out4, lse4
         del attn4, g4, q4, k4, v4
     out["extras"] = extras
 

@@ -437,22 +437,25 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_kernel(const BwdParams p) {
     }
 }
 
-// D[bh, r] = sum over d of dO[b, h, r, :] * O[b, h, r, :]; one wavefront per row
-template <typename T>
+// D[bh, r] = sum over d of dO[b, h, r, :] * O[b, h, r, :]; d / 8 lanes per row, 16 bytes per lane and operand
+template <typename T, int D>
 __global__ __launch_bounds__(256) void attn_bwd_delta_kernel(const T* dout, int64_t g_sb, int64_t g_sh, int64_t g_sl, const T* out,
                                                              int64_t o_sb, int64_t o_sh, int64_t o_sl, float* delta, int H, int L,
-                                                             int d, int64_t n_rows) {
-    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= n_rows) return;
-    const int lane = threadIdx.x & 63;
+                                                             int64_t n_rows) {
+    constexpr int LPR = D / 8;  // lanes per row
+    const int sub = threadIdx.x % LPR;
+    const int64_t row_raw = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPR;
+    const int64_t row = row_raw < n_rows ? row_raw : n_rows - 1;  // surplus lanes shadow the last row and store nothing
     const int r = (int)(row % L);
     const int bh = (int)(row / L);
-    const T* gr = dout + (bh / H) * g_sb + (bh % H) * g_sh + (int64_t)r * g_sl;
-    const T* orow = out + (bh / H) * o_sb + (bh % H) * o_sh + (int64_t)r * o_sl;
+    const Frag<T> gv = global_frag<T>(dout + (bh / H) * g_sb + (bh % H) * g_sh + (int64_t)r * g_sl + 8 * sub);
+    const Frag<T> ov = global_frag<T>(out + (bh / H) * o_sb + (bh % H) * o_sh + (int64_t)r * o_sl + 8 * sub);
     float s = 0.f;
-    for (int c = lane * 2; c < d; c += 128) s += (float)gr[c] * (float)orow[c] + (float)gr[c + 1] * (float)orow[c + 1];
-    s = wave_sum(s);
-    if (lane == 0) delta[row] = s;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s += (float)gv.v[e] * (float)ov.v[e];
+#pragma unroll
+    for (int o = LPR / 2; o > 0; o >>= 1) s += __shfl_xor(s, o);
+    if (sub == 0 && row_raw < n_rows) delta[row] = s;
 }
 
 template <typename T, int D, int MODE>
@@ -518,11 +521,15 @@ extern "C" int splat_attention_bwd(const void* q, int64_t q_sb, int64_t q_sh, in
     {
         begin_launch();
         const int64_t n_rows = (int64_t)B * H * L;
-        const unsigned grid = (unsigned)((n_rows + 3) / 4);
-        if (dtype == SPLAT_F16)
-            attn_bwd_delta_kernel<f16><<<grid, 256, 0, st>>>((const f16*)dout, g_sb, g_sh, g_sl, (const f16*)out, o_sb, o_sh, o_sl, delta, H, L, d, n_rows);
-        else
-            attn_bwd_delta_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)dout, g_sb, g_sh, g_sl, (const bf16*)out, o_sb, o_sh, o_sl, delta, H, L, d, n_rows);
+        const unsigned grid = (unsigned)((n_rows * (d / 8) + 255) / 256);
+        auto run = [&](auto tag) {
+            typedef decltype(tag) E;
+            if (d == 64)
+                attn_bwd_delta_kernel<E, 64><<<grid, 256, 0, st>>>((const E*)dout, g_sb, g_sh, g_sl, (const E*)out, o_sb, o_sh, o_sl, delta, H, L, n_rows);
+            else
+                attn_bwd_delta_kernel<E, 128><<<grid, 256, 0, st>>>((const E*)dout, g_sb, g_sh, g_sl, (const E*)out, o_sb, o_sh, o_sl, delta, H, L, n_rows);
+        };
+        if (dtype == SPLAT_F16) run(f16{}); else run(bf16{});
         if (int rc = check_launch(who)) return rc;
     }
 
