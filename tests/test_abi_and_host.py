@@ -76,6 +76,28 @@ def test_the_allocation_free_forward_rejects_what_its_built_in_buffer_cannot_hol
     assert int(eval(re.search(r"#define SPLAT_STATIC_PLAN_BYTES \((.*?)\)", header).group(1))) == hip.STATIC_PLAN_BYTES
 
 
+def test_the_fused_backward_checks_its_arguments_on_the_host():
+    """splat_attention_bwd refuses what its kernel is not built for before anything is launched."""
+    lib = hip.lib()
+    seg = (hip.AcsrSeg * 1)()
+    seg[0].sTod_lin = seg[0].sTod_trans = seg[0].nnz = 16
+    seg[0].row_stride_hint = 1
+    L, d = 256, 64
+    need = lib.splat_attention_plan_bytes(seg, 1, L)
+
+    def bwd(q=16, lse=16, d=d, dtype=2, scale=1.0, plan_bytes=need, q_sl=d, seg_t=seg):
+        t = [16, 0, 0, d]  # pointer, batch / head / row strides
+        return lib.splat_attention_bwd(q, 0, 0, q_sl, *t, *t, *t, *t, lse, 16, 16, 16, 16, seg, 1, 16, plan_bytes,
+                                       seg_t, 1, 16, need, 1, 1, L, d, scale, dtype, None)
+    assert bwd(q=None) == -1 and bwd(lse=None) == -1 and bwd(seg_t=None) == -1
+    assert bwd(d=96) == -5 and b"64 or 128" in lib.splat_last_error()
+    assert bwd(dtype=0) == -5 and b"16-bit" in lib.splat_last_error()
+    assert bwd(scale=0.0) == -5
+    assert bwd(q=24) == -4 and bwd(q_sl=d + 4) == -4
+    assert bwd(q_sl=32) == -2
+    assert bwd(plan_bytes=need - 16) == -2 and b"plan" in lib.splat_last_error()
+
+
 def test_plan_size_is_host_arithmetic():
     lib = hip.lib()
     seg = (hip.AcsrSeg * 2)()
