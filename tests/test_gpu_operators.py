@@ -324,6 +324,45 @@ def test_spmm_patterns(dev, dtype, make, n_out):
     assert float((out.float().cpu() - want).abs().max()) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n_out", [64, 128])
+@pytest.mark.parametrize("make", [
+    lambda: [A.causal_windowed_pattern(700, 199)], lambda: [A.windowed_pattern(513, 130)], lambda: [A.dilated_pattern(640, 96, 2)],
+    lambda: [A.blocked_pattern(512, 128)], lambda: A.strided_patterns(768, 64, 32), lambda: [A.causal_windowed_pattern(100, 5)]],
+    ids=["causal window", "window", "dilated", "blocked", "strided, two segments", "rows shorter than a piece"])
+def test_spmm_16_bit_whole_rows_of_v(dev, make, n_out, dtype):
+    """16-bit operands with 64 or 128 output columns (one workgroup takes whole rows of V): several row blocks and tiles,
+    a last block that is not full, spans that end inside tiles, gathered keys, two segments, rows with fewer live slots than
+    one 16-byte piece; dead slots hold NaN and must not reach the output."""
+    pats = make()
+    L = pats[0].s
+    segs = A.create_acsr_segments(pats, 16, dev)
+    dms = [np.asarray(pt.device_mask(dev).cpu()) for pt in pats]
+    T = segs.T
+    g = torch.Generator().manual_seed(T + n_out)
+    lv = torch.cat([torch.from_numpy(O.slot_columns(O.create_acsr(m, 16))[1]) for m in dms], dim=-1)
+    pr = torch.rand(2, 2, L, T, generator=g)
+    pr = (pr / torch.where(lv, pr, torch.zeros(())).sum(-1, keepdim=True).clamp(min=1e-9)).to(dtype)
+    pr = torch.where(lv, pr, torch.full((), float("nan"), dtype=dtype))
+    v = torch.randn(2, 2, L, n_out, generator=g).to(dtype)
+    dense = torch.zeros(2, 2, L, L)
+    off = 0
+    for m in dms:
+        acsr_np = O.create_acsr(m, 16)
+        cols, valid = O.slot_columns(acsr_np, first_col=O.row_extents(m)[0])
+        Tk = cols.shape[-1]
+        blk = torch.nan_to_num(pr[..., off:off + Tk].float())
+        rows_i, slots_i = np.nonzero(valid)
+        dense[:, :, torch.from_numpy(rows_i), torch.from_numpy(cols[rows_i, slots_i].astype(np.int64))] += blk[:, :, torch.from_numpy(rows_i), torch.from_numpy(slots_i)]
+        off += Tk
+    want = dense @ v.float()
+    out = torch.full((2, 2, L, n_out), 7.0, dtype=dtype, device=dev)
+    r_spmm.rspmm_launcher(pr.to(dev), v.to(dev), out, None, None, None, None, None, None, T, None, None, 16, 16, segments=segs)
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    assert float((got - want).abs().max()) <= TOL[dtype]
+
+
 def test_comparison_sweeps_run_and_agree_with_dense(dev):
     """The sweep harness (successor of the reference's comparison.py:76-106) at toy size: one record per doubling of
     the sparsity parameter, nnz as the pattern's closed form, fused forward equal to dense attention with the same mask."""
