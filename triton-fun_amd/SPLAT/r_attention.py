@@ -264,10 +264,13 @@ class RegularAttention(nn.Module):
             return attention_backward(q, kT, v, grad_out, self.segments, self._segments_t, self.scale, lse)
         if lse is None or out is None:
             out, lse = self.forward_with_stats(x)
-        if self._plan is None:
-            self._plan = attention_plan(self.segments, self._shape[2], self._device)
-        if self._plan_t is None:
-            self._plan_t = attention_plan(self._segments_t, self._shape[2], self._device)
+        if self._plan is None or self._plan_t is None:
+            if self._plan is None:
+                self._plan = attention_plan(self.segments, self._shape[2], self._device)
+            if self._plan_t is None:
+                self._plan_t = attention_plan(self._segments_t, self._shape[2], self._device)
+            # once, so that later calls may run on any stream without ordering themselves after the plan kernels
+            torch.cuda.current_stream(self._device).synchronize()
         return attention_backward_fused(q, kT, v, out, grad_out, lse, self.segments, self._segments_t, self._plan,
                                         self._plan_t, self.scale)
 
