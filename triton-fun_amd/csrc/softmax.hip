@@ -113,31 +113,60 @@ __global__ __launch_bounds__(256) void softmax_rows_vec(const Tin* __restrict__ 
         float v[NCH][8];
         uint32_t live[NCH];
         float mx = kNegBig;
+        bool whole = true;  // every chunk of this lane is live in all 8 slots
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             const int ch = lane + LPR * c;
             live[c] = (ch < nchunk[i]) ? lr.live8((ch << 3) - shift[i]) : 0u;
-            if (live[c]) {
+            whole = whole && live[c] == 0xffu;
+        }
+        // the common case, decided for the whole wavefront: no dead slot anywhere in its rows, so no per-slot selects
+        const bool all_whole = !__any(!whole);
+        float sum = 0.f;
+        if (all_whole) {
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) {
                 const vin t = raw[i][c];
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    v[c][e] = ((live[c] >> e) & 1u) ? (float)t[e] : kNegBig;
+                    v[c][e] = (float)t[e];
                     mx = fmaxf(mx, v[c][e]);
                 }
             }
-        }
 #pragma unroll
-        for (int o = LPR / 2; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
-        const float mb = mx * kLog2e;
-        float sum = 0.f;
+            for (int o = LPR / 2; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+            const float mb = mx * kLog2e;
 #pragma unroll
-        for (int c = 0; c < NCH; ++c) {
-            if (live[c]) {
+            for (int c = 0; c < NCH; ++c)
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    float p = ((live[c] >> e) & 1u) ? fast_exp2(fmaf(v[c][e], kLog2e, -mb)) : 0.f;
-                    v[c][e] = p;
-                    sum += p;
+                    v[c][e] = fast_exp2(fmaf(v[c][e], kLog2e, -mb));
+                    sum += v[c][e];
+                }
+        } else {
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) {
+                if (live[c]) {
+                    const vin t = raw[i][c];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        v[c][e] = ((live[c] >> e) & 1u) ? (float)t[e] : kNegBig;
+                        mx = fmaxf(mx, v[c][e]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int o = LPR / 2; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+            const float mb = mx * kLog2e;
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) {
+                if (live[c]) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        float p = ((live[c] >> e) & 1u) ? fast_exp2(fmaf(v[c][e], kLog2e, -mb)) : 0.f;
+                        v[c][e] = p;
+                        sum += p;
+                    }
                 }
             }
         }
