@@ -417,3 +417,43 @@ def test_scores_that_outrun_the_first_tiles_reference(dev, dtype, slope):
         got = run_module(mask, 1, 2, L, d, dtype, dev, q, k, v, 1.0, True)
         assert torch.isfinite(got).all(), w
         assert float((got - want).abs().max()) <= TOL[dtype], w
+
+
+@pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 128), (torch.float16, 64)])
+def test_forward_and_backward_replay_from_a_captured_graph(dev, dtype, d):
+    """The entry points neither allocate nor synchronise, so a caller may record them into a HIP graph: the fused forward
+    (its plan built beforehand) and the fused backward are captured once and replayed on new inputs, with eager work and
+    synchronisations between the replays, and every replay must equal the eager result on the same inputs."""
+    from r_backward import attention_backward_fused
+    B, H, L = 2, 2, 520
+    scale = d ** -0.5
+    attn = RegularAttention(B, L, H, d, A.causal_windowed_pattern(L, 150), 16, 16, dev, dtype, scale=scale)
+    g = torch.Generator().manual_seed(11)
+    q, k, v, go = [torch.randn(B, H, L, d, generator=g).to(dtype).to(dev) for _ in range(4)]
+    x = [q, k.transpose(2, 3), v]
+    out, lse = attn.forward_with_stats(x)                     # builds the plan and the statistics buffer
+    attn.backward_pass(x, go, lse.clone(), out.clone())       # builds the transposed mask's ACSR and plan
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            o_g, lse_g = attn.forward_with_stats(x)
+            grads_g = attention_backward_fused(q, x[1], v, o_g, go, lse_g, attn.segments, attn._segments_t, attn._plan,
+                                               attn._plan_t, scale)
+    torch.cuda.current_stream(dev).wait_stream(side)
+    for seed in (1, 2, 3):
+        gen = torch.Generator().manual_seed(seed)
+        for t in (q, k, v, go):
+            t.copy_(torch.randn(B, H, L, d, generator=gen).to(dtype))
+        graph.replay()
+        torch.cuda.synchronize()
+        got_o, got_lse, got_g = o_g.clone(), lse_g.clone(), [t.clone() for t in grads_g]
+        want_o, want_lse = attn.forward_with_stats(x)          # eager, same buffers as the captured forward writes
+        want_o, want_lse = want_o.clone(), want_lse.clone()
+        want_g = attn.backward_pass(x, go, want_lse, want_o)
+        torch.cuda.synchronize()
+        assert torch.equal(got_o, want_o) and torch.equal(got_lse, want_lse), seed
+        for a, b_ in zip(got_g, want_g):
+            assert torch.equal(a, b_), seed
