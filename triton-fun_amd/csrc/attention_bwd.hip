@@ -285,6 +285,77 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_kernel(const BwdParams p) {
         if (!skip) {
             const bool full = (j0 >= w_lo_max) && (j0 + BN <= w_hi_min);
             const uint64_t live = full ? ~0ull : row_live_bits(win, j0, first, pat);
+            if constexpr (!THREE) {
+                // ---- dV: two products only, so the whole 64-position tile fits the registers at once, as in the forward:
+                // all score MFMAs with the fragments requested well ahead, then the exponentials, then the output MFMAs ----
+                constexpr int NMMA = 2 * KS, AHEAD = NMMA < 12 ? NMMA : 12;
+                f32x16 s2[2];
+#pragma unroll
+                for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) s2[nt][j] = 0.f;
+                Frag<T> xfr[NMMA];
+                auto load_x = [&](int i) {
+                    Frag<T> f;
+                    f.v = __builtin_bit_cast(typename Frag<T>::vec, lds_load128(xr_addr[i % KS] + 32 * (i / KS) * ROWB));
+                    return f;
+                };
+#pragma unroll
+                for (int i = 0; i < AHEAD; ++i) xfr[i] = load_x(i);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < NMMA; ++i) {
+                    mma32(s2[i / KS], xfr[i], af[i % KS]);
+                    if (i + AHEAD < NMMA) {
+                        xfr[i + AHEAD] = load_x(i + AHEAD);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    if (i < NDMA) {
+                        if (spread) issue_step(i, stage_pf);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+                Frag<T> pf2[2][2];
+#pragma unroll
+                for (int nt = 0; nt < 2; ++nt) {
+                    if (!full) {
+                        const uint32_t bits = (uint32_t)(live >> (32 * nt)) >> (4 * g);
+#pragma unroll
+                        for (int j = 0; j < 16; ++j) {
+                            const int c = 8 * (j >> 2) + (j & 3);
+                            s2[nt][j] = keep_or_mask(s2[nt][j], ((int)(bits << (31 - c))) >> 31);
+                        }
+                    }
+#pragma unroll
+                    for (int k4 = 0; k4 < 4; ++k4) {
+                        const f32x4 lse4 = __builtin_bit_cast(f32x4, lds_load128(st_addr + (32 * nt + 8 * k4) * 4));
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const int j = 4 * k4 + i;
+                            pf2[nt][j >> 3].v[j & 7] = (T)fast_exp2(fmaf(s2[nt][j], c2, -1.4426950408889634f * lse4[i]));
+                        }
+                    }
+                }
+                auto load_t = [&](int step, int dt) {
+                    const int roff = 16 * step * ROWB;
+                    return frag_from_tr<T>(lds_load_tr16(tr_addr[dt] + roff), lds_load_tr16(tr_addr8[dt] + roff));
+                };
+                Frag<T> tf2[2][DT];
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) tf2[0][dt] = load_t(0, dt);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int step = 0; step < 4; ++step) {
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) {
+                        mma32(acc[dt], tf2[step & 1][dt], pf2[step >> 1][step & 1]);
+                        if (step + 1 < 4) {
+                            tf2[(step + 1) & 1][dt] = load_t(step + 1, dt);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
+                }
+            } else
 #pragma unroll
             for (int nt = 0; nt < 2; ++nt) {
                 // ---- S^T (32 positions x 32 rows) = X rows . A^T ----
