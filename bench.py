@@ -441,6 +441,16 @@ def main() -> int:
                                    "composed_ms_with_forward_lse": round(ms_c, 3), "composed_ms": round(ms_c0, 3)}
         del out4, lse4
         del attn4, g4, q4, k4, v4
+        # the fused backward at the headline shape (config 5), from the forward's output and row statistic
+        g5 = torch.randn_like(qd)
+        x5 = [qd, kT_view, vd]
+        out5, lse5 = attn.forward_with_stats(x5)
+        out5, lse5 = out5.clone(), lse5.clone()
+        attn.backward_pass(x5, g5, lse5, out5, fused=True)  # builds the transposed mask's ACSR and plan
+        ms_b5 = min(time_batch(lambda: attn.backward_pass(x5, g5, lse5, out5, fused=True), 10, 3) for _ in range(3))
+        extras["backward_cfg5"] = {"ms": round(ms_b5, 4), "tflops_nnz": round(2.5 * flops / ms_b5 / 1e9, 2),
+                                   "x_fused_forward": round(ms_b5 / kern_ms, 2)}
+        del g5, out5, lse5
     out["extras"] = extras
 
     if not args.no_cpu:
