@@ -125,6 +125,34 @@ def test_fused_backward(dev, name, make, dense, L, d, dtype):
         assert float((a.float() - b_.float()).abs().max().cpu()) <= 2 * TOL[dtype], nm
 
 
+@pytest.mark.parametrize("d,dtype", [(64, torch.float16), (128, torch.bfloat16)])
+def test_fused_backward_on_views_in_token_major_layout(dev, d, dtype):
+    """q, k, v, the forward's output and the upstream gradient stored as [B, L, H, d] and handed over as [B, H, L, d]
+    views (batch, head and row strides all differ from the contiguous ones; nothing is copied on the way in): the same
+    bits as from contiguous tensors, on a mask with a ragged last block."""
+    B, H, L = 2, 3, 333
+    scale = d ** -0.5
+    q, k, v = O.make_inputs(31 + d, B, H, L, d, dtype)
+    go = O.make_inputs(32 + d, B, H, L, d, dtype)[0]
+    attn = RegularAttention(B, L, H, d, A.windowed_pattern(L, 70), 16, 16, dev, dtype, scale=scale)
+    cont = [t.to(dev) for t in (q, k, v, go)]
+
+    def token_major(t):
+        return t.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    views = [token_major(t) for t in cont]
+    assert all(t.stride(1) == d and t.stride(2) == H * d and not t.is_contiguous() for t in views)
+    out_c, lse_c = attn.forward_with_stats([cont[0], cont[1].transpose(2, 3), cont[2]])
+    out_c, lse_c = out_c.clone(), lse_c.clone()
+    want = attn.backward_pass([cont[0], cont[1].transpose(2, 3), cont[2]], cont[3], lse_c, out_c, fused=True)
+    want = [t.clone() for t in want]
+    got = attn.backward_pass([views[0], views[1].transpose(2, 3), views[2]], views[3], lse_c, token_major(out_c), fused=True)
+    for nm, a, b_ in zip(("dq", "dk", "dv"), got, want):
+        assert torch.equal(a, b_), nm
+    dense = O.dense_masked_attention_grads(q, k.transpose(2, 3), v, np.asarray(O.create_windowed_mask(L, 70)), scale, go)
+    for nm, g, w in zip(("dq", "dk", "dv"), got, dense):
+        assert float((g.float().cpu() - w).abs().max()) <= TOL[dtype], nm
+
+
 def test_fused_backward_arguments_are_checked(dev):
     from _splat_hip import SplatError
     L, d = 128, 64
