@@ -273,3 +273,49 @@ def test_backward_of_a_long_sequence_by_properties(dev):
     col_sums = dv.float().sum(dim=2)  # [1, 1, d]
     assert float((col_sums / L - 1.0).abs().max()) <= 2e-3
     assert torch.isfinite(dv.float()).all()
+
+
+def test_fused_backward_at_the_headline_shape_by_properties(dev):
+    """The fused backward at the largest benchmark configuration (bf16, B=4, H=16, L=16384, d=128, causal window 512),
+    where no dense reference fits: the pass is linear in the upstream gradient and scaling by 2 is exact in binary
+    floating point, so doubling dO must double every gradient bit for bit; and the gradients of a few query rows (dq)
+    and key rows (dk, dv) of one head are recomputed from their windows in fp32."""
+    B, H, L, d, w = 4, 16, 16384, 128, 512
+    dtype, scale = torch.bfloat16, 128 ** -0.5
+    g = torch.Generator(device=dev).manual_seed(50)
+    q, k, v, go = (torch.randn(B, H, L, d, generator=g, device=dev, dtype=torch.float32).to(dtype) for _ in range(4))
+    attn = RegularAttention(B, L, H, d, A.causal_windowed_pattern(L, w - 1), 16, 16, dev, dtype, scale=scale)
+    out, lse = attn.forward_with_stats([q, k.transpose(2, 3), v])
+    out, lse = out.clone(), lse.clone()
+    dq, dk, dv = [t.clone() for t in attn.backward_pass([q, k.transpose(2, 3), v], go, lse, out, fused=True)]
+    dq2, dk2, dv2 = attn.backward_pass([q, k.transpose(2, 3), v], go * 2, lse, out, fused=True)
+    for nm, a, b_ in (("dq", dq, dq2), ("dk", dk, dk2), ("dv", dv, dv2)):
+        assert torch.isfinite(a.float()).all(), nm
+        assert torch.equal(a * 2, b_), nm
+
+    b, h = 3, 11
+    qf, kf, vf, gf = (t[b, h].float() for t in (q, k, v, go))
+
+    def rows_of_p(i0, i1):
+        """P[i0:i1, :] restricted to the key range the rows can see, with that range's first key."""
+        j0 = max(0, i0 - w + 1)
+        s = (qf[i0:i1] @ kf[j0:i1].T) * scale
+        ii = torch.arange(i0, i1, device=dev)[:, None]
+        jj = torch.arange(j0, i1, device=dev)[None, :]
+        s = torch.where((jj <= ii) & (jj > ii - w), s, torch.full_like(s, float("-inf")))
+        return torch.softmax(s, dim=-1), j0
+
+    def ds_of(i0, i1):
+        p, j0 = rows_of_p(i0, i1)
+        dp = gf[i0:i1] @ vf[j0:i1].T
+        return p, p * (dp - (p * dp).sum(-1, keepdim=True)) * scale, j0
+
+    tol = TOL[dtype]
+    for i0 in (0, 700, 8191, L - 64):      # 64 query rows each
+        p, ds, j0 = ds_of(i0, i0 + 64)
+        assert float((dq[b, h, i0:i0 + 64].float() - ds @ kf[j0:i0 + 64]).abs().max()) <= tol, i0
+    for j in (0, 300, 9000, L - 3):        # one key row each: its queries are j .. j + w - 1
+        i1 = min(L, j + w)
+        p, ds, j0 = ds_of(j, i1)
+        assert float((dk[b, h, j].float() - ds[:, j - j0] @ qf[j:i1]).abs().max()) <= tol, j
+        assert float((dv[b, h, j].float() - p[:, j - j0] @ gf[j:i1]).abs().max()) <= tol, j
