@@ -390,6 +390,27 @@ __global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
                         if (ri == 0) *reinterpret_cast<v4*>(ring_row + R_SLOTS * 2) = t;
                     }
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wavefront's LDS writes are visible to its own reads
+                // A tile that lies inside the span of every row of the wavefront adds 64 slots to each of them, so every
+                // row completes exactly one line, and completes it: no tests, no branches (the tests below cost several
+                // times the tile's MFMAs in scalar and branch instructions).  A row that ends with this tile may have a
+                // last, shorter line to store as well: that tile takes the tests.
+                if (__builtin_amdgcn_readfirstlane((full && j0 + kBN < span.hi_min) ? 1 : 0)) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const int s0 = 64 * f_done[c] + 8 * (lane & 7);
+                        const int rix = (s0 + (f_lo[c] & 3)) & (R_SLOTS - 1);
+                        v8 val;
+                        __builtin_memcpy(&val, stg + (8 * c + (lane >> 3)) * R_ROW + rix * 2, 16);
+                        TO* const dst = (TO*)p.out + f_base[c] + s0;
+                        if (p.out_vec) {
+                            __builtin_nontemporal_store(val, reinterpret_cast<v8*>(dst));
+                        } else {
+                            __builtin_memcpy(dst, &val, 16);
+                        }
+                        f_done[c] += 1;
+                    }
+                    return;
+                }
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     const int u_end = j0 + kBN - f_lo[c];
