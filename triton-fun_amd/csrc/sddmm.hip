@@ -80,12 +80,14 @@ __device__ __forceinline__ void store_piece(TO* row_out, const RowWin& w, int jj
 // KSU: 0 = the contraction is longer than one LDS chunk (Q fragments are re-read per chunk); otherwise Q stays in
 // registers, and KSU > 0 says at compile time how many MFMA steps hold data (-1: known at run time only).
 template <typename T, bool KT, int KSU, bool PROBS>
-__global__ __launch_bounds__(256, 2) void sddmm_kernel(const SddmmParams p) {
+__global__ __launch_bounds__(256, (KSU > 0 && KSU * 16 < SddmmGeom<T>::DC && !KT) ? 3 : 2) void sddmm_kernel(const SddmmParams p) {
     constexpr bool QREG = KSU != 0;
     constexpr int ES = sizeof(T);
     constexpr int BM = 128;
     constexpr int NT = kBN / 32;
-    constexpr int DC = SddmmGeom<T>::DC;
+    // one LDS chunk holds the whole contraction when its length is known to be shorter (d = 64 in a 16-bit type: half
+    // the K tile, half the Q registers, and a third workgroup per CU)
+    constexpr int DC = (KSU > 0 && !KT) ? KSU * 16 : SddmmGeom<T>::DC;
     constexpr int KSC = DC / 16;                                  // MFMA steps per chunk
     constexpr int K_ROW = KT ? (kBN * ES + 64) : (DC * ES + 16);  // bytes per LDS row
     constexpr int K_ROWS = KT ? DC : kBN;
