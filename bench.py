@@ -320,6 +320,9 @@ def main() -> int:
                             "pct_mfma_peak": round(100 * fl / ms / 1e9 / peak, 2),
                             "hbm_floor_ms": round(byt / HBM_PEAK_GBPS / 1e6, 4),
                             "pct_of_hbm_floor_rate": round(100 * byt / HBM_PEAK_GBPS / 1e6 / ms, 2)}
+            # the reference's own layout of K: [B, H, d, L] contiguous (rows that step over columns cost a transpose of K)
+            kTc = kTc.contiguous()
+            extras[name]["ms_kT_contiguous"] = round(min(time_batch(run, 60, 60) for _ in range(2)), 4)
             del at, qc, kc, vc, kTc
         # the literal reference layout: K^T contiguous [B, H, d, L]
         kT_c = kT_view.contiguous()

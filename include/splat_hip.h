@@ -224,6 +224,14 @@ int splat_attention_fwd_noalloc(const void* q, int64_t q_sb, int64_t q_sh, int64
                                 int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t d, float scale,
                                 int32_t dtype, void* stream);
 
+/* K^T [B, H, d, L] with unit stride along the keys (the layout the reference documents for `y`, r_sddmm.py:230-231) to
+ * K [B, H, L, d] contiguous.  No counterpart in the reference, whose kernels only read the former: the kernels here read
+ * that layout in dense runs of keys, so for rows that step over columns (dilated windows, strided far fields) the
+ * Python launchers transpose K once per call with this and pass the result as a [B, H, d, L] view (unit stride along d).
+ * kT_sb / kT_sh / kT_sd: element strides of batch, head and the d index (kT_sd >= L); k_rows 16-byte aligned. */
+int splat_transpose_keys(const void* kT, int64_t kT_sb, int64_t kT_sh, int64_t kT_sd, void* k_rows, int32_t B,
+                         int32_t H, int32_t L, int32_t d, int32_t dtype, void* stream);
+
 /* Measurement aid, no counterpart in the reference: copy `bytes` (a multiple of 16; both pointers 16-byte aligned) from
  * src to dst with the access forms of the HBM-bound kernels here (16 bytes per lane, non-temporal, several requests
  * in flight).  Its rate is the read + write streaming ceiling that bench.py quotes splat_softmax against. */

@@ -98,6 +98,18 @@ def test_the_fused_backward_checks_its_arguments_on_the_host():
     assert bwd(plan_bytes=need - 16) == -2 and b"plan" in lib.splat_last_error()
 
 
+def test_the_key_transpose_checks_its_arguments_on_the_host():
+    lib = hip.lib()
+
+    def tr(src=16, dst=16, L=100, d=64, sd=100, dtype=2):
+        return lib.splat_transpose_keys(src, 0, 0, sd, dst, 1, 1, L, d, dtype, None)
+    assert tr(src=None) == -1 and tr(dst=None) == -1
+    assert tr(L=0) == -2 and tr(d=0) == -2
+    assert tr(sd=99) == -2 and b"stride" in lib.splat_last_error()
+    assert tr(dtype=7) == -3
+    assert tr(dst=24) == -4 and tr(src=17) == -4
+
+
 def test_plan_size_is_host_arithmetic():
     lib = hip.lib()
     seg = (hip.AcsrSeg * 2)()

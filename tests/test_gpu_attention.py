@@ -196,6 +196,36 @@ def test_fused_views_that_are_not_piece_aligned(dev):
     assert float((ov.float().cpu() - want).abs().max()) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("name,make", [
+    ("dilated, step 2", lambda: [A.dilated_pattern(640, 96, 2)]),
+    ("strided far field", lambda: A.strided_patterns(768, 64, 32)),
+    ("dense mask with stepping rows", lambda: [O.create_dilated_mask(300, 40, 3)]),
+])
+def test_gathered_rows_with_the_reference_layout_of_k(dev, name, make):
+    """K^T stored contiguously along the keys (the reference's layout) and rows that step over columns: the launchers
+    hand the kernels a row-major copy of K, so the results are those of row-major K bit for bit, for the fused forward
+    and for rsddmm_launcher; a mask without stepping rows leaves the tensor as it is."""
+    from r_sddmm import rsddmm_launcher
+    pats = make()
+    L = A.mask_shape(pats[0])[0]
+    B, H, d, dtype = 2, 2, 64, torch.bfloat16
+    q, k, v = [t.to(dev) for t in O.make_inputs(11, B, H, L, d, dtype)]
+    segs = A.create_acsr_segments(pats, 16, dev)
+    assert segs.gathered
+    kT_rows, kT_cont = k.transpose(2, 3), k.transpose(2, 3).contiguous()
+    assert segs.keys_as_rows(kT_cont).stride(2) == 1 and segs.keys_as_rows(kT_rows) is kT_rows
+    outs = []
+    for kT in (kT_rows, kT_cont):
+        o = torch.empty(B, H, L, d, dtype=dtype, device=dev)
+        attention_launcher(q, kT, v, o, segs, d ** -0.5)
+        s = torch.full((B, H, L, segs.T), 3.0, dtype=dtype, device=dev)
+        rsddmm_launcher(q, kT, s, None, None, None, None, segs.T, None, None, None, None, 16, 16, scale=d ** -0.5, segments=segs)
+        outs.append((o, s))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    plain = A.create_acsr_segments([A.causal_windowed_pattern(L, 31)], 16, dev)
+    assert not plain.gathered and plain.keys_as_rows(kT_cont) is kT_cont
+
+
 def test_empty_and_single_column_rows(dev):
     L, d = 256, 64
     mask = O.create_causal_windowed_mask(L, 31).copy()

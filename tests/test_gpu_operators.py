@@ -432,3 +432,17 @@ def test_mfma_lds_probe_runs_and_checks_its_arguments(dev):
     assert hip.lib().splat_mfma_lds_probe(data.data_ptr(), 65536, out.data_ptr(), wgs * 256 * 4 - 1, wgs, tiles, None) == -2
     assert hip.lib().splat_mfma_lds_probe(data.data_ptr(), 65536, out.data_ptr(), wgs * 256 * 4, 0, tiles, None) == -2
     assert hip.lib().splat_mfma_lds_probe(data.data_ptr() + 2, 65536, out.data_ptr(), wgs * 256 * 4, wgs, tiles, None) == -4
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("L,d", [(64, 64), (1000, 128), (333, 64), (77, 40), (130, 7), (1, 128)])
+def test_key_transpose(dev, L, d, dtype):
+    """K^T with the keys contiguous -> K with rows contiguous, bit for bit: whole tensors, a slice of a wider one (longer
+    stride of the d index), and a source that starts off a 16-byte boundary (element loads)."""
+    B, H = 2, 3
+    g = torch.Generator().manual_seed(L * 131 + d)
+    wide = torch.randn(B, H, d, L + 24, generator=g).to(dtype).to(dev)
+    for kT in (wide[..., :L].contiguous(), wide[..., 8:8 + L], wide[..., 3:3 + L]):
+        got = A.transpose_keys(kT)
+        assert got.is_contiguous() and tuple(got.shape) == (B, H, L, d)
+        assert torch.equal(got, kT.transpose(2, 3).contiguous())

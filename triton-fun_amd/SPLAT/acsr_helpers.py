@@ -235,7 +235,7 @@ def mask_shape(mask) -> tuple[int, int]:
 class AcsrBuild:
     """Everything one ``splat_acsr_build`` call produced for (mask, BLOCK_HEIGHT)."""
     __slots__ = ("dTos_lin", "dTos_trans", "sTod_lin", "sTod_trans", "nnz", "T", "span_start", "span_end",
-                 "row_first", "row_last", "row_stride")
+                 "row_first", "row_last", "row_stride", "max_step")
 
 
 def build_acsr(mask, BLOCK_HEIGHT: int, dev: torch.device) -> AcsrBuild:
@@ -270,6 +270,8 @@ def build_acsr(mask, BLOCK_HEIGHT: int, dev: torch.device) -> AcsrBuild:
     b.T = int(found[0])
     # rows whose columns step by n and start in phase with the row index (dilated windows): kernels group them by phase
     b.row_stride = int(found[2]) if (int(found[2]) == int(found[3]) and int(found[3]) > 1 and int(found[4]) == 0) else 1
+    # the largest column step of any row: above 1 some rows are gathered (dilated windows, strided far fields)
+    b.max_step = int(found[3])
     entry.builds[BLOCK_HEIGHT] = b
     return b
 
@@ -292,7 +294,7 @@ def create_acsr(mask, BLOCK_HEIGHT: int, GPU_ID: Any):
     The returned ``sTod_translations`` tensor carries an attribute ``splat_first_col`` (int32 tensor, first
     live column per row) that the launchers pick up: rows with a single live column store translation 0
     whatever that column is, so the column itself has to travel separately.  ``splat_row_stride`` (int) is a speed
-    hint for patterns whose rows alternate column phase."""
+    hint for patterns whose rows alternate column phase, ``splat_max_step`` (int) the largest column step of any row."""
     dev = _hip.resolve_device(GPU_ID)
     b = build_acsr(mask, BLOCK_HEIGHT, dev)
     # every caller gets tensors of its own, as from the reference's create_acsr: a build shared through the cache must
@@ -300,7 +302,24 @@ def create_acsr(mask, BLOCK_HEIGHT: int, GPU_ID: Any):
     arrays = [t.clone() for t in (b.dTos_lin, b.dTos_trans, b.sTod_lin, b.sTod_trans, b.nnz, b.span_start, b.span_end)]
     arrays[3].splat_first_col = b.row_first.clone()
     arrays[3].splat_row_stride = b.row_stride
+    arrays[3].splat_max_step = b.max_step
     return (arrays[0], arrays[1], arrays[2], arrays[3], arrays[4], b.T, arrays[5], arrays[6])
+
+
+def transpose_keys(kT: torch.Tensor) -> torch.Tensor:
+    """K [B, H, L, d] (contiguous, new) from K^T [B, H, d, L] with unit stride along the keys: one streaming kernel."""
+    _hip.require_device_tensor(kT, "kT")
+    if kT.dim() != 4 or kT.stride(3) != 1:
+        raise _hip.SplatError("kT must be [B, H, d, L] with unit stride along the keys")
+    B, H, d, L = kT.shape
+    out = torch.empty((B, H, L, d), dtype=kT.dtype, device=kT.device)
+    if out.numel() == 0:
+        return out
+    with torch.cuda.device(kT.device):
+        rc = _hip.lib().splat_transpose_keys(kT.data_ptr(), kT.stride(0), kT.stride(1), kT.stride(2), out.data_ptr(), B, H, L, d,
+                                             _hip.dtype_code(kT.dtype), _hip.stream_ptr(kT.device))
+    _hip.check(rc, "splat_transpose_keys")
+    return out
 
 
 class ACSRSegments:
@@ -322,6 +341,27 @@ class ACSRSegments:
 
     def __len__(self) -> int:
         return len(self.tuples)
+
+    @property
+    def max_step(self) -> int:
+        """The largest column step of any row of any segment (1 when unknown: metadata not built by ``create_acsr``)."""
+        return max(int(getattr(t[3], "splat_max_step", 1)) for t in self.tuples)
+
+    @property
+    def gathered(self) -> bool:
+        """Some row of some segment steps over columns."""
+        return self.max_step > 1
+
+    def keys_as_rows(self, kT: torch.Tensor, min_step: int = 2) -> torch.Tensor:
+        """``kT`` ([B, H, d, L]) as the kernels should get it.  The reference stores K^T contiguously along the keys;
+        the kernels read that layout in dense runs of keys, which for gathered rows (every second key of a dilated
+        window, every 128th of a strided far field) means walking, and masking, all the keys in between.  With rows
+        of K contiguous they fetch only the keys a tile needs, so for masks whose rows step by ``min_step`` columns or
+        more K is transposed once per call (its bytes read and written once) and handed on as a [B, H, d, L] view of
+        the [B, H, L, d] copy."""
+        if self.max_step >= min_step and kT.dim() == 4 and kT.stride(3) == 1 and kT.stride(2) != 1:
+            return transpose_keys(kT).transpose(2, 3)
+        return kT
 
     def seg_args(self) -> list[tuple]:
         return [(t[0], t[1], t[2], t[3], t[4], fc, off) for t, fc, off in zip(self.tuples, self.first_cols, self.offsets)]

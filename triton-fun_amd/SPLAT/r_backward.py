@@ -23,7 +23,7 @@ import numpy as np
 import torch
 
 import _splat_hip as _hip
-from acsr_helpers import ACSRSegments, MaskPattern, create_acsr_segments
+from acsr_helpers import ACSRSegments, MaskPattern, create_acsr_segments, transpose_keys
 from r_sddmm import rsddmm_launcher
 from r_softmax import rsoftmax_launcher
 from r_spmm import rspmm_launcher
@@ -172,7 +172,8 @@ def attention_backward_fused(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor,
     dt, dev = q.dtype, q.device
     if dt not in (torch.float16, torch.bfloat16) or d not in (64, 128):
         raise _hip.SplatError("the fused backward takes fp16 / bf16 tensors with d in {64, 128}")
-    k = kT.transpose(2, 3)
+    # K^T with the keys contiguous (the reference's layout): one streaming transpose instead of a strided copy
+    k = transpose_keys(kT) if (kT.dim() == 4 and kT.stride(3) == 1 and kT.stride(2) != 1) else kT.transpose(2, 3)
 
     def rows(t, name):
         _hip.require_device_tensor(t, name)

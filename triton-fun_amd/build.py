@@ -13,7 +13,7 @@ OBJ = os.path.join(HERE, "build")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIB_DIR, "libsplat_hip.so")
 
-SOURCES = ["api_common.cpp", "acsr_build.hip", "softmax.hip", "sddmm.hip", "spmm.hip", "attention.hip", "backward.hip", "attention_bwd.hip", "mfma_probe.hip"]
+SOURCES = ["api_common.cpp", "acsr_build.hip", "softmax.hip", "sddmm.hip", "spmm.hip", "attention.hip", "backward.hip", "attention_bwd.hip", "mfma_probe.hip", "transpose.hip"]
 # packed fp32 VALU forms are switched off for every device compile
 FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function", "-Wno-inline-asm",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
