@@ -19,7 +19,7 @@ import torch.nn as nn
 
 import _splat_hip as _hip
 from acsr_helpers import (ACSRSegments, MaskPattern, create_acsr, create_acsr_segments, create_blocked_mask,  # noqa: F401
-                          create_causal_windowed_mask, create_windowed_mask, mask_shape)
+                          create_causal_windowed_mask, create_windowed_mask, mask_shape, transpose_keys)
 from r_sddmm import rsddmm_launcher, rsddmm_preamble
 from r_softmax import rsoftmax_launcher, rsoftmax_preamble
 from r_spmm import rspmm_launcher, rspmm_preamble
@@ -84,7 +84,7 @@ def attention_launcher(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor, outpu
         pass  # K^T contiguous along the keys, the reference's layout, in whole 16-byte pieces
     else:
         # e.g. the reference's contiguous [B, H, d, L] with L not a multiple of the piece: rows of K made contiguous
-        kT = kT.transpose(2, 3).contiguous().transpose(2, 3)
+        kT = (transpose_keys(kT) if kT.stride(3) == 1 else kT.transpose(2, 3).contiguous()).transpose(2, 3)
     target = output
     if not piecewise(output, (0, 1, 2)):
         output = torch.empty((B, H, L, d), dtype=target.dtype, device=target.device)
