@@ -18,7 +18,7 @@ import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-for _p in (ROOT, os.path.join(ROOT, "triton-fun_amd", "SPLAT")):
+for _p in (ROOT, os.path.join(ROOT, "triton-fun_amd", "SPLAT"), os.path.join(ROOT, "triton-fun_amd")):
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
@@ -275,20 +275,27 @@ def main() -> int:
         probe_data = torch.randn(32768, dtype=torch.float32).to(dtype).to(dev)
         if args.zero_operands:
             probe_data.zero_()
-        probe_wgs, probe_tiles = B * H * (L // 128), 40
-        probe_out = torch.empty(probe_wgs * 256, dtype=torch.float32, device=dev)
-        probe = lambda: hip.check(hip.lib().splat_mfma_lds_probe(probe_data.data_ptr(), probe_data.numel() * 2, probe_out.data_ptr(),
-                                                                 probe_out.numel() * 4, probe_wgs, probe_tiles, hip.stream_ptr(dev)),
-                                  "splat_mfma_lds_probe")
-        settle(probe)
-        probe_ms = min(time_batch(probe, 20, 5) for _ in range(3))
-        probe_tflops = probe_wgs * probe_tiles * 4 * 32 * 32768 / (probe_ms * 1e-3) / 1e12
-        out["roofline"]["mfma_lds_loop"] = {
-            "tflops": round(probe_tflops, 1), "frac_of_peak": round(probe_tflops / MFMA_PEAK_TFLOPS, 4),
-            "fused_frac_of_loop": round(kern_tflops / probe_tflops, 4), "sustained": sample_power_and_clock(probe, 10),
-            "note": "splat_mfma_lds_probe: the fused kernel's LDS reads and MFMAs per tile and nothing else, N(0,1) bf16 "
-                    "operands, same grid; its MFMAs are all counted, the fused figure counts nonzero FLOPs only"}
-        del probe_data, probe_out
+        import bench_probes as BP
+        probe_tiles = 40
+        loops = {}
+        for shape, label in BP.PROBE_SHAPES.items():
+            probe_wgs = B * H * (L // (256 if shape == 1 else 128))
+            probe_out = torch.empty(probe_wgs * BP.PROBE_THREADS[shape], dtype=torch.float32, device=dev)
+            probe = lambda s=shape, w=probe_wgs, o=probe_out: BP.check(BP.lib().splat_bench_mfma_lds_probe(
+                probe_data.data_ptr(), probe_data.numel() * 2, o.data_ptr(), o.numel() * 4, s, w, probe_tiles, hip.stream_ptr(dev)),
+                "splat_bench_mfma_lds_probe")
+            settle(probe)
+            probe_ms = min(time_batch(probe, 20, 5) for _ in range(3))
+            probe_tflops = BP.lib().splat_bench_mfma_lds_probe_flops(shape, probe_wgs, probe_tiles) / (probe_ms * 1e-3) / 1e12
+            loops[shape] = {"shape": label, "tflops": round(probe_tflops, 1), "frac_of_peak": round(probe_tflops / MFMA_PEAK_TFLOPS, 4),
+                            "sustained": sample_power_and_clock(probe, 10)}
+            del probe_out
+        out["roofline"]["mfma_lds_loop"] = dict(
+            loops[0], fused_frac_of_loop=round(kern_tflops / loops[0]["tflops"], 4),
+            note="splat_bench_mfma_lds_probe shape 0: the fused kernel's LDS reads and MFMAs per tile and nothing else, N(0,1) "
+                 "bf16 operands, same grid; its MFMAs are all counted, the fused figure counts nonzero FLOPs only",
+            other_shapes=[loops[1], loops[2]])
+        del probe_data
 
     extras = {}
     if args.calibrate_copy:
@@ -404,8 +411,9 @@ def main() -> int:
         # the read + write streaming ceiling: a plain 1 GiB copy by a kernel of this library with the softmax's access forms
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
-        copy = lambda: hip.check(hip.lib().splat_stream_copy(src.data_ptr(), dst.data_ptr(), src.numel(), hip.stream_ptr(dev)),
-                                 "splat_stream_copy")
+        import bench_probes as BP
+        copy = lambda: BP.check(BP.lib().splat_bench_stream_copy(src.data_ptr(), dst.data_ptr(), src.numel(), hip.stream_ptr(dev)),
+                                "splat_bench_stream_copy")
         ms = min(time_batch(copy, 10, 3) for _ in range(3))
         extras["stream_copy_1GiB"] = {"ms": round(ms, 4), "gbps_read_plus_write": round(2 * src.numel() / ms / 1e6, 1)}
         # both sides timed the same way: back-to-back launches

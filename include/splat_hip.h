@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define SPLAT_VERSION 500 /* major*10000 + minor*100 + patch; 0.2.0 added the planned forward, 0.3.0 splat_spmm_t, 0.4.0 splat_attention_fwd_stats, splat_sddmm_probs, 0.5.0 splat_attention_fwd_noalloc */
+#define SPLAT_VERSION 600 /* major*10000 + minor*100 + patch; 0.2.0 added the planned forward, 0.3.0 splat_spmm_t, 0.4.0 splat_attention_fwd_stats, splat_sddmm_probs, 0.5.0 splat_attention_fwd_noalloc, 0.6.0 moved the two measurement aids out (libsplat_bench.so, splat_bench.h) */
 
 /* element types of q/k/v/score/output buffers */
 #define SPLAT_F32 0
@@ -215,7 +215,10 @@ int splat_attention_fwd_stats(const void* q, int64_t q_sb, int64_t q_sh, int64_t
  * holds one until the process ends), then the forward runs from it on the same stream.  The call allocates and frees
  * nothing.  Masks whose plan is larger (splat_attention_plan_bytes; 4256 bytes per 128-row block and segment) are
  * rejected with SPLAT_E_SHAPE.  All calls on one GPU share that one buffer: two calls whose work may overlap on a
- * GPU (different streams, different threads) race; order them. */
+ * GPU (different streams, different threads) race; order them.  The first call on a GPU for a given element type, head
+ * size and K layout also looks up the buffer's address and raises its kernel's LDS limit, which are not stream
+ * operations: make that call outside any stream capture (one eager warm-up call per configuration is enough; every
+ * later call only enqueues two kernels and can be captured, and a replay rebuilds the plan it runs from). */
 #define SPLAT_STATIC_PLAN_BYTES (4 << 20)
 int splat_attention_fwd_noalloc(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT,
                                 int64_t k_sb, int64_t k_sh, int64_t k_sd, int64_t k_sl, const void* v,
@@ -231,21 +234,6 @@ int splat_attention_fwd_noalloc(const void* q, int64_t q_sb, int64_t q_sh, int64
  * kT_sb / kT_sh / kT_sd: element strides of batch, head and the d index (kT_sd >= L); k_rows 16-byte aligned. */
 int splat_transpose_keys(const void* kT, int64_t kT_sb, int64_t kT_sh, int64_t kT_sd, void* k_rows, int32_t B,
                          int32_t H, int32_t L, int32_t d, int32_t dtype, void* stream);
-
-/* Measurement aid, no counterpart in the reference: copy `bytes` (a multiple of 16; both pointers 16-byte aligned) from
- * src to dst with the access forms of the HBM-bound kernels here (16 bytes per lane, non-temporal, several requests
- * in flight).  Its rate is the read + write streaming ceiling that bench.py quotes splat_softmax against. */
-int splat_stream_copy(const void* src, void* dst, int64_t bytes, void* stream);
-
-/* Measurement aid, no counterpart in the reference: `workgroups` workgroups of 256 threads each run `tiles` times the
- * LDS reads and MFMAs of one 64-key tile of the fused forward at d = 128 in bf16 (2 x 16 MFMAs of 32x32x16 per
- * wavefront and tile, i.e. workgroups * tiles * 4 * 32 * 32768 floating-point operations per call), with no global
- * loads, copies, exponentials or barriers in the loop.  The 64 KiB at `data` (16-byte aligned; give it random bf16
- * values: the switching activity of the operands decides the clock a power-limited part reaches) fill the LDS; `out`
- * receives one float per thread.  The rate of this loop is the matrix ceiling that bench.py quotes the fused forward
- * against, beside the rated peak. */
-int splat_mfma_lds_probe(const void* data, int64_t data_bytes, void* out, int64_t out_bytes, int32_t workgroups,
-                         int32_t tiles, void* stream);
 
 /* ---- backward pass (the reference has none: r_attention.py:77-100 is forward only) ----
  * With S~ the compressed scores, P~ = softmax(S~), O = P~ . V:

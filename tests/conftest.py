@@ -4,7 +4,7 @@ import sys
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-for p in (ROOT, os.path.join(ROOT, "triton-fun_amd", "SPLAT")):
+for p in (ROOT, os.path.join(ROOT, "triton-fun_amd", "SPLAT"), os.path.join(ROOT, "triton-fun_amd")):
     if p not in sys.path:
         sys.path.insert(0, p)
 

@@ -31,6 +31,23 @@ def test_library_exports_every_declared_symbol():
     assert sorted(hip.EXPORTS) == syms
 
 
+def test_the_measurement_library_exports_what_its_header_declares():
+    """libsplat_bench.so (bench.py's two ceilings) against include/splat_bench.h and its binding; and the operator header
+    declares none of it."""
+    import bench_probes as BP
+    text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "splat_bench.h")).read(), flags=re.S)
+    syms = sorted(set(re.findall(r"\b(splat_bench_[a-z_0-9]+)\s*\(", text)))
+    assert "splat_bench_stream_copy" in syms and "splat_bench_mfma_lds_probe" in syms
+    handle = ctypes.CDLL(BP.LIB_PATH)
+    for s in syms:
+        assert hasattr(handle, s), s
+    assert sorted(BP.EXPORTS) == syms
+    want = int(re.search(r"#define SPLAT_BENCH_VERSION (\d+)", open(os.path.join(ROOT, "include", "splat_bench.h")).read()).group(1))
+    assert BP.lib().splat_bench_version() == want
+    assert not [s for s in header_symbols() if "probe" in s or "stream_copy" in s or "bench" in s]
+    assert BP.lib().splat_bench_stream_copy(None, None, 16, None) == -1 and b"null" in BP.lib().splat_bench_last_error()
+
+
 def test_version_matches_header():
     want = int(re.search(r"#define SPLAT_VERSION (\d+)", open(HEADER).read()).group(1))
     assert hip.lib().splat_version() == want

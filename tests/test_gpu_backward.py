@@ -319,3 +319,56 @@ def test_fused_backward_at_the_headline_shape_by_properties(dev):
         p, ds, j0 = ds_of(j, i1)
         assert float((dk[b, h, j].float() - ds[:, j - j0] @ qf[j:i1]).abs().max()) <= tol, j
         assert float((dv[b, h, j].float() - p[:, j - j0] @ gf[j:i1]).abs().max()) <= tol, j
+
+
+def _dead_ends_mask(L=256, p=31):
+    """Causal window with the last row emptied (so the last key column is seen by no query) and the row before it cut
+    down to its diagonal entry (a single live column that is not column 0).  Both cuts take the last entries of the
+    columns they touch, so every column still meets an arithmetic progression of rows."""
+    mask = O.create_causal_windowed_mask(L, p).copy()
+    mask[L - 1] = 0
+    mask[L - 2, :L - 2] = 0
+    return mask
+
+
+@pytest.mark.parametrize("fused", [False, True], ids=["composed", "fused"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_gradients_with_an_empty_row_a_single_column_row_and_an_unseen_key(dev, dtype, fused):
+    """The forward gives an empty row out = 0 and lse = +inf; the backward recomputes exp(score - lse) from that and
+    must come out with zeros there, not NaN: the empty query row's dq, and dk / dv of the key nobody attends to."""
+    L, d, B, H = 256, 64, 1, 2
+    mask = _dead_ends_mask(L)
+    scale = d ** -0.5
+    q, k, v = O.make_inputs(77, B, H, L, d, dtype)
+    go = O.make_inputs(78, B, H, L, d, dtype)[0]
+    want = O.dense_masked_attention_grads_explicit(q, k.transpose(2, 3), v, mask, scale, go)
+    attn = RegularAttention(B, L, H, d, torch.from_numpy(mask), 16, 16, dev, dtype, scale=scale)
+    qd, kd, vd = [t.to(dev) for t in (q, k, v)]
+    got = attn.backward_pass([qd, kd.transpose(2, 3), vd], go.to(dev), fused=fused)
+    for name, g, w in zip(("dq", "dk", "dv"), got, want):
+        assert torch.isfinite(g.float()).all(), name
+        assert float((g.float().cpu() - w).abs().max()) <= TOL[dtype], name
+    dq, dk, dv = got
+    assert torch.all(dq[:, :, L - 1] == 0)
+    assert torch.all(dk[:, :, L - 1] == 0) and torch.all(dv[:, :, L - 1] == 0)
+
+
+def test_a_mask_whose_columns_are_not_affine_is_refused_by_the_backward(dev):
+    """Rows affine, columns not: the forward runs, the backward raises instead of handing out wrong dk / dv."""
+    from _splat_hip import SplatError
+    L, d = 256, 64
+    mask = O.create_causal_windowed_mask(L, 31).copy()
+    mask[100] = 0
+    mask[100, 40] = 1                      # column 40 now meets rows 40..71 and 100
+    attn = RegularAttention(1, L, 1, d, torch.from_numpy(mask), 16, 16, dev, torch.float16, scale=0.125)
+    q, k, v = [t.to(dev) for t in O.make_inputs(5, 1, 1, L, d, torch.float16)]
+    out = attn([q, k.transpose(2, 3), v]).float().cpu()
+    want = O.dense_masked_attention(q.cpu(), k.cpu().transpose(2, 3), v.cpu(), mask, 0.125)
+    assert float((out - want).abs().max()) <= 1e-2
+    with pytest.raises(SplatError, match="arithmetic progression"):
+        attn.backward_pass([q, k.transpose(2, 3), v], torch.ones_like(q))
+    with pytest.raises(SplatError, match="column 40"):
+        transposed_segments([torch.from_numpy(mask)], 16, dev)
+    # the same rows without the stray entry: accepted
+    ok = O.create_causal_windowed_mask(L, 31)
+    assert len(transposed_segments([torch.from_numpy(ok)], 16, dev)) == 1

@@ -396,42 +396,49 @@ def test_a_segment_that_is_empty_everywhere_is_dropped(dev):
 
 @pytest.mark.parametrize("n_bytes", [16, 4096 * 16, (4096 * 3 + 1000) * 16 + 48, 64 << 20])
 def test_stream_copy_copies(dev, n_bytes):
-    """splat_stream_copy, the streaming ceiling bench.py quotes the softmax against, is a faithful copy: whole chunks
-    and the tail that does not fill one, and nothing past the end."""
+    """splat_bench_stream_copy, the streaming ceiling bench.py quotes the softmax against, is a faithful copy: whole
+    chunks and the tail that does not fill one, and nothing past the end."""
     import _splat_hip as hip
+    import bench_probes as BP
     g = torch.Generator().manual_seed(n_bytes % 1000)
     src = torch.randint(0, 256, (n_bytes + 64,), dtype=torch.uint8, generator=g).to(dev)
     dst = torch.full((n_bytes + 64,), 7, dtype=torch.uint8, device=dev)
-    hip.check(hip.lib().splat_stream_copy(src.data_ptr(), dst.data_ptr(), n_bytes, hip.stream_ptr(dev)), "splat_stream_copy")
+    BP.check(BP.lib().splat_bench_stream_copy(src.data_ptr(), dst.data_ptr(), n_bytes, hip.stream_ptr(dev)), "splat_bench_stream_copy")
     assert torch.equal(dst[:n_bytes], src[:n_bytes])
     assert torch.all(dst[n_bytes:] == 7)
-    assert hip.lib().splat_stream_copy(src.data_ptr(), dst.data_ptr(), 24, None) == -2
-    assert hip.lib().splat_stream_copy(src.data_ptr() + 8, dst.data_ptr(), 32, None) == -4
+    assert BP.lib().splat_bench_stream_copy(src.data_ptr(), dst.data_ptr(), 24, None) == -2
+    assert BP.lib().splat_bench_stream_copy(src.data_ptr() + 8, dst.data_ptr(), 32, None) == -4
 
 
-def test_mfma_lds_probe_runs_and_checks_its_arguments(dev):
-    """splat_mfma_lds_probe, the matrix loop bench.py quotes the fused forward against: every workgroup computes the same
-    figures from the same 64 KiB, zeros give zeros, two calls agree, and short buffers are refused."""
+@pytest.mark.parametrize("shape", [0, 1, 2])
+def test_mfma_lds_probe_runs_and_checks_its_arguments(dev, shape):
+    """splat_bench_mfma_lds_probe, the matrix loops bench.py quotes the fused forward against: every workgroup computes
+    the same figures from the same 64 KiB, zeros give zeros, two calls agree, and short buffers are refused."""
     import _splat_hip as hip
+    import bench_probes as BP
     data = torch.randn(32768, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16).to(dev)
-    wgs, tiles = 6, 3
-    out = torch.full((wgs * 256 + 8,), 7.0, dtype=torch.float32, device=dev)
-    call = lambda d, o, w=wgs, t=tiles: hip.lib().splat_mfma_lds_probe(d.data_ptr(), d.numel() * 2, o.data_ptr(), wgs * 256 * 4, w, t,
-                                                                     hip.stream_ptr(dev))
-    hip.check(call(data, out), "splat_mfma_lds_probe")
-    res = out[:wgs * 256].view(wgs, 256)
+    wgs, tiles, nt = 6, 3, BP.PROBE_THREADS[shape]
+    out = torch.full((wgs * nt + 8,), 7.0, dtype=torch.float32, device=dev)
+    fn = BP.lib().splat_bench_mfma_lds_probe
+    call = lambda d, o, w=wgs, t=tiles: fn(d.data_ptr(), d.numel() * 2, o.data_ptr(), wgs * nt * 4, shape, w, t, hip.stream_ptr(dev))
+    BP.check(call(data, out), "splat_bench_mfma_lds_probe")
+    res = out[:wgs * nt].view(wgs, nt)
     assert torch.isfinite(res).all() and float(res.abs().max()) > 0
     assert torch.equal(res, res[0].expand_as(res))
-    assert torch.all(out[wgs * 256:] == 7.0)
+    assert torch.all(out[wgs * nt:] == 7.0)
     again = torch.empty_like(out)
-    hip.check(call(data, again), "splat_mfma_lds_probe")
-    assert torch.equal(again[:wgs * 256], out[:wgs * 256])
-    hip.check(call(torch.zeros_like(data), again), "splat_mfma_lds_probe")
-    assert torch.all(again[:wgs * 256] == 0)
-    assert hip.lib().splat_mfma_lds_probe(data.data_ptr(), 65535, out.data_ptr(), wgs * 256 * 4, wgs, tiles, None) == -2
-    assert hip.lib().splat_mfma_lds_probe(data.data_ptr(), 65536, out.data_ptr(), wgs * 256 * 4 - 1, wgs, tiles, None) == -2
-    assert hip.lib().splat_mfma_lds_probe(data.data_ptr(), 65536, out.data_ptr(), wgs * 256 * 4, 0, tiles, None) == -2
-    assert hip.lib().splat_mfma_lds_probe(data.data_ptr() + 2, 65536, out.data_ptr(), wgs * 256 * 4, wgs, tiles, None) == -4
+    BP.check(call(data, again), "splat_bench_mfma_lds_probe")
+    assert torch.equal(again[:wgs * nt], out[:wgs * nt])
+    BP.check(call(torch.zeros_like(data), again), "splat_bench_mfma_lds_probe")
+    assert torch.all(again[:wgs * nt] == 0)
+    assert fn(data.data_ptr(), 65535, out.data_ptr(), wgs * nt * 4, shape, wgs, tiles, None) == -2
+    assert fn(data.data_ptr(), 65536, out.data_ptr(), wgs * nt * 4 - 1, shape, wgs, tiles, None) == -2
+    assert fn(data.data_ptr(), 65536, out.data_ptr(), wgs * nt * 4, shape, 0, tiles, None) == -2
+    assert fn(data.data_ptr() + 2, 65536, out.data_ptr(), wgs * nt * 4, shape, wgs, tiles, None) == -4
+    assert fn(data.data_ptr(), 65536, out.data_ptr(), wgs * nt * 4, 3, wgs, tiles, None) == -5
+    rows = 256 if shape == 1 else 128
+    assert BP.lib().splat_bench_mfma_lds_probe_flops(shape, wgs, tiles) == wgs * tiles * rows * 64 * 128 * 4
+    assert BP.lib().splat_bench_mfma_lds_probe_flops(3, wgs, tiles) == 0
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])

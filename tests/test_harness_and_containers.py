@@ -22,6 +22,31 @@ def oracle_meta(mask, BH=16):
 
 
 # ------------------------------------------------------------------ checkers, on the host (plain tensor code)
+def test_is_correct_reads_the_first_column_attribute_before_it_slices():
+    """Rows with one live column that is not column 0 (a strided far field's first rows): the metadata stores
+    translation 0 for them (acsr_helpers.py:126-130), so the checkers need the builder's first-column array, which
+    lives as an attribute on the translations tensor and would be lost by the checkers' own ``[:rows]`` slices."""
+    far = O.create_strided_segment_masks(64, 8, 8)[1]          # row i: columns j <= i - 8 with j % 8 == 7
+    counts = far.sum(1)
+    assert (counts == 1).any() and far[counts == 1].argmax(1).min() > 0
+    acsr_np = O.create_acsr(far, 16)
+    first, _ = O.row_extents(far)
+    meta = oracle_meta(far)
+    meta[3].splat_first_col = torch.from_numpy(np.asarray(first)).int()
+    g = torch.Generator().manual_seed(5)
+    x = torch.randint(0, 100, (1, 2, 64, 64), generator=g).float()
+    y = torch.randint(0, 100, (1, 2, 64, 64), generator=g).float()
+    comp = O.sddmm(x, y, acsr_np, first_col=first)
+    assert r_sddmm.is_correct(r_sddmm.truth(x, y, "cpu"), comp, meta[2], meta[3], meta[4], 1, 2, far.tolist())
+    # without the attribute the single-column rows are looked up at column 0 and a correct result is rejected
+    bare = oracle_meta(far)
+    assert not r_sddmm.is_correct(r_sddmm.truth(x, y, "cpu"), comp, bare[2], bare[3], bare[4], 1, 2, far.tolist())
+    p = torch.rand(1, 2, 64, int(acsr_np[5]), generator=g)
+    out = O.spmm(p, y, acsr_np, first_col=first)
+    assert r_spmm.is_correct(p, y, out, meta[2], meta[3], meta[4], 2, 1, far.tolist())
+    assert not r_spmm.is_correct(p, y, out, bare[2], bare[3], bare[4], 2, 1, far.tolist())
+
+
 @pytest.mark.parametrize("make", [lambda: O.create_blocked_mask(10, 2), lambda: O.create_blocked_mask(32, 10),
                                   lambda: O.create_causal_windowed_mask(40, 7), lambda: O.create_dilated_mask(48, 8, 2)])
 def test_checkers_accept_the_oracle_and_reject_a_wrong_slot(make):
@@ -224,3 +249,59 @@ def test_the_modules_own_tests_at_the_reference_large_case(dev):
     assert r_sddmm.test(1024, 64, 1024, 2, 2, mask, 0, 16, 16, torch.float32)
     assert r_softmax.test(1024, 1024, 2, 2, mask, 0, 16, torch.float32)
     assert r_spmm.test(1024, 1024, 1024, 2, 2, mask, 0, 16, 16, torch.float32)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n,p", REF_SMALL + [(1024, 256)])
+def test_the_modules_own_tests_at_the_reference_dtype(dev, n, p, dtype, capsys):
+    """The reference's ``__main__`` blocks call ``test`` with ``out_dtype=torch.bfloat16`` (r_sddmm.py:262-410,
+    r_softmax.py:230-386, r_spmm.py:266-441).  What those calls print with the drop-in underneath:
+      * SDDMM: passed -- inputs and ``truth`` are in the 16-bit type too, and both sides round the exact integer sum (fp32
+        accumulation) to it the same way, so every live slot agrees bit for bit;
+      * softmax: passed -- a row of 16-bit probabilities sums to 1 well within the rule's 1e-2;
+      * SpMM: failed -- its inputs stay float32 and only the output is 16-bit, which cannot hold sums of products of
+        integers below 100 to within 1e-3 (fp16 overflows to inf); the rule says so of any correct 16-bit result.
+    The SpMM output is therefore also checked for what it should be: the exact sum, rounded once."""
+    mask = A.create_blocked_mask(n, p)
+    k = n if n < 1024 else 64
+    assert r_sddmm.test(n, k, n, 2, 2, mask, 0, 16, 16, dtype) is True
+    assert r_softmax.test(n, n, 2, 2, mask, 0, 16, dtype) is True
+    assert r_spmm.test(n, n, n, 2, 2, mask, 0, 16, 16, dtype) is False
+    out = capsys.readouterr().out
+    assert out.count("test case passed!") == 2 and out.count("test case failed") == 1
+    # the 16-bit SpMM output is the correctly rounded exact result
+    acsr = A.create_acsr(mask, 16, dev)
+    T = acsr[5]
+    g = torch.Generator().manual_seed(n * 31 + p)
+    left = torch.randint(0, 100, (2, 2, n, T), generator=g, dtype=torch.float32).to(dev)
+    right = torch.randint(0, 100, (2, 2, n, n), generator=g, dtype=torch.float32).to(dev)
+    got = torch.empty(2, 2, n, n, dtype=dtype, device=dev)
+    r_spmm.rspmm_launcher(left, right, got, acsr[0], acsr[1], acsr[2], acsr[3], acsr[6], acsr[7], T, acsr[4], (1, 1, 4), 16, 16)
+    want = O.spmm(left.cpu().double(), right.cpu().double(), tuple(x.cpu().numpy() if isinstance(x, torch.Tensor) else x for x in acsr))
+    assert torch.equal(got.cpu(), want.to(dtype))
+
+
+def test_rows_that_are_not_arithmetic_progressions_are_found_on_the_host():
+    """``non_affine_rows`` (the check behind the backward's refusal of masks whose transpose has no ACSR) on host tensors,
+    with the metadata the oracle gives: the closed-form patterns and their transposes have none, a row with a stray
+    column is named, and so is a row whose first, second and last column fit a progression that a middle column leaves."""
+    for mask in (O.create_blocked_mask(40, 8), O.create_causal_windowed_mask(48, 9), O.create_dilated_mask(48, 8, 3),
+                 sum(O.create_strided_segment_masks(64, 8, 8))[:, :], O.create_windowed_mask(33, 4)):
+        for m in (mask, np.ascontiguousarray(mask.T)):
+            if m is mask and m.shape[0] == 64:
+                continue   # the union of the two strided segments is not one progression per row; its parts are
+            acsr = O.create_acsr(m, 16)
+            first, _ = O.row_extents(m)
+            bad = A.non_affine_rows(torch.from_numpy(m.astype(np.uint8)), torch.from_numpy(np.asarray(first)),
+                                    torch.from_numpy(acsr[2]), torch.from_numpy(acsr[4]))
+            assert bad.numel() == 0
+    m = O.create_causal_windowed_mask(48, 9).copy()
+    m[30, 2] = 1                           # stray column in front of the window
+    m[40] = 0
+    m[40, [0, 2, 3, 6]] = 1                # first + step * (n - 1) = 6 is the last column, yet 3 is off the progression
+    acsr = O.create_acsr(m, 16)
+    first, _ = O.row_extents(m)
+    bad = A.non_affine_rows(torch.from_numpy(m.astype(np.uint8)), torch.from_numpy(np.asarray(first)),
+                            torch.from_numpy(acsr[2]), torch.from_numpy(acsr[4]))
+    assert bad.tolist() == [30, 40]

@@ -58,3 +58,46 @@ def test_noalloc_forward_rejects_a_plan_beyond_its_buffer(dev):
     assert rc == -2
     with pytest.raises(hip.SplatError, match="built-in buffer"):
         hip.check(rc, "splat_attention_fwd_noalloc")
+
+
+def test_noalloc_forward_replays_from_a_captured_graph_after_another_mask_used_the_buffer(dev):
+    """Captured after one eager warm-up call (the first call on a device resolves the built-in buffer's address, which is
+    not a stream operation).  Between capture and replays an eager call with another mask overwrites the shared plan
+    buffer; a replay rebuilds its own plan first, so every replay must equal the planned forward on the same inputs."""
+    B, H, L, d, dtype = 2, 2, 520, 128, torch.bfloat16
+    segs = A.create_acsr_segments([A.causal_windowed_pattern(L, 150)], 16, dev)
+    arr = hip.seg_array(segs.seg_args(), L)
+    plan = attention_plan(segs, L, dev)
+    other = A.create_acsr_segments(A.strided_patterns(1024, 64, 64), 16, dev)
+    arr_o = hip.seg_array(other.seg_args(), 1024)
+    g = torch.Generator().manual_seed(21)
+    q, k, v = (torch.randn(B, H, L, d, generator=g).to(dtype).to(dev) for _ in range(3))
+    q2, k2, v2 = (torch.randn(1, 1, 1024, d, generator=g).to(dtype).to(dev) for _ in range(3))
+    out_g, want, junk = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q2)
+    lib = hip.lib()
+    noalloc = lambda st: hip.check(lib.splat_attention_fwd_noalloc(*forward_args(q, k.transpose(2, 3), v, out_g, arr, 1, d ** -0.5), st),
+                                   "splat_attention_fwd_noalloc")
+    noalloc(hip.stream_ptr(dev))                                # warm-up, eager
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            noalloc(hip.stream_ptr(dev))
+    torch.cuda.current_stream(dev).wait_stream(side)
+    for seed in (1, 2, 3):
+        gen = torch.Generator().manual_seed(seed)
+        for t in (q, k, v):
+            t.copy_(torch.randn(B, H, L, d, generator=gen).to(dtype))
+        # another mask's call leaves its plan in the shared buffer
+        hip.check(lib.splat_attention_fwd_noalloc(*forward_args(q2, k2.transpose(2, 3), v2, junk, arr_o, len(other), 0.1),
+                                                  hip.stream_ptr(dev)), "splat_attention_fwd_noalloc")
+        torch.cuda.synchronize()
+        out_g.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        hip.check(lib.splat_attention_fwd_planned(*forward_args(q, k.transpose(2, 3), v, want, arr, 1, d ** -0.5), plan.data_ptr(),
+                                                  plan.numel(), hip.stream_ptr(dev)), "splat_attention_fwd_planned")
+        torch.cuda.synchronize()
+        assert torch.equal(out_g.view(torch.int16), want.view(torch.int16)), seed

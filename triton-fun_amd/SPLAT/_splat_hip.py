@@ -56,9 +56,7 @@ _SIGNATURES = {
     "splat_attention_fwd_noalloc": (ctypes.c_int, [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _vp,
                                                    _i64, _i64, _i64, ctypes.POINTER(AcsrSeg), _i32, _i32, _i32, _i32, _i32,
                                                    _f32, _i32, _vp]),
-    "splat_stream_copy": (ctypes.c_int, [_vp, _vp, _i64, _vp]),
     "splat_transpose_keys": (ctypes.c_int, [_vp, _i64, _i64, _i64, _vp, _i32, _i32, _i32, _i32, _i32, _vp]),
-    "splat_mfma_lds_probe": (ctypes.c_int, [_vp, _i64, _vp, _i64, _i32, _i32, _vp]),
     "splat_softmax_bwd": (ctypes.c_int, [_vp, _vp, _vp, ctypes.POINTER(AcsrSeg), _i32, _i64, _i32, _i32, _f32, _i32, _vp]),
     "splat_spmm_t": (ctypes.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, ctypes.POINTER(AcsrSeg), ctypes.POINTER(AcsrSeg), _i32, _i32,
                                    _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),

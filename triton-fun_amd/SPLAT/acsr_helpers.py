@@ -378,6 +378,30 @@ def create_acsr_segments(masks: Sequence, BLOCK_HEIGHT: int, GPU_ID: Any) -> ACS
     return ACSRSegments(tuples, [t[3].splat_first_col for t in tuples])
 
 
+def non_affine_rows(mask_u8: torch.Tensor, row_first: torch.Tensor, sTod_lin: torch.Tensor, nnz: torch.Tensor,
+                    chunk_rows: int = 2048) -> torch.Tensor:
+    """Indices (int64, on the mask's device) of the rows of a 0/1 byte mask whose live columns are not the arithmetic
+    progression ``first + step * t, t < nnz`` that the row's metadata stands for (``instantiate_metadata`` takes the step
+    from the first two live columns only, acsr_helpers.py:112-124, and nothing in the reference looks at the rest of the
+    row).  A row passes when all of its ``nnz`` ones sit on the progression's ``nnz`` positions, which makes the two sets
+    equal.  Plain tensor code, so it runs on host tensors as well."""
+    rows, cols = mask_u8.shape
+    n = nnz.to(torch.int64)
+    step = sTod_lin.to(torch.int64).clamp(min=1)
+    first = row_first.to(torch.int64)
+    bad = []
+    width = int(n.max()) if rows else 0
+    t = torch.arange(max(width, 1), device=mask_u8.device, dtype=torch.int64)[None, :]
+    for r0 in range(0, rows, chunk_rows):
+        r1 = min(rows, r0 + chunk_rows)
+        pos = first[r0:r1, None] + step[r0:r1, None] * t
+        live = t < n[r0:r1, None]
+        inside = live & (pos >= 0) & (pos < cols)
+        hits = (mask_u8[r0:r1].gather(1, pos.clamp(0, cols - 1)).to(torch.int64) * inside).sum(1)
+        bad.append(torch.nonzero(hits != n[r0:r1]).flatten() + r0)
+    return torch.cat(bad) if bad else torch.empty(0, dtype=torch.int64, device=mask_u8.device)
+
+
 def row_extents(mask, GPU_ID: Any) -> tuple[torch.Tensor, torch.Tensor]:
     """(first, last) nonzero column per row as int32 device tensors (cols / -1 for an empty row)."""
     b = build_acsr(mask, 16, _hip.resolve_device(GPU_ID))

@@ -13,7 +13,8 @@ The transposed products read the compressed matrices as they are and take the AC
 which rows a column meets (``compressed_transpose_launcher`` can also store a matrix in that ACSR's layout, after which
 ``rspmm_launcher`` gives the same products).  The transposed mask must have affine rows as well, which holds for every
 closed-form pattern (band, blocked, dilated, strided); for arbitrary affine-row masks it need not, and the gradients
-with respect to k and v would then be wrong.
+with respect to k and v would then be wrong: ``transposed_segments`` checks every row of a transposed mask that came as
+an array or tensor against its metadata and raises ``SplatError`` instead.
 """
 from __future__ import annotations
 
@@ -23,7 +24,7 @@ import numpy as np
 import torch
 
 import _splat_hip as _hip
-from acsr_helpers import ACSRSegments, MaskPattern, create_acsr_segments, transpose_keys
+from acsr_helpers import ACSRSegments, MaskPattern, build_acsr, create_acsr_segments, non_affine_rows, transpose_keys
 from r_sddmm import rsddmm_launcher
 from r_softmax import rsoftmax_launcher
 from r_spmm import rspmm_launcher
@@ -43,8 +44,22 @@ def transposed_mask(mask, device: Any):
 
 
 def transposed_segments(masks: Sequence, BLOCK_HEIGHT: int, GPU_ID: Any) -> ACSRSegments:
-    """The ACSR of the transpose of every segment mask, in the same order."""
-    return create_acsr_segments([transposed_mask(m, GPU_ID) for m in masks], BLOCK_HEIGHT, GPU_ID)
+    """The ACSR of the transpose of every segment mask, in the same order.  A mask whose transpose has a row that is not
+    an arithmetic progression of columns (the mask's rows may all be affine while its columns are not) cannot be walked
+    from that ACSR: ``SplatError``.  Closed-form patterns are exempt: their transposes are closed-form too."""
+    dev = _hip.resolve_device(GPU_ID)
+    t_masks = [transposed_mask(m, GPU_ID) for m in masks]
+    for k, tm in enumerate(t_masks):
+        if isinstance(tm, MaskPattern):
+            continue
+        b = build_acsr(tm, BLOCK_HEIGHT, dev)
+        bad = non_affine_rows(tm, b.row_first, b.sTod_lin, b.nnz)
+        if bad.numel() > 0:
+            raise _hip.SplatError(
+                f"segment {k}: {bad.numel()} column(s) of the mask (the first is column {int(bad[0])}) meet rows that do not "
+                "form an arithmetic progression, so the transposed mask has no ACSR and the gradients with respect to k "
+                "and v cannot be computed from it; split the mask into segments whose columns are affine as well")
+    return create_acsr_segments(t_masks, BLOCK_HEIGHT, GPU_ID)
 
 
 def softmax_backward_launcher(p: torch.Tensor, dp: torch.Tensor, ds: torch.Tensor, segments: ACSRSegments,

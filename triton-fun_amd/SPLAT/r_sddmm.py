@@ -116,20 +116,22 @@ def rsddmm_launcher(x: torch.Tensor, y: torch.Tensor, output: torch.Tensor,
 
 
 def live_slot_columns(sTod_linear_transformations: torch.Tensor, sTod_translations: torch.Tensor, nnzs: torch.Tensor,
-                      trailing_dim: int) -> tuple[torch.Tensor, torch.Tensor]:
+                      trailing_dim: int, first_col: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
     """(columns int64 [rows, T], live bool [rows, T]): the dense column behind every compressed slot by the builder's
     rule c = sTod_lin * (s + sTod_trans) (acsr_helpers.py:122-124; for unit steps the same as the reference checkers'
     round(s * lin + trans), r_sddmm.py:210), and which slots are live (s < nnz).  Rows with one live column store
-    translation 0 whatever the column is; their column is taken from the builder's ``splat_first_col``."""
+    translation 0 whatever the column is; their column is taken from ``first_col`` (int tensor [rows]) or, when that is
+    not given, from the builder's ``splat_first_col`` attribute of ``sTod_translations`` (a slice or copy of that tensor
+    no longer carries the attribute, so callers that slice pass ``first_col`` themselves)."""
     lin = sTod_linear_transformations.double()
     trans = sTod_translations.double()
     slots = torch.arange(trailing_dim, device=lin.device, dtype=torch.float64)
     cols = torch.round(lin[:, None] * (slots[None, :] + trans[:, None])).long()
     live = slots[None, :] < nnzs.double()[:, None]
-    first = getattr(sTod_translations, "splat_first_col", None)
+    first = first_col if first_col is not None else getattr(sTod_translations, "splat_first_col", None)
     if first is not None:
         single = nnzs == 1
-        cols[single, 0] = first.long()[single]
+        cols[single, 0] = first.to(cols.device).long()[single]
     return cols, live
 
 
@@ -145,7 +147,9 @@ def is_correct(out_torch: torch.Tensor, out_rsddmm: torch.Tensor,
     column.  Prints the reference's verdict lines and returns the verdict."""
     rows = len(mask) if not isinstance(mask, torch.Tensor) else mask.shape[0]
     T = out_rsddmm.shape[-1]
-    cols, live = live_slot_columns(sTod_linear_transofrmations[:rows], sTod_translations[:rows], nnzs[:rows], T)
+    first = getattr(sTod_translations, "splat_first_col", None)  # read before slicing: a slice drops the attribute
+    cols, live = live_slot_columns(sTod_linear_transofrmations[:rows], sTod_translations[:rows], nnzs[:rows], T,
+                                   None if first is None else first[:rows])
     cols = cols.clamp_(0, out_torch.shape[-1] - 1).to(out_torch.device)
     want = out_torch[:batch_size, :num_heads, :rows].double().gather(3, cols.expand(batch_size, num_heads, rows, T))
     diff = (want - out_rsddmm[:batch_size, :num_heads, :rows].double().to(want.device)).abs()

@@ -74,7 +74,9 @@ def is_correct(left_tensor: torch.Tensor, right_tensor: torch.Tensor, out_rspmm:
     dev = left_tensor.device
     T = left_tensor.shape[-1]
     n_keys = right_tensor.shape[2]
-    cols, live = live_slot_columns(sTod_linear_transofrmations[:rows], sTod_translations[:rows], nnzs[:rows], T)
+    first = getattr(sTod_translations, "splat_first_col", None)  # read before slicing: a slice drops the attribute
+    cols, live = live_slot_columns(sTod_linear_transofrmations[:rows], sTod_translations[:rows], nnzs[:rows], T,
+                                   None if first is None else first[:rows])
     cols, live = cols.clamp_(0, n_keys - 1).to(dev), live.to(dev)
     total, n_bad = 0.0, 0
     for b in range(batch_size):

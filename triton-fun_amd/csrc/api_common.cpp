@@ -24,15 +24,30 @@ int fail(int code, const char* fmt, ...) {
     return code;
 }
 
-// An error left behind by another user of the runtime on this thread (it is sticky until someone reads it) must not
-// be reported as this library's: read it away before launching.
-void begin_launch() { (void)hipGetLastError(); }
+// An error left behind by another user of the runtime on this thread stays pending until someone reads it.  It must not
+// be taken for a failure of this library's launch, and it must not vanish either (its owner may not have looked yet):
+// it is read away before launching, remembered, and handed to the caller by check_launch() under its own name.
+static thread_local hipError_t g_foreign = hipSuccess;
+
+void begin_launch() {
+    if (hipPeekAtLastError() != hipSuccess) g_foreign = hipGetLastError();
+}
 
 int check_launch(const char* what) {
+    const hipError_t foreign = g_foreign;
+    g_foreign = hipSuccess;
     hipError_t e = hipGetLastError();
-    if (e == hipSuccess) return 0;
-    set_error("%s: launch failed: %s", what, hipGetErrorString(e));
-    return (int)e;
+    if (e != hipSuccess) {
+        set_error("%s: launch failed: %s", what, hipGetErrorString(e));
+        return (int)e;
+    }
+    if (foreign != hipSuccess) {
+        set_error("%s: a runtime error from an earlier call on this thread was still pending when this call began (%s); "
+                  "this call's own launch went through",
+                  what, hipGetErrorString(foreign));
+        return (int)foreign;
+    }
+    return 0;
 }
 
 int reserve_dynamic_lds(uint64_t* done, const void* kernel, size_t bytes, const char* who) {

@@ -272,38 +272,9 @@ static int dispatch_out(const void* x, void* y, const SoftmaxSegs& segs, int64_t
     return fail(SPLAT_E_DTYPE, "splat_softmax: unknown out_dtype %d", out_dtype);
 }
 
-// The streaming ceiling the HBM-bound kernels here are held against: a plain copy with the loads and stores the row
-// softmax uses (16 bytes per lane, non-temporal, four requests in flight per lane), workgroups striding over the buffer.
-__global__ __launch_bounds__(256) void stream_copy_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, int64_t n16) {
-    constexpr int UNROLL = 4;
-    int64_t chunk = (int64_t)blockIdx.x * (UNROLL * 256);
-    const int64_t stride = (int64_t)gridDim.x * (UNROLL * 256);
-    for (; chunk + UNROLL * 256 <= n16; chunk += stride) {
-        u32x4 r[UNROLL];
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) r[u] = __builtin_nontemporal_load(src + chunk + u * 256 + threadIdx.x);
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) __builtin_nontemporal_store(r[u], dst + chunk + u * 256 + threadIdx.x);
-    }
-    // the tail that does not fill a whole chunk
-    const int64_t n_full = n16 / (UNROLL * 256) * (UNROLL * 256);
-    if (blockIdx.x == 0)
-        for (int64_t i = n_full + threadIdx.x; i < n16; i += 256) dst[i] = src[i];
-}
-
 }  // namespace splat
 
 using namespace splat;
-
-extern "C" int splat_stream_copy(const void* src, void* dst, int64_t bytes, void* stream) {
-    begin_launch();
-    if (!src || !dst) return fail(SPLAT_E_NULL, "splat_stream_copy: null pointer argument");
-    if (bytes <= 0 || (bytes & 15) != 0) return fail(SPLAT_E_SHAPE, "splat_stream_copy: bytes must be a positive multiple of 16 (got %lld)", (long long)bytes);
-    if (((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) != 0)
-        return fail(SPLAT_E_ALIGN, "splat_stream_copy: src and dst must be 16-byte aligned");
-    stream_copy_kernel<<<8192, 256, 0, (hipStream_t)stream>>>(static_cast<const u32x4*>(src), static_cast<u32x4*>(dst), bytes / 16);
-    return check_launch("splat_stream_copy");
-}
 
 extern "C" int splat_softmax(const void* x, void* y, const splat_acsr_seg* segs, int32_t n_seg, int64_t BH, int32_t L,
                              int32_t T, int32_t in_dtype, int32_t out_dtype, void* stream) {
