@@ -193,3 +193,37 @@ def test_pattern_builder_needs_no_mask_for_long_sequences(dev):
     a = np.maximum(0, i - w + 1).astype(np.float64)
     assert np.array_equal(bits(got[3]), bits(a)) and np.array_equal(bits(got[4]), bits(np.minimum(i + 1, w)))
     assert got[5] == w
+
+
+def test_a_trailing_dimension_given_by_the_caller_spares_the_read_back(dev):
+    """create_acsr(..., T=) returns the same arrays without reading the builder's record back; the record is read when
+    a launcher first needs its hints, and a wrong figure is refused there."""
+    import _splat_hip as hip
+    L, p = 1024, 99
+    pat = A.causal_windowed_pattern(L, p)
+    A._MASK_CACHE.clear()
+    got = A.create_acsr(pat, 16, dev, T=p + 1)
+    assert A.build_acsr(pat, 16, dev).summary is not None        # nothing has been read back yet
+    A._MASK_CACHE.clear()
+    want = A.create_acsr(pat, 16, dev)
+    assert got[5] == want[5] == p + 1
+    for a, b in zip(got, want):
+        if isinstance(a, torch.Tensor):
+            assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+    assert int(got[3].splat_row_stride) == int(want[3].splat_row_stride) == 1 and int(got[3].splat_max_step) == 1
+    # used by a launcher like any other metadata
+    x = torch.rand(1, 1, L, p + 1, device=dev)
+    y = torch.empty_like(x)
+    r_softmax.rsoftmax_launcher(x, y, got[0], got[1], got[2], got[3], got[5], 128, got[4], (1, 1), 16)
+    live = torch.arange(p + 1, device=dev)[None, :] < got[4][:, None]
+    sums = torch.where(live, y[0, 0], torch.zeros((), device=dev)).sum(-1)
+    assert torch.allclose(sums, torch.ones_like(sums), atol=1e-5)
+    # a wrong figure: refused when the metadata is first used (and at once when the build has been read back already)
+    A._MASK_CACHE.clear()
+    wrong = A.create_acsr(pat, 16, dev, T=p)
+    z = torch.rand(1, 1, L, p, device=dev)
+    with pytest.raises(hip.SplatError, match="longest row has 100"):
+        r_softmax.rsoftmax_launcher(z, z, wrong[0], wrong[1], wrong[2], wrong[3], wrong[5], 128, wrong[4], (1, 1), 16)
+    with pytest.raises(hip.SplatError, match="longest row has 100"):
+        A.create_acsr(pat, 16, dev, T=p)
+    A._MASK_CACHE.clear()

@@ -183,8 +183,9 @@ def _host_mask_bytes(mask) -> np.ndarray:
 
 def _cache_key(mask, host_bytes: np.ndarray | None = None) -> tuple:
     """What identifies a mask's contents.  Tensors: storage address, version counter (bumped by every in-place
-    edit), shape, strides, storage offset and dtype -- a transposed or offset view of the same storage is another
-    mask.  Patterns: the (frozen) descriptor.  Lists and arrays are mutable without a trace, so they are keyed on a
+    edit made through the tensor itself; writes through ``.data``, ``.numpy()`` or another alias leave it alone, and a
+    mask edited that way needs ``_MASK_CACHE.clear()`` before it is built again), shape, strides, storage offset and
+    dtype -- a transposed or offset view of the same storage is another mask.  Patterns: the (frozen) descriptor.  Lists and arrays are mutable without a trace, so they are keyed on a
     digest of their bytes, taken from the uint8 copy that the upload needs anyway."""
     if isinstance(mask, torch.Tensor):
         return ("t", mask.data_ptr(), mask._version, tuple(mask.shape), tuple(mask.stride()), mask.storage_offset(),
@@ -232,10 +233,57 @@ def mask_shape(mask) -> tuple[int, int]:
     return (len(mask), len(mask[0]))
 
 
+class _FromSummary:
+    """An integer the builder left on the device (its summary record), read back when somebody asks for its value and
+    not before: ``int(x)`` synchronises once, then every figure of the record is known."""
+    __slots__ = ("build", "name")
+
+    def __init__(self, build: "AcsrBuild", name: str):
+        self.build, self.name = build, name
+
+    def __int__(self) -> int:
+        self.build.resolve()
+        return getattr(self.build, "_" + self.name)
+
+    __index__ = __int__
+
+    def __repr__(self) -> str:
+        return f"<{self.name} of an ACSR build, read back on use>"
+
+
 class AcsrBuild:
-    """Everything one ``splat_acsr_build`` call produced for (mask, BLOCK_HEIGHT)."""
-    __slots__ = ("dTos_lin", "dTos_trans", "sTod_lin", "sTod_trans", "nnz", "T", "span_start", "span_end",
-                 "row_first", "row_last", "row_stride", "max_step")
+    """Everything one ``splat_acsr_build`` call produced for (mask, BLOCK_HEIGHT).  ``T``, ``row_stride`` and
+    ``max_step`` come from a summary record the kernels leave on the device; reading it is the build's only
+    synchronisation and happens on first use (``resolve``)."""
+    __slots__ = ("dTos_lin", "dTos_trans", "sTod_lin", "sTod_trans", "nnz", "span_start", "span_end",
+                 "row_first", "row_last", "summary", "_T", "_row_stride", "_max_step")
+
+    def resolve(self) -> None:
+        if self.summary is None:
+            return
+        found = self.summary.cpu()  # the one synchronisation: T is returned as a Python int, like the reference
+        self.summary = None
+        assert int(found[1]) == 0, "Incorrect unpacking of affine-indices."
+        self._T = int(found[0])
+        # rows whose columns step by n and start in phase with the row index (dilated windows): kernels group them by phase
+        self._row_stride = int(found[2]) if (int(found[2]) == int(found[3]) and int(found[3]) > 1 and int(found[4]) == 0) else 1
+        # the largest column step of any row: above 1 some rows are gathered (dilated windows, strided far fields)
+        self._max_step = int(found[3])
+
+    @property
+    def T(self) -> int:
+        self.resolve()
+        return self._T
+
+    @property
+    def row_stride(self) -> int:
+        self.resolve()
+        return self._row_stride
+
+    @property
+    def max_step(self) -> int:
+        self.resolve()
+        return self._max_step
 
 
 def build_acsr(mask, BLOCK_HEIGHT: int, dev: torch.device) -> AcsrBuild:
@@ -253,9 +301,9 @@ def build_acsr(mask, BLOCK_HEIGHT: int, dev: torch.device) -> AcsrBuild:
     b.span_start, b.span_end = torch.empty(n_blocks, **f32), torch.empty(n_blocks, **f32)
     b.row_first = torch.empty(rows, dtype=torch.int32, device=dev)
     b.row_last = torch.empty(rows, dtype=torch.int32, device=dev)
-    summary = torch.empty(8, dtype=torch.int32, device=dev)
+    b.summary = torch.empty(8, dtype=torch.int32, device=dev)
     outs = (b.dTos_lin.data_ptr(), b.dTos_trans.data_ptr(), b.sTod_lin.data_ptr(), b.sTod_trans.data_ptr(), b.nnz.data_ptr(),
-            b.span_start.data_ptr(), b.span_end.data_ptr(), b.row_first.data_ptr(), b.row_last.data_ptr(), summary.data_ptr())
+            b.span_start.data_ptr(), b.span_end.data_ptr(), b.row_first.data_ptr(), b.row_last.data_ptr(), b.summary.data_ptr())
     with torch.cuda.device(dev):
         if dm is None:  # a MaskPattern: O(rows) work, no rows x cols buffer
             rc = _hip.lib().splat_acsr_build_pattern(mask.kind, mask.s, mask.p0, mask.p1, BLOCK_HEIGHT, *outs,
@@ -265,13 +313,6 @@ def build_acsr(mask, BLOCK_HEIGHT: int, dev: torch.device) -> AcsrBuild:
             rc = _hip.lib().splat_acsr_build(dm.data_ptr(), rows, cols, dm.stride(0), BLOCK_HEIGHT, *outs,
                                              _hip.stream_ptr(dev))
             _hip.check(rc, "splat_acsr_build")
-    found = summary.cpu()  # the one synchronisation: T is returned as a Python int, like the reference
-    assert int(found[1]) == 0, "Incorrect unpacking of affine-indices."
-    b.T = int(found[0])
-    # rows whose columns step by n and start in phase with the row index (dilated windows): kernels group them by phase
-    b.row_stride = int(found[2]) if (int(found[2]) == int(found[3]) and int(found[3]) > 1 and int(found[4]) == 0) else 1
-    # the largest column step of any row: above 1 some rows are gathered (dilated windows, strided far fields)
-    b.max_step = int(found[3])
     entry.builds[BLOCK_HEIGHT] = b
     return b
 
@@ -287,23 +328,56 @@ def instantiate_metadata(mask, BLOCK_HEIGHT: int, GPU_ID: Any = 0) -> ACSR:
     return ACSR(d2s, s2d, list(zip(b.span_start.tolist(), b.span_end.tolist())))
 
 
-def create_acsr(mask, BLOCK_HEIGHT: int, GPU_ID: Any):
+def create_acsr(mask, BLOCK_HEIGHT: int, GPU_ID: Any, *, T: int | None = None):
     """(dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnzs, T, span_loop_start, span_loop_end): seven float32
     device tensors and the trailing dimension T = max row nnz as an int.
 
+    The reference returns ``T`` as a Python int (acsr_helpers.py:153), which here means reading one word back from the
+    device: the call's only synchronisation.  A caller that knows the trailing dimension of its pattern passes it as
+    ``T=`` and the call only enqueues work; the builder's own figure (and its assertion on rows it could not solve) are
+    then checked when the metadata is first used by a launcher, where a mismatch raises ``SplatError``.
+
     The returned ``sTod_translations`` tensor carries an attribute ``splat_first_col`` (int32 tensor, first
     live column per row) that the launchers pick up: rows with a single live column store translation 0
-    whatever that column is, so the column itself has to travel separately.  ``splat_row_stride`` (int) is a speed
-    hint for patterns whose rows alternate column phase, ``splat_max_step`` (int) the largest column step of any row."""
+    whatever that column is, so the column itself has to travel separately.  ``splat_row_stride`` is a speed
+    hint for patterns whose rows alternate column phase, ``splat_max_step`` the largest column step of any row (both
+    convert with ``int()``; after a call with ``T=`` that conversion is what reads the builder's record back)."""
     dev = _hip.resolve_device(GPU_ID)
     b = build_acsr(mask, BLOCK_HEIGHT, dev)
+    if T is None:
+        b.resolve()
     # every caller gets tensors of its own, as from the reference's create_acsr: a build shared through the cache must
     # not change under one caller because another one wrote into its metadata
     arrays = [t.clone() for t in (b.dTos_lin, b.dTos_trans, b.sTod_lin, b.sTod_trans, b.nnz, b.span_start, b.span_end)]
     arrays[3].splat_first_col = b.row_first.clone()
-    arrays[3].splat_row_stride = b.row_stride
-    arrays[3].splat_max_step = b.max_step
-    return (arrays[0], arrays[1], arrays[2], arrays[3], arrays[4], b.T, arrays[5], arrays[6])
+    if b.summary is None:
+        if T is not None and int(T) != b.T:
+            raise _hip.SplatError(f"T={T} was given, the mask's longest row has {b.T} live columns")
+        arrays[3].splat_row_stride = b.row_stride
+        arrays[3].splat_max_step = b.max_step
+        t_out = b.T
+    else:
+        arrays[3].splat_row_stride = _CheckedHint(b, "row_stride", int(T))
+        arrays[3].splat_max_step = _CheckedHint(b, "max_step", int(T))
+        t_out = int(T)
+    return (arrays[0], arrays[1], arrays[2], arrays[3], arrays[4], t_out, arrays[5], arrays[6])
+
+
+class _CheckedHint(_FromSummary):
+    """A hint of a build whose trailing dimension the caller supplied: reading it also compares that figure with the
+    builder's."""
+    __slots__ = ("claimed_T",)
+
+    def __init__(self, build: AcsrBuild, name: str, claimed_T: int):
+        super().__init__(build, name)
+        self.claimed_T = claimed_T
+
+    def __int__(self) -> int:
+        if self.build.T != self.claimed_T:
+            raise _hip.SplatError(f"create_acsr was given T={self.claimed_T}, the mask's longest row has {self.build.T} live columns")
+        return super().__int__()
+
+    __index__ = __int__
 
 
 def transpose_keys(kT: torch.Tensor) -> torch.Tensor:

@@ -163,7 +163,9 @@ __global__ __launch_bounds__(256) void softmax_rows_vec(const Tin* __restrict__ 
                 if (live[c]) {
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
-                        float p = ((live[c] >> e) & 1u) ? fast_exp2(fmaf(v[c][e], kLog2e, -mb)) : 0.f;
+                        // dead slots hold -1e30 and underflow to exactly 0 against any real maximum; a row without live
+                        // slots stores nothing, so what its lanes compute does not matter
+                        float p = fast_exp2(fmaf(v[c][e], kLog2e, -mb));
                         v[c][e] = p;
                         sum += p;
                     }
@@ -234,7 +236,10 @@ static int launch_softmax(const void* x, void* y, const SoftmaxSegs& segs, int64
         if (chunks <= 16)
             softmax_rows_vec<Tin, Tout, 1, 16, 1, true><<<groups(4), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
         else if (chunks <= 32)
-            softmax_rows_vec<Tin, Tout, 1, 32, 4, true><<<groups(2 * 4), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
+            // 8 lanes and four chunks per row, eight rows per wavefront: the per-row work (live counts, masks, two
+            // reductions, the element-wise stores at a row's ends) is what such short rows cost, and eight rows share
+            // every instruction of it (+46 % over 32 lanes per row at T = 191)
+            softmax_rows_vec<Tin, Tout, 4, 8, 1, true><<<groups(8), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
         else if (chunks <= 64)
             softmax_rows_vec<Tin, Tout, 1, 64, 4, true><<<groups(4), 256, 0, st>>>(xi, yo, segs, n_rows, L, T);
         else if (chunks <= 128)
