@@ -206,6 +206,50 @@ __global__ __launch_bounds__(256) void acsr_rows_wide_kernel(const uint8_t* __re
     }
 }
 
+// Long rows, one wavefront per row: a wavefront takes its rows one after the other (consecutive wavefronts hold
+// consecutive rows at any time), each row in batches of eight 16-byte chunks per lane with the next batch requested
+// before the current one is scanned; no cross-wavefront reduction, no barrier, no LDS.
+__global__ __launch_bounds__(256) void acsr_rows_stream_kernel(const uint8_t* __restrict__ mask, int rows, int cols,
+                                                               int64_t ld, float* __restrict__ dTos_lin,
+                                                               float* __restrict__ dTos_trans, float* __restrict__ sTod_lin,
+                                                               float* __restrict__ sTod_trans, float* __restrict__ nnz_out,
+                                                               int32_t* __restrict__ row_first,
+                                                               int32_t* __restrict__ row_last, int32_t* __restrict__ summary) {
+    init_summary(summary);
+    const int lane = threadIdx.x & 63;
+    const int n_waves = gridDim.x * 4;
+    const int nvec = cols >> 4;
+    constexpr int NB = 8;
+    auto load_batch = [&](u32x4 (&xs)[NB], const u32x4* pv, int i0) {
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int i = i0 + 64 * u;
+            xs[u] = i < nvec ? __builtin_nontemporal_load(pv + i) : u32x4{0, 0, 0, 0};
+        }
+    };
+    for (int row = blockIdx.x * 4 + (threadIdx.x >> 6); row < rows; row += n_waves) {
+        const uint8_t* p = mask + (int64_t)row * ld;
+        const u32x4* pv = reinterpret_cast<const u32x4*>(p);
+        RowScan s;
+        s.init();
+        u32x4 cur[NB], nxt[NB];
+        load_batch(cur, pv, lane);
+        for (int i0 = lane; i0 < nvec; i0 += 64 * NB) {
+            const bool more = i0 + 64 * NB < nvec;
+            if (more) load_batch(nxt, pv, i0 + 64 * NB);
+#pragma unroll
+            for (int u = 0; u < NB; ++u) scan_chunk(s, cur[u], (i0 + 64 * u) << 4);
+            if (more) {
+#pragma unroll
+                for (int u = 0; u < NB; ++u) cur[u] = nxt[u];
+            }
+        }
+        for (int c = (nvec << 4) + lane; c < cols; c += 64) s.byte(p[c], c);
+        s.wave_reduce();
+        if (lane == 0) finish_row(s, row, cols, dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnz_out, row_first, row_last);
+    }
+}
+
 // One thread per row block: span_start = min(cols, min_r trans_r), span_end = max(-1, max_r nnz_r*lin_r + trans_r)
 // evaluated in double from the exact integers (a, lin, nnz) and rounded once to float32.  The same pass reduces
 // the summary: T = max nnz, smallest / largest column step over rows with nnz > 1, and how many rows with
@@ -431,7 +475,13 @@ extern "C" int splat_acsr_build(const uint8_t* mask, int64_t rows, int64_t cols,
         return fail(SPLAT_E_SHAPE, "splat_acsr_build: rows and cols are limited to 2^23 (got %lld, %lld)", (long long)rows, (long long)cols);
     hipStream_t st = (hipStream_t)stream;
     const int vec_ok = ((reinterpret_cast<uintptr_t>(mask) & 15) == 0 && (ld & 15) == 0) ? 1 : 0;
-    if (vec_ok && cols >= 4096)
+    // rows of 16 KiB and more: a workgroup per row; 4 to 16 KiB: a wavefront per row, each wavefront taking several rows
+    // (at 8 KiB rows 0.028 against 0.038 ms with caches flushed; at 16 KiB the two are equal and the workgroup form is
+    // 5 % faster on a mask that is found in the caches)
+    if (vec_ok && cols >= 4096 && cols < 16384)
+        acsr_rows_stream_kernel<<<(unsigned)min((int64_t)1024, (rows + 3) / 4), 256, 0, st>>>(mask, (int)rows, (int)cols, ld, dTos_lin, dTos_trans, sTod_lin,
+                                                              sTod_trans, nnz, row_first, row_last, summary);
+    else if (vec_ok && cols >= 4096)
         acsr_rows_wide_kernel<<<(unsigned)rows, 256, 0, st>>>(mask, (int)rows, (int)cols, ld, dTos_lin, dTos_trans, sTod_lin,
                                                               sTod_trans, nnz, row_first, row_last, summary);
     else
