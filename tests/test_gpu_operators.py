@@ -204,6 +204,116 @@ def test_sddmm_line_wise_output_two_segments(dev):
     assert torch.all(got[~lv] == SENTINEL)
 
 
+def _random_rows_mask(L, seed, steps, max_cnt):
+    """Rows with a random first column, count and (if `steps` has more than one entry) step; row 3 empty, row 5 a single
+    column, one row with exactly `max_cnt` columns."""
+    rng = np.random.default_rng(seed)
+    m = np.zeros((L, L), np.uint8)
+    for r in range(L):
+        st = int(rng.choice(steps))
+        n = int(rng.integers(0, max_cnt + 1))
+        if r == 3:
+            n = 0
+        if r == 5:
+            n = 1
+        if r == 7:
+            n, st = max_cnt, 1
+        a = int(rng.integers(0, L - st * max(n, 1)))
+        m[r, a:a + st * n:st] = 1
+    return m
+
+
+MANY_BLOCKS = {
+    # d = 128, rows of one or two lines: steps of 64 keys, half lines; L is not a multiple of the row block
+    "causal128_d128": (lambda: O.create_causal_windowed_mask(1000, 127), 128),
+    # d = 64, rows of one line: half lines
+    "causal64_d64": (lambda: O.create_causal_windowed_mask(1000, 63), 64),
+    # d = 128, long rows: steps of 32 keys, whole lines; row-stride grouping
+    "dilated512_d128": (lambda: O.create_dilated_mask(1024, 512, 2), 128),
+    "blocked512_d128": (lambda: O.create_blocked_mask(1024, 256), 128),
+    # every row its own span (an empty row, a single-column row): uniform plans whose wavefronts never drop the tests
+    "ragged304_d128": (lambda: _random_rows_mask(1024, 31, [1], 304), 128),
+    "ragged96_d64": (lambda: _random_rows_mask(1024, 32, [1], 96), 64),
+    # rows with differing steps: dense walks, element-wise stores
+    "steps200_d64": (lambda: _random_rows_mask(1024, 33, [1, 2, 3], 200), 64),
+    "steps200_d128": (lambda: _random_rows_mask(1024, 34, [1, 2, 3], 200), 128),
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", list(MANY_BLOCKS))
+def test_sddmm_16_bit_in_launches_of_many_row_blocks(dev, case, dtype):
+    """16-bit SDDMM with d = 64 / 128, aligned rows and at least 512 row blocks runs the kernel of thin wavefronts
+    (K through an LDS-DMA ring, scores through per-row rings, stores of whole or half lines): every variant it has, on
+    uniform and non-uniform plans, against the oracle; dead slots untouched."""
+    make, d = MANY_BLOCKS[case]
+    mask = make()
+    L = mask.shape[0]
+    B, H = 8, 8  # 64 x 8 row blocks = 512
+    q, k, _ = O.make_inputs(41, B, H, L, d, dtype)
+    acsr, acsr_np = acsr_pair(mask, 16, dev)
+    T = acsr[5]
+    assert T % 8 == 0
+    scale = d ** -0.5
+    out = torch.full((B, H, L, T), SENTINEL, dtype=dtype, device=dev)
+    r_sddmm.rsddmm_launcher(q.to(dev), k.to(dev).transpose(2, 3), out, acsr[0], acsr[1], acsr[2], acsr[3], T, acsr[4],
+                            (1, 1), None, None, 16, 16, scale=scale)
+    want = O.sddmm(q, k.transpose(2, 3), acsr_np, scale, first_col=O.row_extents(mask)[0])
+    got = out.float().cpu()
+    lv = live(acsr_np)
+    tol = TOL[dtype] * max(1.0, float(want.abs().max()))
+    assert float((got - want)[..., lv].abs().max()) <= tol
+    assert torch.all(got[..., ~lv] == SENTINEL), "dead slots must not be written"
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("make,d", [(lambda: O.create_causal_windowed_mask(1000, 255), 128),
+                                    (lambda: O.create_dilated_mask(1024, 128, 2), 64)], ids=["causal256_d128", "dilated64_d64"])
+def test_sddmm_probabilities_in_launches_of_many_row_blocks(dev, make, d, dtype):
+    """The same kernel with a row statistic: exp(scale * score - lse[row]) in the live slots."""
+    mask = make()
+    L = mask.shape[0]
+    B, H = 8, 8
+    q, k, _ = O.make_inputs(42, B, H, L, d, dtype)
+    acsr, acsr_np = acsr_pair(mask, 16, dev)
+    T = acsr[5]
+    assert T % 8 == 0
+    scale = d ** -0.5
+    scores = torch.einsum("bhqd,bhkd->bhqk", q.float(), k.float()) * scale
+    lse = torch.logsumexp(scores.masked_fill(torch.as_tensor(mask == 0), float("-inf")), dim=-1)
+    want = O.softmax_compressed(O.sddmm(q, k.transpose(2, 3), acsr_np, scale), live(acsr_np))
+    out = torch.full((B, H, L, T), SENTINEL, dtype=dtype, device=dev)
+    r_sddmm.rsddmm_launcher(q.to(dev), k.to(dev).transpose(2, 3), out, acsr[0], acsr[1], acsr[2], acsr[3], T, acsr[4],
+                            (1, 1), None, None, 16, 16, scale=scale, lse=lse.to(dev).contiguous())
+    got = out.float().cpu()
+    lv = live(acsr_np)
+    tol = {torch.float16: 1e-3, torch.bfloat16: 8e-3}[dtype]   # rounding of values <= 1
+    assert float((got - want)[..., lv].abs().max()) <= tol
+    assert torch.all(got[..., ~lv] == SENTINEL)
+
+
+def test_sddmm_two_aligned_segments_in_a_launch_of_many_row_blocks(dev):
+    """Two segments per row whose slots both start on 16-byte boundaries (local window 384 + every 8th earlier column: the
+    second segment's slots start at offset 384 of a row of 464): the thin-wavefront kernel walks one segment after the
+    other through the same rings."""
+    L, d = 1024, 128
+    pats = A.strided_patterns(L, 384, 8)
+    dms = O.create_strided_segment_masks(L, 384, 8)
+    segs = A.create_acsr_segments(pats, 16, dev)
+    assert segs.T % 8 == 0 and len(segs) == 2
+    B, H = 8, 8
+    q, k, _ = O.make_inputs(43, B, H, L, d, torch.bfloat16)
+    out = torch.full((B, H, L, segs.T), SENTINEL, dtype=torch.bfloat16, device=dev)
+    r_sddmm.rsddmm_launcher(q.to(dev), k.to(dev).transpose(2, 3), out, None, None, None, None, segs.T, None, None, None, None,
+                            16, 16, scale=d ** -0.5, segments=segs)
+    dense = (q.float() @ k.float().transpose(2, 3)) * d ** -0.5
+    want = torch.cat([O.compress(dense, O.create_acsr(m, 16), first_col=O.row_extents(m)[0], fill=SENTINEL) for m in dms], dim=-1)
+    got = out.float().cpu()
+    lv = want != SENTINEL
+    assert float((got - want)[lv].abs().max()) <= TOL[torch.bfloat16] * max(1.0, float(dense.abs().max()))
+    assert torch.all(got[~lv] == SENTINEL)
+
+
 # ---------------------------------------------------------------- softmax
 @pytest.mark.parametrize("n,p", REF_SMALL)
 def test_softmax_reference_cases(dev, n, p):

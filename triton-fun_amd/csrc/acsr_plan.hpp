@@ -61,46 +61,58 @@ __device__ __forceinline__ void gather_row_maps(const SegPtrs* seg, int n_seg, i
                                                 PlanScratch<BM>* ps, int tid) {
     static_assert(BM <= 256, "one row per thread");
     const int lane = tid & 63, wave = tid >> 6;
+    // wavefronts that hold no row leave neutral partial results and only take part in the barriers
+    const bool has_rows = (wave * 64 < BM);  // wavefront-uniform
     RowMap mine[SPLAT_MAX_SEGMENTS];
+    if (has_rows) {
 #pragma unroll
-    for (int sg = 0; sg < SPLAT_MAX_SEGMENTS; ++sg) {
-        RowMap m = {0, 1, 0};
-        if (sg < n_seg && tid < BM && r0 + rs * tid < n_rows) m = load_row_map(seg[sg], r0 + rs * tid);
-        mine[sg] = m;
-        if (sg < n_seg) {
-            if (tid < BM) {
-                ps->row_a[sg][tid] = m.a;
-                ps->row_lin[sg][tid] = m.lin;
-                ps->row_cnt[sg][tid] = m.cnt;
-            }
-            const int amin = wave_min_i(m.cnt > 0 ? m.a : 0x7fffffff);
-            const int cmax = wave_max_i(m.cnt > 0 ? m.a + m.lin * (m.cnt - 1) : -1);
-            const int linmin = wave_min_i(m.cnt > 1 ? m.lin : 0x7fffffff);
-            const int linmax = wave_max_i(m.cnt > 1 ? m.lin : 0);
-            if (lane == 0 && wave < 4) {
-                ps->part[wave][sg][0] = amin;
-                ps->part[wave][sg][1] = cmax;
-                ps->part[wave][sg][2] = linmin;
-                ps->part[wave][sg][3] = linmax;
+        for (int sg = 0; sg < SPLAT_MAX_SEGMENTS; ++sg) {
+            RowMap m = {0, 1, 0};
+            if (sg < n_seg && tid < BM && r0 + rs * tid < n_rows) m = load_row_map(seg[sg], r0 + rs * tid);
+            mine[sg] = m;
+            if (sg < n_seg) {
+                if (tid < BM) {
+                    ps->row_a[sg][tid] = m.a;
+                    ps->row_lin[sg][tid] = m.lin;
+                    ps->row_cnt[sg][tid] = m.cnt;
+                }
+                const int amin = wave_min_i(m.cnt > 0 ? m.a : 0x7fffffff);
+                const int cmax = wave_max_i(m.cnt > 0 ? m.a + m.lin * (m.cnt - 1) : -1);
+                const int linmin = wave_min_i(m.cnt > 1 ? m.lin : 0x7fffffff);
+                const int linmax = wave_max_i(m.cnt > 1 ? m.lin : 0);
+                if (lane == 0) {
+                    ps->part[wave][sg][0] = amin;
+                    ps->part[wave][sg][1] = cmax;
+                    ps->part[wave][sg][2] = linmin;
+                    ps->part[wave][sg][3] = linmax;
+                }
             }
         }
+    } else if (lane < SPLAT_MAX_SEGMENTS && wave < 4) {
+        ps->part[wave][lane][0] = 0x7fffffff;
+        ps->part[wave][lane][1] = -1;
+        ps->part[wave][lane][2] = 0x7fffffff;
+        ps->part[wave][lane][3] = 0;
+        ps->flag[wave][lane] = 0;
     }
     __syncthreads();
+    if (has_rows) {
 #pragma unroll
-    for (int sg = 0; sg < SPLAT_MAX_SEGMENTS; ++sg) {
-        if (sg < n_seg) {
-            int amin = 0x7fffffff, linmin = 0x7fffffff, linmax = 0;
+        for (int sg = 0; sg < SPLAT_MAX_SEGMENTS; ++sg) {
+            if (sg < n_seg) {
+                int amin = 0x7fffffff, linmin = 0x7fffffff, linmax = 0;
 #pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                amin = min(amin, ps->part[w][sg][0]);
-                linmin = min(linmin, ps->part[w][sg][2]);
-                linmax = max(linmax, ps->part[w][sg][3]);
+                for (int w = 0; w < 4; ++w) {
+                    amin = min(amin, ps->part[w][sg][0]);
+                    linmin = min(linmin, ps->part[w][sg][2]);
+                    linmax = max(linmax, ps->part[w][sg][3]);
+                }
+                bool bad = (linmax != 0 && linmin != linmax);
+                const int step = (linmax == 0) ? 1 : linmin;  // no row with 2+ columns: any step fits
+                if (!bad && step > 1) bad = mine[sg].cnt > 0 && ((mine[sg].a - amin) % step) != 0;
+                const int any_bad = __any(bad) ? 1 : 0;
+                if (lane == 0) ps->flag[wave][sg] = any_bad;
             }
-            bool bad = (linmax != 0 && linmin != linmax);
-            const int step = (linmax == 0) ? 1 : linmin;  // no row with 2+ columns: any step fits
-            if (!bad && step > 1) bad = mine[sg].cnt > 0 && ((mine[sg].a - amin) % step) != 0;
-            const int any_bad = __any(bad) ? 1 : 0;
-            if (lane == 0 && wave < 4) ps->flag[wave][sg] = any_bad;
         }
     }
     __syncthreads();

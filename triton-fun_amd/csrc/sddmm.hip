@@ -13,28 +13,9 @@
 #include <algorithm>
 #include <type_traits>
 
-#include "acsr_plan.hpp"
+#include "sddmm_params.hpp"
 
 namespace splat {
-
-struct SddmmParams {
-    const void* q;
-    const void* k;
-    void* out;
-    int64_t q_sb, q_sh, q_sl;
-    int64_t k_sb, k_sh, k_sd, k_sl;
-    int B, H, L, n_keys, d, T;
-    float scale;
-    const float* row_lse;  // optional [B*H, L]: the output is exp(scale * score - row_lse[row]) instead of scale * score
-    int out_dtype;
-    int n_seg;
-    SegPtrs seg[SPLAT_MAX_SEGMENTS];
-    int n_row_blocks, total;
-    int q_vec, k_vec;  // 16-byte loads are legal for q / k
-    int out_vec;       // 16-bit outputs: every row's segment starts on a 16-byte boundary
-    int row_stride;
-    int key_split;  // workgroups per row block: each takes a contiguous share of every segment's tiles
-};
 
 template <typename T>
 struct SddmmGeom {
@@ -540,6 +521,8 @@ static int sddmm_common(const char* who, const void* q, int64_t q_sb, int64_t q_
     for (int k = 0; k < n_seg; ++k)
         if (segs[k].slot_offset % 8 != 0) p.out_vec = 0;
     hipStream_t st = (hipStream_t)stream;
+    begin_launch();
+    if (const int rc = launch_sddmm_lines(who, p, in_dtype, st)) return rc < 0 ? rc : check_launch(who);
     switch (in_dtype) {
         case SPLAT_F32: return launch_sddmm<float>(who, p, kt, st);
         case SPLAT_F16: return launch_sddmm<f16>(who, p, kt, st);
