@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define SPLAT_VERSION 600 /* major*10000 + minor*100 + patch; 0.2.0 added the planned forward, 0.3.0 splat_spmm_t, 0.4.0 splat_attention_fwd_stats, splat_sddmm_probs, 0.5.0 splat_attention_fwd_noalloc, 0.6.0 moved the two measurement aids out (libsplat_bench.so, splat_bench.h) */
+#define SPLAT_VERSION 700 /* major*10000 + minor*100 + patch; 0.2.0 added the planned forward, 0.3.0 splat_spmm_t, 0.4.0 splat_attention_fwd_stats, splat_sddmm_probs, 0.5.0 splat_attention_fwd_noalloc, 0.6.0 moved the two measurement aids out (libsplat_bench.so, splat_bench.h), 0.7.0 added splat_sddmm_planned */
 
 /* element types of q/k/v/score/output buffers */
 #define SPLAT_F32 0
@@ -138,6 +138,20 @@ int splat_sddmm_probs(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, c
                       const splat_acsr_seg* segs /* host */, int32_t n_seg, int32_t B, int32_t H,
                       int32_t L, int32_t n_keys, int32_t d, int32_t T, float scale, int32_t in_dtype,
                       int32_t out_dtype, const float* lse, void* stream);
+
+/* splat_sddmm (lse == NULL) or splat_sddmm_probs (lse != NULL) with the mask's plan table: `plan` is what
+ * splat_attention_plan wrote for the same segments and L (its per-block column ranges and per-row windows are those of
+ * every tiled kernel here, not only the fused one).  The kernel for 16-bit types, d = 64 / 128 and launches of at least
+ * 512 row blocks then starts its copies after two scalar loads instead of deriving the plan from the ACSR arrays
+ * (-7 % at B=2 H=32 L=8192 d=128 T=512, -18 % at B=4 H=16 L=4096 d=64 T=256); other shapes ignore the plan.  Same
+ * results bit for bit.  A plan built from other metadata gives wrong scores but no access outside the buffers.
+ * Replaces the same reference code as splat_sddmm (rsddmm_launcher, r_sddmm.py:153-188). */
+int splat_sddmm_planned(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT,
+                        int64_t k_sb, int64_t k_sh, int64_t k_sd, int64_t k_sl, void* out,
+                        const splat_acsr_seg* segs /* host */, int32_t n_seg, int32_t B, int32_t H,
+                        int32_t L, int32_t n_keys, int32_t d, int32_t T, float scale, int32_t in_dtype,
+                        int32_t out_dtype, const float* lse /* may be NULL */, const void* plan,
+                        int64_t plan_bytes, void* stream);
 
 /* Row softmax over the live slots of compressed rows: y[bh,r,s] = exp(x[bh,r,s]-max_r)/sum_r.
  * Replaces rsoftmax_launcher / r_softmax_1d_kernel, r_softmax.py:16-59,126-150, applied to every

@@ -292,6 +292,51 @@ def test_sddmm_probabilities_in_launches_of_many_row_blocks(dev, make, d, dtype)
     assert torch.all(got[..., ~lv] == SENTINEL)
 
 
+@pytest.mark.parametrize("case", list(MANY_BLOCKS))
+def test_sddmm_with_the_plan_table_equals_sddmm_without(dev, case):
+    """By default such launches read the mask's plan table (built on the first call, kept with the metadata); plan=False
+    makes every workgroup derive its plan from the ACSR arrays.  Same bits, live and dead slots alike; the table is built
+    once per metadata."""
+    make, d = MANY_BLOCKS[case]
+    mask = make()
+    L = mask.shape[0]
+    B, H = 8, 8
+    q, k, _ = O.make_inputs(44, B, H, L, d, torch.bfloat16)
+    acsr = A.create_acsr(mask, 16, dev)
+    T = acsr[5]
+    outs = []
+    for plan in (None, False, None):
+        out = torch.full((B, H, L, T), SENTINEL, dtype=torch.bfloat16, device=dev)
+        r_sddmm.rsddmm_launcher(q.to(dev), k.to(dev).transpose(2, 3), out, acsr[0], acsr[1], acsr[2], acsr[3], T, acsr[4],
+                                (1, 1), None, None, 16, 16, scale=d ** -0.5, plan=plan)
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    plans = acsr[3].splat_plans
+    assert len(plans) == 1
+
+
+def test_sddmm_refuses_a_plan_that_is_too_small_and_ignores_one_it_has_no_use_for(dev):
+    mask = O.create_causal_windowed_mask(1024, 127)
+    acsr = A.create_acsr(mask, 16, dev)
+    T = acsr[5]
+    segs = A.ACSRSegments.single(acsr[0], acsr[1], acsr[2], acsr[3], acsr[4], T)
+    plan = segs.plan(1024, dev)
+    q, k, _ = O.make_inputs(45, 8, 8, 1024, 64, torch.bfloat16)
+    out = torch.empty(8, 8, 1024, T, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(Exception, match="plan holds"):
+        r_sddmm.rsddmm_launcher(q.to(dev), k.to(dev).transpose(2, 3), out, acsr[0], acsr[1], acsr[2], acsr[3], T, acsr[4],
+                                (1, 1), None, None, 16, 16, plan=plan[:plan.numel() // 2])
+    # float32 takes the general kernel, which has no use for the table: same result with and without
+    q32, k32, _ = O.make_inputs(46, 1, 2, 1024, 40, torch.float32)
+    a = torch.full((1, 2, 1024, T), SENTINEL, dtype=torch.float32, device=dev)
+    b = torch.full_like(a, SENTINEL)
+    r_sddmm.rsddmm_launcher(q32.to(dev), k32.to(dev).transpose(2, 3), a, acsr[0], acsr[1], acsr[2], acsr[3], T, acsr[4],
+                            (1, 1), None, None, 16, 16, plan=plan)
+    r_sddmm.rsddmm_launcher(q32.to(dev), k32.to(dev).transpose(2, 3), b, acsr[0], acsr[1], acsr[2], acsr[3], T, acsr[4],
+                            (1, 1), None, None, 16, 16, plan=False)
+    assert torch.equal(a, b)
+
+
 def test_sddmm_two_aligned_segments_in_a_launch_of_many_row_blocks(dev):
     """Two segments per row whose slots both start on 16-byte boundaries (local window 384 + every 8th earlier column: the
     second segment's slots start at offset 384 of a row of 464): the thin-wavefront kernel walks one segment after the

@@ -47,6 +47,8 @@ _SIGNATURES = {
                                    _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _i32, _vp]),
     "splat_sddmm_probs": (ctypes.c_int, [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, ctypes.POINTER(AcsrSeg), _i32,
                                          _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _i32, _vp, _vp]),
+    "splat_sddmm_planned": (ctypes.c_int, [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, ctypes.POINTER(AcsrSeg), _i32,
+                                           _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _i32, _vp, _vp, _i64, _vp]),
     "splat_softmax": (ctypes.c_int, [_vp, _vp, ctypes.POINTER(AcsrSeg), _i32, _i64, _i32, _i32, _i32, _i32, _vp]),
     "splat_spmm": (ctypes.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, ctypes.POINTER(AcsrSeg), _i32, _i32, _i32, _i32, _i32,
                                   _i32, _i32, _i32, _i32, _vp]),

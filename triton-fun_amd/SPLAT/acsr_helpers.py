@@ -412,6 +412,7 @@ class ACSRSegments:
             self.offsets.append(off)
             off += int(t[5])
         self.T = off
+        self._plan_holder = None  # where plan() keeps its tables when not with this object
 
     def __len__(self) -> int:
         return len(self.tuples)
@@ -437,13 +438,41 @@ class ACSRSegments:
             return transpose_keys(kT).transpose(2, 3)
         return kT
 
+    def plan(self, L: int, device) -> torch.Tensor:
+        """The plan table of these segments for ``L`` rows (``splat_attention_plan``: which key tiles each 128-row block
+        walks, every row's window), built on first use and kept: with the segments themselves, or, for metadata that
+        came in as separate tensors, with its ``sTod_translations`` tensor (attribute ``splat_plans``), so that the
+        next launcher call with the same tensors finds it.  The metadata is taken to be immutable from then on."""
+        dev = _hip.resolve_device(device)
+        holder = self._plan_holder if self._plan_holder is not None else self
+        plans = getattr(holder, "splat_plans", None)
+        if plans is None:
+            plans = {}
+            holder.splat_plans = plans
+        key = (int(L), len(self), tuple(self.offsets), dev.index)
+        if key not in plans:
+            arr = _hip.seg_array(self.seg_args(), L)
+            nbytes = int(_hip.lib().splat_attention_plan_bytes(arr, len(self), L))
+            if nbytes <= 0:
+                raise _hip.SplatError(f"no plan for {len(self)} segments and L={L}")
+            table = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            with torch.cuda.device(dev):
+                rc = _hip.lib().splat_attention_plan(arr, len(self), L, table.data_ptr(), nbytes, _hip.stream_ptr(dev))
+                _hip.check(rc, "splat_attention_plan")
+                # once, so that later launches may run on any stream without ordering themselves after the plan kernel
+                torch.cuda.current_stream(dev).synchronize()
+            plans[key] = table
+        return plans[key]
+
     def seg_args(self) -> list[tuple]:
         return [(t[0], t[1], t[2], t[3], t[4], fc, off) for t, fc, off in zip(self.tuples, self.first_cols, self.offsets)]
 
     @staticmethod
     def single(dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnzs, T) -> "ACSRSegments":
         fc = getattr(sTod_trans, "splat_first_col", None)
-        return ACSRSegments([(dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnzs, T, None, None)], [fc])
+        segs = ACSRSegments([(dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnzs, T, None, None)], [fc])
+        segs._plan_holder = sTod_trans
+        return segs
 
 
 def create_acsr_segments(masks: Sequence, BLOCK_HEIGHT: int, GPU_ID: Any) -> ACSRSegments:

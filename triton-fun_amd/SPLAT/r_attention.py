@@ -32,16 +32,7 @@ def _is_segment_list(mask) -> bool:
 def attention_plan(segments: ACSRSegments, L: int, device) -> torch.Tensor:
     """The fused kernel's plan for these segments and ``L`` rows (which key tiles each 128-row block walks, every
     row's window): an opaque uint8 device tensor, built once per mask and handed to ``attention_launcher``."""
-    dev = _hip.resolve_device(device)
-    arr = _hip.seg_array(segments.seg_args(), L)
-    nbytes = int(_hip.lib().splat_attention_plan_bytes(arr, len(segments), L))
-    if nbytes <= 0:
-        raise _hip.SplatError(f"no plan for {len(segments)} segments and L={L}")
-    plan = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
-        rc = _hip.lib().splat_attention_plan(arr, len(segments), L, plan.data_ptr(), nbytes, _hip.stream_ptr(dev))
-    _hip.check(rc, "splat_attention_plan")
-    return plan
+    return segments.plan(L, device)
 
 
 def attention_launcher(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor, output: torch.Tensor,

@@ -64,19 +64,33 @@ def _strides4(t: torch.Tensor, name: str):
     return t.stride()
 
 
+def _takes_a_plan(x, output, y, B: int, H: int, L: int, d: int, T: int, segs: ACSRSegments) -> bool:
+    """Whether this launch runs the kernel that reads a plan table (the library decides by the same rules and ignores the
+    plan otherwise): 16-bit types, d = 64 / 128, rows of K contiguous, 16-byte alignment, at least 512 row blocks."""
+    if x.dtype not in (torch.float16, torch.bfloat16) or output.dtype != x.dtype or d not in (64, 128):
+        return False
+    if y.stride(2) != 1 or T % 8 != 0 or any(off % 8 for off in segs.offsets):
+        return False
+    return B * H * ((L + 127) // 128) >= 512
+
+
 def rsddmm_launcher(x: torch.Tensor, y: torch.Tensor, output: torch.Tensor,
                     dTos_linear_transformations: torch.Tensor, dTos_translations: torch.Tensor,
                     sTod_linear_transformations: torch.Tensor, sTod_translations: torch.Tensor,
                     trailing_dim: int, nnzs: torch.Tensor, grid_dim: tuple[int],
                     tb_map_x: torch.Tensor, tb_map_y: torch.Tensor,
                     BLOCK_SIZE_Y: int, BLOCK_SIZE_X: int, *, scale: float | None = None,
-                    segments: ACSRSegments | None = None, lse: torch.Tensor | None = None):
+                    segments: ACSRSegments | None = None, lse: torch.Tensor | None = None,
+                    plan: torch.Tensor | None | bool = None):
     """x = Q [B, H, L, d]; y = K^T [B, H, d, L] (any strides with unit stride along d or along L, so
     ``k.transpose(2, 3)`` of a [B, H, L, d] tensor needs no copy); output [B, H, L, T] is written in place for
     the live slots only.  ``grid_dim`` / ``tb_map_*`` / ``BLOCK_SIZE_*`` describe the reference's launch
     geometry and are accepted unchanged; the HIP kernel tiles by itself from the row maps.  With ``lse`` (float32
     [B, H, L], contiguous: every row's log of its sum of exp(scale * score), as the fused forward hands it out) the
     stored value is exp(scale * score - lse[row]), the row's softmax probability, instead of the score.
+    ``plan``: the mask's plan table (``ACSRSegments.plan``); by default the launches that use one (16-bit types, d = 64 or
+    128, at least 512 row blocks of 128 rows) build it on their first call and keep it with the metadata, ``False``
+    launches without one.  The results are the same bit for bit.
     Returns (output, sTod_linear_transformations, sTod_translations, nnzs)."""
     for name, t in (("x", x), ("y", y), ("output", output)):
         _hip.require_device_tensor(t, name)
@@ -105,6 +119,17 @@ def rsddmm_launcher(x: torch.Tensor, y: torch.Tensor, output: torch.Tensor,
         _hip.require_device_tensor(lse, "lse")
         if lse.dtype != torch.float32 or tuple(lse.shape) != (B, H, L) or not lse.is_contiguous() or lse.device != dev:
             raise _hip.SplatError(f"lse must be a contiguous float32 tensor of shape {(B, H, L)} on {dev}")
+    if plan is None and _takes_a_plan(x, output, y, B, H, L, d, trailing_dim, segs):
+        plan = segs.plan(L, dev)
+    if plan is not None and plan is not False:
+        _hip.require_device_tensor(plan, "plan")
+        if plan.device != dev:
+            raise _hip.SplatError(f"the plan lives on {plan.device}, the tensors on {dev}")
+        with torch.cuda.device(dev):
+            rc = _hip.lib().splat_sddmm_planned(*args, lse.data_ptr() if lse is not None else None, plan.data_ptr(),
+                                                plan.numel() * plan.element_size(), _hip.stream_ptr(dev))
+            _hip.check(rc, "splat_sddmm_planned")
+        return (output, sTod_linear_transformations, sTod_translations, nnzs)
     with torch.cuda.device(dev):
         if lse is None:
             rc = _hip.lib().splat_sddmm(*args, _hip.stream_ptr(dev))

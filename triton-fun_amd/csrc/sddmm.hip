@@ -486,7 +486,7 @@ using namespace splat;
 static int sddmm_common(const char* who, const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT, int64_t k_sb,
                         int64_t k_sh, int64_t k_sd, int64_t k_sl, void* out, const splat_acsr_seg* segs, int32_t n_seg, int32_t B,
                         int32_t H, int32_t L, int32_t n_keys, int32_t d, int32_t T, float scale, int32_t in_dtype,
-                        int32_t out_dtype, const float* row_lse, void* stream) {
+                        int32_t out_dtype, const float* row_lse, const void* plan, int64_t plan_bytes, void* stream) {
     if (!q || !kT || !out || !segs) return fail(SPLAT_E_NULL, "%s: null pointer argument", who);
     if (B <= 0 || H <= 0 || L <= 0 || n_keys <= 0 || d <= 0 || T <= 0)
         return fail(SPLAT_E_SHAPE, "%s: need B, H, L, n_keys, d, T > 0 (got %d, %d, %d, %d, %d, %d)", who, B, H, L, n_keys, d, T);
@@ -505,6 +505,14 @@ static int sddmm_common(const char* who, const void* q, int64_t q_sb, int64_t q_
     p.B = B; p.H = H; p.L = L; p.n_keys = n_keys; p.d = d; p.T = T;
     p.scale = scale;
     p.row_lse = row_lse;
+    p.plan = nullptr;
+    if (plan) {
+        if ((reinterpret_cast<uintptr_t>(plan) & 15) != 0) return fail(SPLAT_E_ALIGN, "%s: the plan must be 16-byte aligned", who);
+        const int64_t need = splat_attention_plan_bytes(segs, n_seg, L);
+        if (need <= 0 || plan_bytes < need)
+            return fail(SPLAT_E_SHAPE, "%s: the plan holds %lld bytes, this mask needs %lld", who, (long long)plan_bytes, (long long)need);
+        p.plan = static_cast<const PlanRec*>(plan);  // the variant for rows of K that are contiguous comes first
+    }
     p.out_dtype = out_dtype;
     p.n_seg = n_seg;
     if (int rc = fill_segs(who, segs, n_seg, p.seg, T)) return rc;
@@ -535,7 +543,7 @@ extern "C" int splat_sddmm(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_
                            int32_t L, int32_t n_keys, int32_t d, int32_t T, float scale, int32_t in_dtype, int32_t out_dtype,
                            void* stream) {
     return sddmm_common("splat_sddmm", q, q_sb, q_sh, q_sl, kT, k_sb, k_sh, k_sd, k_sl, out, segs, n_seg, B, H, L, n_keys, d, T,
-                        scale, in_dtype, out_dtype, nullptr, stream);
+                        scale, in_dtype, out_dtype, nullptr, nullptr, 0, stream);
 }
 
 extern "C" int splat_sddmm_probs(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT, int64_t k_sb,
@@ -546,5 +554,17 @@ extern "C" int splat_sddmm_probs(const void* q, int64_t q_sb, int64_t q_sh, int6
     if (!lse) return fail(SPLAT_E_NULL, "%s: null lse", who);
     if ((reinterpret_cast<uintptr_t>(lse) & 3) != 0) return fail(SPLAT_E_ALIGN, "%s: lse must be 4-byte aligned", who);
     return sddmm_common(who, q, q_sb, q_sh, q_sl, kT, k_sb, k_sh, k_sd, k_sl, out, segs, n_seg, B, H, L, n_keys, d, T, scale,
-                        in_dtype, out_dtype, lse, stream);
+                        in_dtype, out_dtype, lse, nullptr, 0, stream);
+}
+
+extern "C" int splat_sddmm_planned(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* kT, int64_t k_sb,
+                                   int64_t k_sh, int64_t k_sd, int64_t k_sl, void* out, const splat_acsr_seg* segs, int32_t n_seg,
+                                   int32_t B, int32_t H, int32_t L, int32_t n_keys, int32_t d, int32_t T, float scale,
+                                   int32_t in_dtype, int32_t out_dtype, const float* lse, const void* plan, int64_t plan_bytes,
+                                   void* stream) {
+    const char* who = "splat_sddmm_planned";
+    if (!plan) return fail(SPLAT_E_NULL, "%s: null plan", who);
+    if (lse && (reinterpret_cast<uintptr_t>(lse) & 3) != 0) return fail(SPLAT_E_ALIGN, "%s: lse must be 4-byte aligned", who);
+    return sddmm_common(who, q, q_sb, q_sh, q_sl, kT, k_sb, k_sh, k_sd, k_sl, out, segs, n_seg, B, H, L, n_keys, d, T, scale,
+                        in_dtype, out_dtype, lse, plan, plan_bytes, stream);
 }

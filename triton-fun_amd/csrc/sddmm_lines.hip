@@ -48,9 +48,10 @@ __device__ __forceinline__ void static_for(F&& f) {
 }
 
 // KEYS: keys per step (64 or 32); HL: slots per store unit (64: whole 128-byte lines, 32: halves of lines)
-template <int D, int NST, int KEYS, int HL>
+template <int D, int NST, int KEYS, int HL, int BM_, bool PLANNED>
 struct LinesGeom {
-    static constexpr int BM = 128;
+    static constexpr int BM = BM_;
+    static constexpr int NW = BM / 16;          // wavefronts per workgroup
     static constexpr int ROWB = D * 2;          // bytes per key row
     static constexpr int STAGE = KEYS * ROWB;   // bytes per step
     static constexpr int R_SLOTS = 2 * HL;      // ring slots per row: what waits for its unit to fill up, plus a unit's worth
@@ -59,19 +60,21 @@ struct LinesGeom {
     static constexpr int R_ROW = R_SLOTS * 2 + 16;
     static constexpr int RING_AT = NST * STAGE;
     static constexpr int PLAN_AT = RING_AT + BM * R_ROW;
-    static constexpr int LDS_BYTES = PLAN_AT + (int)sizeof(PlanScratch<BM>) + SPLAT_MAX_SEGMENTS * ((int)sizeof(SegPlan) + 4);
+    static constexpr int LDS_BYTES = PLANNED ? PLAN_AT : PLAN_AT + (int)sizeof(PlanScratch<BM>) + SPLAT_MAX_SEGMENTS * ((int)sizeof(SegPlan) + 4);
 };
 
-template <typename T, int D, int NST, int KEYS, int HL, bool PROBS>
-__global__ __launch_bounds__(512, 4) void sddmm_lines_kernel(const SddmmParams p) {
-    using G = LinesGeom<D, NST, KEYS, HL>;
+template <typename T, int D, int NST, int KEYS, int HL, int BM_, bool PROBS, bool PLANNED>
+__global__ __launch_bounds__(BM_ * 4, 4) void sddmm_lines_kernel(const SddmmParams p) {
+    using G = LinesGeom<D, NST, KEYS, HL, BM_, PLANNED>;
+    static_assert(!PLANNED || BM_ == kPlanBM, "the plan table is laid out for 128-row blocks");
+    constexpr int NW = G::NW;
     constexpr int NH = KEYS / 32;  // halves of 32 positions per step
-    static_assert(G::STAGE % 8192 == 0, "every wavefront copies whole kilobytes");
+    static_assert(G::STAGE % (NW * 1024) == 0, "every wavefront copies whole kilobytes");
     constexpr int NC = HL / 32;  // store instructions per unit and wavefront (16 or 8 rows each)
     constexpr int BM = G::BM, ROWB = G::ROWB, STAGE = G::STAGE, R_SLOTS = G::R_SLOTS, R_ROW = G::R_ROW;
     constexpr int KS = D / 32;          // MFMA steps over the contraction
     constexpr int CPR = ROWB / 16;      // 16-byte chunks per key row
-    constexpr int NI = STAGE / 8192;    // copy instructions per wavefront and step
+    constexpr int NI = STAGE / (NW * 1024);  // copy instructions per wavefront and step
     constexpr int AFTER = (NST - 2) * NI;  // copy instructions issued after those of the step that is waited for
     static_assert(G::PLAN_AT % 16 == 0, "plan scratch alignment");
 
@@ -112,14 +115,20 @@ __global__ __launch_bounds__(512, 4) void sddmm_lines_kernel(const SddmmParams p
     float exp_sub = 0.f;
     if constexpr (PROBS) exp_sub = p.row_lse[(int64_t)bh * L + min(my_r, L - 1)] * 1.4426950408889634f;
 
-    if (tid < SPLAT_MAX_SEGMENTS) s_off[tid] = p.seg[tid].slot_offset;
-    plan_segments<BM>(p.seg, p.n_seg, r0, rs, L, true, s_plan, s_ps, tid);
+    // the plan: computed here from the rows' maps, or taken from the mask's plan table (scalar loads for what the copies
+    // need, so that they can start at once; no LDS, no barrier)
+    if constexpr (!PLANNED) {
+        if (tid < SPLAT_MAX_SEGMENTS) s_off[tid] = p.seg[tid].slot_offset;
+        plan_segments<BM>(p.seg, p.n_seg, r0, rs, L, true, s_plan, s_ps, tid);
+    }
+    const PlanRec* const pt = p.plan;
+    const int n_rb = p.n_row_blocks;
 
     // this lane's 16 bytes of each of the step's copy instructions: chunk position `flat` of the stage
     int d_row[NI], d_col[NI];
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-        const int flat = (wave + 8 * i) * 64 + lane;
+        const int flat = (wave + NW * i) * 64 + lane;
         d_row[i] = flat / CPR;
         d_col[i] = logical_chunk<ROWB, 1>(d_row[i], flat % CPR) * 16;
     }
@@ -141,15 +150,40 @@ __global__ __launch_bounds__(512, 4) void sddmm_lines_kernel(const SddmmParams p
     const int64_t out_bh = (int64_t)bh * L * p.T;
 
     for (int sg = 0; sg < p.n_seg; ++sg) {
-        const SegPlan pl = s_plan[sg];
+        SegPlan pl;
+        if constexpr (PLANNED) {
+            const PlanRec r = plan_uniform_load(pt + plan_seg_at(p.n_seg, rb, sg));
+            pl = SegPlan{r[0], r[1], r[2], r[3]};
+        } else {
+            pl = s_plan[sg];
+        }
         const int n_steps = pl.n_tiles * (kBN / KEYS);
         if (n_steps == 0) continue;  // workgroup-uniform
-        const int off = s_off[sg];
+        const int off = PLANNED ? p.seg[sg].slot_offset : s_off[sg];
         const bool uniform = pl.uniform != 0;
 
-        RowWin mine = make_row_win(cached_row_map<BM>(s_ps, sg, my_rr), pl);
-        if (my_r >= L) mine.cnt = 0;
-        const WaveSpan span = wave_span(mine, uniform);
+        auto row_win = [&](int rr) {
+            RowWin w;
+            if constexpr (PLANNED) {
+                // (counts are clamped to the slots the segment owns in this buffer, like the ones read from the metadata)
+                const PlanRec r = pt[plan_row_at(n_rb, p.n_seg, rb, sg, rr)];
+                const int64_t most = uniform ? (int64_t)p.seg[sg].max_cnt : (int64_t)r[2] * (p.seg[sg].max_cnt - 1) + 1;
+                w = RowWin{r[0], (int)min((int64_t)r[1], most), r[2]};
+            } else {
+                w = make_row_win(cached_row_map<BM>(s_ps, sg, rr), pl);
+            }
+            if (r0 + rs * rr >= L) w.cnt = 0;
+            return w;
+        };
+        const RowWin mine = row_win(my_rr);
+        WaveSpan span;
+        if constexpr (PLANNED) {
+            // the table holds the spans of 32 rows: wider than this wavefront's 16, which only makes the tests below pass less often
+            const PlanRec r = plan_uniform_load(pt + plan_span_at(n_rb, p.n_seg, rb, sg, wave >> 1));
+            span = WaveSpan{r[0], r[1], r[2], r[3]};
+        } else {
+            span = wave_span(mine, uniform);
+        }
         const int lmin = span.lo_min, hmax = span.hi_max;
         const int lo4 = mine.lo & ~3;
         const int64_t my_base = out_bh + (int64_t)my_r * p.T + off;
@@ -158,12 +192,11 @@ __global__ __launch_bounds__(512, 4) void sddmm_lines_kernel(const SddmmParams p
         int64_t f_base[NC];
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
-            const RowWin w = make_row_win(cached_row_map<BM>(s_ps, sg, f_rr[c]), pl);
-            const int r = r0 + rs * f_rr[c];
+            const RowWin w = row_win(f_rr[c]);
             f_lo[c] = w.lo;
-            f_cnt[c] = (r < L) ? w.cnt : 0;
+            f_cnt[c] = w.cnt;
             f_done[c] = 0;
-            f_base[c] = out_bh + (int64_t)r * p.T + off;
+            f_base[c] = out_bh + (int64_t)(r0 + rs * f_rr[c]) * p.T + off;
         }
 
         // Steps whose keys all exist copy from a wavefront-uniform base (the step's first key) plus a per-lane byte offset
@@ -179,13 +212,13 @@ __global__ __launch_bounds__(512, 4) void sddmm_lines_kernel(const SddmmParams p
                 const char* base = kbytes + key_first * k_rowb;
 #pragma unroll
                 for (int i = 0; i < NI; ++i)
-                    dma16_uniform(base, d_off[i], s_kring + stage * STAGE + (wave + 8 * i) * 1024);
+                    dma16_uniform(base, d_off[i], s_kring + stage * STAGE + (wave + NW * i) * 1024);
                 return;
             }
 #pragma unroll
             for (int i = 0; i < NI; ++i) {
                 const int n = min(max(pl.c0 + pl.cs * (s * KEYS + d_row[i]), 0), p.n_keys - 1);
-                dma16(kbytes + n * k_rowb + d_col[i], s_kring + stage * STAGE + (wave + 8 * i) * 1024);
+                dma16(kbytes + n * k_rowb + d_col[i], s_kring + stage * STAGE + (wave + NW * i) * 1024);
             }
         };
 
@@ -344,44 +377,50 @@ __global__ __launch_bounds__(512, 4) void sddmm_lines_kernel(const SddmmParams p
     }
 }
 
-template <typename T, int D, int NST, int KEYS, int HL, bool PROBS>
-static int launch_lines_variant(const char* who, const SddmmParams& p, hipStream_t st) {
-    using G = LinesGeom<D, NST, KEYS, HL>;
-    static_assert(G::LDS_BYTES <= 80 * 1024, "two workgroups per compute unit");
+template <typename T, int D, int NST, int KEYS, int HL, int BM, bool PROBS, bool PLANNED>
+static int launch_lines_variant(const char* who, SddmmParams p, hipStream_t st) {
+    using G = LinesGeom<D, NST, KEYS, HL, BM, PLANNED>;
+    static_assert(G::LDS_BYTES * (256 / BM) <= 160 * 1024, "16 wavefronts per compute unit");
+    p.n_row_blocks = count_row_blocks(p.L, BM, p.row_stride);
+    const int64_t blocks = (int64_t)p.B * p.H * p.n_row_blocks;
+    if (blocks > 0x7ffffff0) return 0;
+    p.key_split = 1;
+    p.total = (int)blocks;
     static uint64_t reserved = 0;
-    auto kern = sddmm_lines_kernel<T, D, NST, KEYS, HL, PROBS>;
+    auto kern = sddmm_lines_kernel<T, D, NST, KEYS, HL, BM, PROBS, PLANNED>;
     if (int rc = reserve_dynamic_lds(&reserved, reinterpret_cast<const void*>(kern), G::LDS_BYTES, who)) return rc;
     const int grid = ((p.total + 7) / 8) * 8;
-    kern<<<grid, 512, G::LDS_BYTES, st>>>(p);
+    kern<<<grid, BM * 4, G::LDS_BYTES, st>>>(p);
     return 1;
 }
 
 // Whole 128-byte lines are what the memory system likes best (a blocked mask at d = 128: 0.25 ms against 0.34 ms with
 // halves), but their rings take 34 KiB of LDS, which at d = 128 leaves room for steps of 32 keys only (two barriers per
 // 64 keys).  Short rows (one or two lines) are better off with halves and steps of 64 keys.
-template <typename T, bool PROBS>
+template <typename T, bool PROBS, bool PLANNED>
 static int launch_lines_typed(const char* who, const SddmmParams& p, hipStream_t st) {
     if (p.d == 128) {
-        if (p.T >= 256) return launch_lines_variant<T, 128, 4, 32, 64, PROBS>(who, p, st);
-        return launch_lines_variant<T, 128, 3, 64, 32, PROBS>(who, p, st);
+        if (p.T >= 256) return launch_lines_variant<T, 128, PLANNED ? 5 : 4, 32, 64, 128, PROBS, PLANNED>(who, p, st);
+        return launch_lines_variant<T, 128, 3, 64, 32, 128, PROBS, PLANNED>(who, p, st);
     }
-    if (p.T >= 128) return launch_lines_variant<T, 64, 4, 64, 64, PROBS>(who, p, st);
-    return launch_lines_variant<T, 64, 4, 64, 32, PROBS>(who, p, st);
+    if (p.T >= 128) return launch_lines_variant<T, 64, 4, 64, 64, 128, PROBS, PLANNED>(who, p, st);
+    return launch_lines_variant<T, 64, 4, 64, 32, 128, PROBS, PLANNED>(who, p, st);
 }
 
 int launch_sddmm_lines(const char* who, const SddmmParams& p_in, int in_dtype, hipStream_t st) {
     if (in_dtype == SPLAT_F32 || p_in.out_dtype != in_dtype) return 0;
     if (p_in.d != 64 && p_in.d != 128) return 0;
     if (p_in.k_sd != 1 || !p_in.q_vec || !p_in.k_vec || !p_in.out_vec) return 0;
-    SddmmParams p = p_in;
-    p.n_row_blocks = count_row_blocks(p.L, 128, p.row_stride);
-    const int64_t blocks = (int64_t)p.B * p.H * p.n_row_blocks;
-    if (blocks < 512 || blocks > 0x7ffffff0) return 0;
-    p.key_split = 1;
-    p.total = (int)blocks;
+    const SddmmParams& p = p_in;
+    if ((int64_t)p.B * p.H * count_row_blocks(p.L, 128, p.row_stride) < 512) return 0;
     const bool probs = p.row_lse != nullptr;
-    if (in_dtype == SPLAT_BF16) return probs ? launch_lines_typed<bf16, true>(who, p, st) : launch_lines_typed<bf16, false>(who, p, st);
-    return probs ? launch_lines_typed<f16, true>(who, p, st) : launch_lines_typed<f16, false>(who, p, st);
+    const SddmmParams& pp = p;
+    auto go = [&](auto t, auto probs_c, auto planned_c) {
+        return launch_lines_typed<decltype(t), decltype(probs_c)::value, decltype(planned_c)::value>(who, pp, st);
+    };
+    auto by_plan = [&](auto t, auto probs_c) { return pp.plan ? go(t, probs_c, std::true_type{}) : go(t, probs_c, std::false_type{}); };
+    auto by_probs = [&](auto t) { return probs ? by_plan(t, std::true_type{}) : by_plan(t, std::false_type{}); };
+    return in_dtype == SPLAT_BF16 ? by_probs(bf16{}) : by_probs(f16{});
 }
 
 }  // namespace splat

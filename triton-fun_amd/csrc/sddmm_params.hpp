@@ -21,6 +21,7 @@ struct SddmmParams {
     int out_vec;       // 16-bit outputs: every row's segment starts on a 16-byte boundary
     int row_stride;
     int key_split;  // workgroups per row block: each takes a contiguous share of every segment's tiles
+    const PlanRec* plan;  // optional: the mask's plan table for 128-row blocks (variant for row-major K), else nullptr
 };
 
 // Launches the line-wise kernel when the problem has its shape (see sddmm_lines.hip); returns 1 when it did, 0 when the
