@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define SPLAT_VERSION 700 /* major*10000 + minor*100 + patch; 0.2.0 added the planned forward, 0.3.0 splat_spmm_t, 0.4.0 splat_attention_fwd_stats, splat_sddmm_probs, 0.5.0 splat_attention_fwd_noalloc, 0.6.0 moved the two measurement aids out (libsplat_bench.so, splat_bench.h), 0.7.0 added splat_sddmm_planned */
+#define SPLAT_VERSION 700 /* major*10000 + minor*100 + patch; 0.2.0 added the planned forward, 0.3.0 splat_spmm_t, 0.4.0 splat_attention_fwd_stats, splat_sddmm_probs, 0.5.0 splat_attention_fwd_noalloc, 0.6.0 moved the two measurement aids out (libsplat_bench.so, splat_bench.h), 0.7.0 added splat_sddmm_planned, splat_spmm_planned */
 
 /* element types of q/k/v/score/output buffers */
 #define SPLAT_F32 0
@@ -169,6 +169,18 @@ int splat_spmm(const void* p, const void* v, int64_t v_sb, int64_t v_sh, int64_t
                const splat_acsr_seg* segs /* host */, int32_t n_seg, int32_t B, int32_t H,
                int32_t L, int32_t n_keys, int32_t n_out, int32_t T, int32_t in_dtype,
                int32_t out_dtype, void* stream);
+
+/* splat_spmm with the mask's plan table (`plan` as in splat_sddmm_planned).  For 16-bit types, 64 or 128 output columns and
+ * launches of at least 512 row blocks this runs a kernel of thin wavefronts (16 rows, four per SIMD) that starts from the
+ * table: -11 % at B=2 H=32 L=8192 d=128 T=512, -15 % at B=4 H=16 L=4096 d=64 T=256, -30 % on rows of 64 slots; masks
+ * whose rows all start on multiples of 8 positions of their block's walk (blocked masks) are better served by splat_spmm
+ * (the Python launcher looks that up in the table once and picks).  Other shapes ignore the plan.  Same results as
+ * splat_spmm up to the order of the float32 additions.  Replaces the same reference code (rspmm_launcher,
+ * r_spmm.py:128-190). */
+int splat_spmm_planned(const void* p, const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sl, void* out,
+                       const splat_acsr_seg* segs /* host */, int32_t n_seg, int32_t B, int32_t H, int32_t L,
+                       int32_t n_keys, int32_t n_out, int32_t T, int32_t in_dtype, int32_t out_dtype,
+                       const void* plan, int64_t plan_bytes, void* stream);
 
 /* Fused forward: out = softmax_over_live_columns(scale * q.kT) . v with online softmax; the
  * compressed score matrix is never written to memory.  Equals the composition

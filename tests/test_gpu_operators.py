@@ -518,6 +518,92 @@ def test_spmm_16_bit_whole_rows_of_v(dev, make, n_out, dtype):
     assert float((got - want).abs().max()) <= TOL[dtype]
 
 
+def _spmm_case(mask, n_out, dtype, B=8, H=8, seed=51):
+    """Probabilities (NaN in the dead slots), V and the dense fp32 answer for one mask."""
+    L = mask.shape[0]
+    acsr_np = O.create_acsr(mask, 16)
+    cols, valid = O.slot_columns(acsr_np, first_col=O.row_extents(mask)[0])
+    T = cols.shape[-1]
+    lv = torch.from_numpy(valid)
+    g = torch.Generator().manual_seed(seed + n_out)
+    pr = torch.rand(B, H, L, T, generator=g)
+    pr = (pr / torch.where(lv, pr, torch.zeros(())).sum(-1, keepdim=True).clamp(min=1e-9)).to(dtype)
+    pr = torch.where(lv, pr, torch.full((), float("nan"), dtype=dtype))
+    v = torch.randn(B, H, L, n_out, generator=g).to(dtype)
+    dense = torch.zeros(B, H, L, L)
+    rows_i, slots_i = np.nonzero(valid)
+    ri, si = torch.from_numpy(rows_i), torch.from_numpy(slots_i)
+    dense[:, :, ri, torch.from_numpy(cols[rows_i, slots_i].astype(np.int64))] = torch.nan_to_num(pr.float())[:, :, ri, si]
+    return pr, v, dense @ v.float(), T
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", list(MANY_BLOCKS))
+def test_spmm_16_bit_in_launches_of_many_row_blocks(dev, case, dtype):
+    """16-bit SpMM with 64 / 128 output columns and at least 512 row blocks: with the mask's plan table (the default unless
+    every row starts on a multiple of 8 positions) the kernel of thin wavefronts runs -- probabilities straight from
+    memory or through per-row rings, spans that end inside half steps, rows that are empty or hold one column, rows with
+    differing steps -- and must agree with the dense product; dead slots hold NaN and must not reach the output; the
+    general kernel (plan=False) must agree too."""
+    make, d = MANY_BLOCKS[case]
+    mask = make()
+    L = mask.shape[0]
+    pr, v, want, T = _spmm_case(mask, d, dtype)
+    acsr = A.create_acsr(mask, 16, dev)
+    assert acsr[5] == T
+    outs = []
+    for plan in (None, False):
+        out = torch.full((8, 8, L, d), 7.0, dtype=dtype, device=dev)
+        r_spmm.rspmm_launcher(pr.to(dev), v.to(dev), out, acsr[0], acsr[1], acsr[2], acsr[3], acsr[6], acsr[7], T, acsr[4],
+                              (1, 1, 1), 16, 16, plan=plan)
+        got = out.float().cpu()
+        assert torch.isfinite(got).all()
+        assert float((got - want).abs().max()) <= TOL[dtype]
+        outs.append(got)
+    assert float((outs[0] - outs[1]).abs().max()) <= TOL[dtype] / 4
+    segs = A.ACSRSegments.single(acsr[0], acsr[1], acsr[2], acsr[3], acsr[4], T)
+    assert segs.plan_is_aligned(L, dev) == case.startswith("blocked")
+
+
+def test_spmm_with_a_plan_forced_on_an_aligned_mask_and_two_segments(dev):
+    """A blocked mask takes the general kernel by default; given its plan explicitly it runs the thin wavefronts, whose
+    rows then read their aligned chunks straight from memory.  Two aligned segments per row go one after the other."""
+    mask = O.create_blocked_mask(1024, 256)
+    pr, v, want, T = _spmm_case(mask, 128, torch.bfloat16, seed=52)
+    acsr = A.create_acsr(mask, 16, dev)
+    segs = A.ACSRSegments.single(acsr[0], acsr[1], acsr[2], acsr[3], acsr[4], T)
+    out = torch.full((8, 8, 1024, 128), 7.0, dtype=torch.bfloat16, device=dev)
+    r_spmm.rspmm_launcher(pr.to(dev), v.to(dev), out, acsr[0], acsr[1], acsr[2], acsr[3], acsr[6], acsr[7], T, acsr[4],
+                          (1, 1, 1), 16, 16, plan=segs.plan(1024, dev))
+    assert float((out.float().cpu() - want).abs().max()) <= TOL[torch.bfloat16]
+    with pytest.raises(Exception, match="plan holds"):
+        r_spmm.rspmm_launcher(pr.to(dev), v.to(dev), out, acsr[0], acsr[1], acsr[2], acsr[3], acsr[6], acsr[7], T, acsr[4],
+                              (1, 1, 1), 16, 16, plan=segs.plan(1024, dev)[:4096])
+    # two segments
+    L, d = 1024, 64
+    pats = A.strided_patterns(L, 384, 8)
+    dms = O.create_strided_segment_masks(L, 384, 8)
+    segs2 = A.create_acsr_segments(pats, 16, dev)
+    parts = [_spmm_case(m, d, torch.float16, seed=53 + i) for i, m in enumerate(dms)]
+    pr2 = torch.cat([pt[0] for pt in parts], dim=-1)
+    v2 = parts[0][1]
+    dense = torch.zeros(8, 8, L, L)
+    off = 0
+    for m, pt in zip(dms, parts):
+        cols, valid = O.slot_columns(O.create_acsr(m, 16), first_col=O.row_extents(m)[0])
+        rows_i, slots_i = np.nonzero(valid)
+        ri, si = torch.from_numpy(rows_i), torch.from_numpy(slots_i)
+        dense[:, :, ri, torch.from_numpy(cols[rows_i, slots_i].astype(np.int64))] += torch.nan_to_num(pt[0].float())[:, :, ri, si]
+    want2 = dense @ v2.float()
+    assert pr2.shape[-1] == segs2.T
+    out2 = torch.full((8, 8, L, d), 7.0, dtype=torch.float16, device=dev)
+    r_spmm.rspmm_launcher(pr2.to(dev), v2.to(dev), out2, None, None, None, None, None, None, segs2.T, None, None, 16, 16,
+                          segments=segs2)
+    got2 = out2.float().cpu()
+    assert torch.isfinite(got2).all()
+    assert float((got2 - want2).abs().max()) <= 2 * TOL[torch.float16]
+
+
 def test_comparison_sweeps_run_and_agree_with_dense(dev):
     """The sweep harness (successor of the reference's comparison.py:76-106) at toy size: one record per doubling of
     the sparsity parameter, nnz as the pattern's closed form, fused forward equal to dense attention with the same mask."""

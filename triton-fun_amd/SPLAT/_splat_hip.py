@@ -52,6 +52,8 @@ _SIGNATURES = {
     "splat_softmax": (ctypes.c_int, [_vp, _vp, ctypes.POINTER(AcsrSeg), _i32, _i64, _i32, _i32, _i32, _i32, _vp]),
     "splat_spmm": (ctypes.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, ctypes.POINTER(AcsrSeg), _i32, _i32, _i32, _i32, _i32,
                                   _i32, _i32, _i32, _i32, _vp]),
+    "splat_spmm_planned": (ctypes.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, ctypes.POINTER(AcsrSeg), _i32, _i32, _i32, _i32, _i32,
+                                          _i32, _i32, _i32, _i32, _vp, _i64, _vp]),
     "splat_attention_fwd": (ctypes.c_int, [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _vp,
                                            _i64, _i64, _i64, ctypes.POINTER(AcsrSeg), _i32, _i32, _i32, _i32, _i32, _f32,
                                            _i32, _vp]),

@@ -461,8 +461,22 @@ class ACSRSegments:
                 _hip.check(rc, "splat_attention_plan")
                 # once, so that later launches may run on any stream without ordering themselves after the plan kernel
                 torch.cuda.current_stream(dev).synchronize()
-            plans[key] = table
-        return plans[key]
+                # whether every live row starts on a multiple of 8 positions of its block's walk (blocked masks): one look
+                # at the rows' records of the first variant (gathered walks), which follow its 5 records per block and
+                # segment: [lo, cnt, lin, phase] each
+                n_rb = nbytes // (2 * len(self) * (5 + 128) * 16)
+                recs = table.view(torch.int32).view(-1, 4)
+                rows = recs[n_rb * len(self) * 5:n_rb * len(self) * (5 + 128)]
+                aligned = bool((((rows[:, 0] & 7) == 0) | (rows[:, 1] <= 0)).all())
+            plans[key] = (table, aligned)
+        return plans[key][0]
+
+    def plan_is_aligned(self, L: int, device) -> bool:
+        """Whether every row of the plan for ``L`` rows starts on a multiple of 8 positions (see ``plan``)."""
+        self.plan(L, device)
+        holder = self._plan_holder if self._plan_holder is not None else self
+        dev = _hip.resolve_device(device)
+        return holder.splat_plans[(int(L), len(self), tuple(self.offsets), dev.index)][1]
 
     def seg_args(self) -> list[tuple]:
         return [(t[0], t[1], t[2], t[3], t[4], fc, off) for t, fc, off in zip(self.tuples, self.first_cols, self.offsets)]

@@ -31,10 +31,16 @@ def rspmm_launcher(x: torch.Tensor, y: torch.Tensor, output: torch.Tensor,
                    sTod_linear_transformations: torch.Tensor, sTod_translations: torch.Tensor,
                    span_loop_start: torch.Tensor, span_loop_end: torch.Tensor,
                    acsr_trailing_dim: int, nnzs: torch.Tensor, grid_dim: tuple[int],
-                   BLOCK_SIZE_Y: int, BLOCK_SIZE_X: int, *, segments: ACSRSegments | None = None):
+                   BLOCK_SIZE_Y: int, BLOCK_SIZE_X: int, *, segments: ACSRSegments | None = None,
+                   plan: torch.Tensor | None | bool = None):
     """x = compressed probabilities [B, H, L, T]; y = V [B, H, n_keys, n]; output [B, H, L, n] written in place.
     ``span_loop_start/end`` (the reference's per-row-block key range) are accepted unchanged; the HIP
     kernel derives each workgroup's key range from the row maps themselves.
+    ``plan``: the mask's plan table (``ACSRSegments.plan``), which selects the kernel of thin wavefronts where the library
+    has one (16-bit types, 64 or 128 output columns, at least 512 row blocks of 128 rows); by default such launches build
+    the table on their first call, keep it with the metadata and use it unless every row of the mask starts on a multiple
+    of 8 positions (blocked masks: the general kernel is faster there); ``False`` always runs the general kernel.  The
+    two kernels agree up to the order of the float32 additions.
     Returns (output, sTod_linear_transformations, sTod_translations, nnzs)."""
     for name, t in (("x", x), ("y", y), ("output", output)):
         _hip.require_device_tensor(t, name)
@@ -55,6 +61,20 @@ def rspmm_launcher(x: torch.Tensor, y: torch.Tensor, output: torch.Tensor,
     vs = y.stride()
     dev = x.device
     arr = _hip.seg_array(segs.seg_args(), L, T)
+    if plan is None and x.dtype in (torch.float16, torch.bfloat16) and output.dtype == x.dtype and n_out in (64, 128) \
+            and B * H * ((L + 127) // 128) >= 512 and not segs.plan_is_aligned(L, dev):
+        plan = segs.plan(L, dev)
+    if plan is not None and plan is not False:
+        _hip.require_device_tensor(plan, "plan")
+        if plan.device != dev:
+            raise _hip.SplatError(f"the plan lives on {plan.device}, the tensors on {dev}")
+        with torch.cuda.device(dev):
+            rc = _hip.lib().splat_spmm_planned(x.data_ptr(), y.data_ptr(), vs[0], vs[1], vs[2], output.data_ptr(), arr,
+                                               len(segs), B, H, L, n_keys, n_out, T, _hip.dtype_code(x.dtype),
+                                               _hip.dtype_code(output.dtype), plan.data_ptr(),
+                                               plan.numel() * plan.element_size(), _hip.stream_ptr(dev))
+        _hip.check(rc, "splat_spmm_planned")
+        return (output, sTod_linear_transformations, sTod_translations, nnzs)
     with torch.cuda.device(dev):
         rc = _hip.lib().splat_spmm(x.data_ptr(), y.data_ptr(), vs[0], vs[1], vs[2], output.data_ptr(), arr, len(segs),
                                    B, H, L, n_keys, n_out, T, _hip.dtype_code(x.dtype), _hip.dtype_code(output.dtype),

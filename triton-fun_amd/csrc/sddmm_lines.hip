@@ -29,24 +29,6 @@
 
 namespace splat {
 
-typedef float f32x4v __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ void mma16(f32x4v& acc, const Frag<bf16>& a, const Frag<bf16>& b) {
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc, 0, 0, 0);
-}
-__device__ __forceinline__ void mma16(f32x4v& acc, const Frag<f16>& a, const Frag<f16>& b) {
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.v, b.v, acc, 0, 0, 0);
-}
-
-// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>)
-template <int N, int I = 0, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<N, I + 1>(f);
-    }
-}
-
 // KEYS: keys per step (64 or 32); HL: slots per store unit (64: whole 128-byte lines, 32: halves of lines)
 template <int D, int NST, int KEYS, int HL, int BM_, bool PLANNED>
 struct LinesGeom {

@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "../../include/splat_hip.h"
 
 namespace splat {
@@ -32,6 +34,15 @@ int check_launch(const char* what);
 int reserve_dynamic_lds(uint64_t* done, const void* kernel, size_t bytes, const char* who);
 
 constexpr int kWave = 64;
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>)
+template <int N, int I = 0, typename F>
+__host__ __device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<N, I + 1>(f);
+    }
+}
 
 template <typename T>
 struct ElemTraits;
@@ -67,6 +78,16 @@ __device__ __forceinline__ void mma32(f32x16& acc, const Frag<f16>& a, const Fra
 __device__ __forceinline__ void mma32(f32x16& acc, const Frag<float>& a, const Frag<float>& b) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.v[j], b.v[j], acc, 0, 0, 0);
+}
+
+// acc[16x16] += A[16x32] * B[32x16].  Lane (i = lane%16, g = lane/16) holds contraction slots 8g..8g+7 of row i (A) or
+// column i (B); of the output, lane (n = lane%16, g = lane/16) holds rows 4g..4g+3 of column n.
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void mma16(f32x4v& acc, const Frag<bf16>& a, const Frag<bf16>& b) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc, 0, 0, 0);
+}
+__device__ __forceinline__ void mma16(f32x4v& acc, const Frag<f16>& a, const Frag<f16>& b) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.v, b.v, acc, 0, 0, 0);
 }
 
 // Row (within a 32-row tile) held by accumulator register j of lane group g.

@@ -7,24 +7,9 @@
 // plan 8 consecutive positions of a row are 8 consecutive slots, one (possibly unaligned) 16-byte load.
 // Output orientation rows = queries, columns = output features, so stores are contiguous per row.
 // Bound by reading the compressed probabilities (HBM), not by MFMA.
-#include "acsr_plan.hpp"
+#include "spmm_params.hpp"
 
 namespace splat {
-
-struct SpmmParams {
-    const void* p;
-    const void* v;
-    void* out;
-    int64_t v_sb, v_sh, v_sl;
-    int B, H, L, n_keys, n_out, T;
-    int out_dtype;
-    int out_vec;  // 16-byte stores are legal for every row of out
-    int n_seg;
-    SegPtrs seg[SPLAT_MAX_SEGMENTS];
-    int n_row_blocks, total, n_col_chunks;
-    int v_vec;
-    int row_stride;
-};
 
 // Write a wavefront's 32 x (32*DVT) block of accumulators to rows r0 + rs*(32*wave + k) of out[bh] ([rows, n_out],
 // columns col0..).  An accumulator register holds one row's value at column lane%32: stored directly, a wavefront
@@ -602,25 +587,34 @@ static int launch_spmm_t(SpmmTParams p, hipStream_t st) {
 
 using namespace splat;
 
-extern "C" int splat_spmm(const void* pp, const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sl, void* out,
-                          const splat_acsr_seg* segs, int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t n_keys,
-                          int32_t n_out, int32_t T, int32_t in_dtype, int32_t out_dtype, void* stream) {
-    if (!pp || !v || !out || !segs) return fail(SPLAT_E_NULL, "splat_spmm: null pointer argument");
+static int spmm_common(const char* who, const void* pp, const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sl, void* out,
+                       const splat_acsr_seg* segs, int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t n_keys,
+                       int32_t n_out, int32_t T, int32_t in_dtype, int32_t out_dtype, const void* plan, int64_t plan_bytes,
+                       void* stream) {
+    if (!pp || !v || !out || !segs) return fail(SPLAT_E_NULL, "%s: null pointer argument", who);
     if (B <= 0 || H <= 0 || L <= 0 || n_keys <= 0 || n_out <= 0 || T <= 0)
-        return fail(SPLAT_E_SHAPE, "splat_spmm: need B, H, L, n_keys, n_out, T > 0 (got %d, %d, %d, %d, %d, %d)", B, H, L, n_keys, n_out, T);
-    if (L > (1 << 23) || n_keys > (1 << 23)) return fail(SPLAT_E_SHAPE, "splat_spmm: L and n_keys are limited to 2^23");
+        return fail(SPLAT_E_SHAPE, "%s: need B, H, L, n_keys, n_out, T > 0 (got %d, %d, %d, %d, %d, %d)", who, B, H, L, n_keys, n_out, T);
+    if (L > (1 << 23) || n_keys > (1 << 23)) return fail(SPLAT_E_SHAPE, "%s: L and n_keys are limited to 2^23", who);
     if (out_dtype != SPLAT_F32 && out_dtype != SPLAT_F16 && out_dtype != SPLAT_BF16)
-        return fail(SPLAT_E_DTYPE, "splat_spmm: unknown out_dtype %d", out_dtype);
+        return fail(SPLAT_E_DTYPE, "%s: unknown out_dtype %d", who, out_dtype);
     if (in_dtype != SPLAT_F32 && in_dtype != SPLAT_F16 && in_dtype != SPLAT_BF16)
-        return fail(SPLAT_E_DTYPE, "splat_spmm: unknown in_dtype %d", in_dtype);
-    if (v_sl < n_out) return fail(SPLAT_E_SHAPE, "splat_spmm: v row stride %lld < n_out %d", (long long)v_sl, n_out);
+        return fail(SPLAT_E_DTYPE, "%s: unknown in_dtype %d", who, in_dtype);
+    if (v_sl < n_out) return fail(SPLAT_E_SHAPE, "%s: v row stride %lld < n_out %d", who, (long long)v_sl, n_out);
     SpmmParams p;
     p.p = pp; p.v = v; p.out = out;
     p.v_sb = v_sb; p.v_sh = v_sh; p.v_sl = v_sl;
     p.B = B; p.H = H; p.L = L; p.n_keys = n_keys; p.n_out = n_out; p.T = T;
     p.out_dtype = out_dtype;
+    p.plan = nullptr;
+    if (plan) {
+        if ((reinterpret_cast<uintptr_t>(plan) & 15) != 0) return fail(SPLAT_E_ALIGN, "%s: the plan must be 16-byte aligned", who);
+        const int64_t need = splat_attention_plan_bytes(segs, n_seg, L);
+        if (need <= 0 || plan_bytes < need)
+            return fail(SPLAT_E_SHAPE, "%s: the plan holds %lld bytes, this mask needs %lld", who, (long long)plan_bytes, (long long)need);
+        p.plan = static_cast<const PlanRec*>(plan);  // the variant with gathered walks comes first
+    }
     p.n_seg = n_seg;
-    if (int rc = fill_segs("splat_spmm", segs, n_seg, p.seg, T)) return rc;
+    if (int rc = fill_segs(who, segs, n_seg, p.seg, T)) return rc;
     p.row_stride = common_row_stride(segs, n_seg);
     const int es = in_dtype == SPLAT_F32 ? 4 : 2;
     const int epc = 16 / es;
@@ -630,11 +624,29 @@ extern "C" int splat_spmm(const void* pp, const void* v, int64_t v_sb, int64_t v
         p.out_vec = ((reinterpret_cast<uintptr_t>(out) & 15) == 0 && ((int64_t)n_out * es_out) % 16 == 0) ? 1 : 0;
     }
     hipStream_t st = (hipStream_t)stream;
+    begin_launch();
+    if (const int rc = launch_spmm_thin(who, p, in_dtype, st)) return rc < 0 ? rc : check_launch(who);
     switch (in_dtype) {
         case SPLAT_F32: return launch_spmm<float>(p, st);
         case SPLAT_F16: return launch_spmm<f16>(p, st);
         default: return launch_spmm<bf16>(p, st);
     }
+}
+
+extern "C" int splat_spmm(const void* pp, const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sl, void* out,
+                          const splat_acsr_seg* segs, int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t n_keys,
+                          int32_t n_out, int32_t T, int32_t in_dtype, int32_t out_dtype, void* stream) {
+    return spmm_common("splat_spmm", pp, v, v_sb, v_sh, v_sl, out, segs, n_seg, B, H, L, n_keys, n_out, T, in_dtype, out_dtype,
+                       nullptr, 0, stream);
+}
+
+extern "C" int splat_spmm_planned(const void* pp, const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sl, void* out,
+                                  const splat_acsr_seg* segs, int32_t n_seg, int32_t B, int32_t H, int32_t L, int32_t n_keys,
+                                  int32_t n_out, int32_t T, int32_t in_dtype, int32_t out_dtype, const void* plan,
+                                  int64_t plan_bytes, void* stream) {
+    if (!plan) return fail(SPLAT_E_NULL, "splat_spmm_planned: null plan");
+    return spmm_common("splat_spmm_planned", pp, v, v_sb, v_sh, v_sl, out, segs, n_seg, B, H, L, n_keys, n_out, T, in_dtype,
+                       out_dtype, plan, plan_bytes, stream);
 }
 
 extern "C" int splat_spmm_t(const void* pp, const void* x, int64_t x_sb, int64_t x_sh, int64_t x_sl, void* out,
