@@ -75,8 +75,9 @@ __device__ __forceinline__ u32x4 shift_elements(u32x4 x, int k) {
 }
 
 // NB: register sets for probabilities in flight: requested NB steps (rings) or NB - 1 steps (straight from memory) ahead
-// RING: probabilities as whole aligned lines through per-row rings in LDS instead of per lane straight from memory
-template <typename T, int D, int NB, bool PLANNED, bool RING>
+// RING: probabilities as whole aligned lines through per-row rings in LDS instead of per lane straight from memory;
+// STREAM: those lines with non-temporal loads
+template <typename T, int D, int NB, bool PLANNED, bool RING, bool STREAM>
 __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
     using G = ThinGeom<D, PLANNED, RING>;
     constexpr int R_ROW = G::R_ROW;
@@ -211,7 +212,13 @@ __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
         auto load_line = [&](int t, int c) {
             u32x4 raw = {0u, 0u, 0u, 0u};
             const int slot = 64 * (t + f_la[c] + 1) + 8 * f_piece;
-            if (slot >= 0 && slot < f_cnt[c]) raw = *reinterpret_cast<const u32x4*>(f_row[c] + slot);  // 16-byte aligned
+            if (slot >= 0 && slot < f_cnt[c]) {  // 16-byte aligned
+                // a compressed matrix too large for the last-level cache streams past the L2, where V stays
+                if constexpr (STREAM)
+                    raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(f_row[c] + slot));
+                else
+                    raw = *reinterpret_cast<const u32x4*>(f_row[c] + slot);
+            }
             return raw;
         };
         auto write_line = [&](int t, int c, const u32x4& raw) {
@@ -425,7 +432,7 @@ __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
     }
 }
 
-template <typename T, int D, bool PLANNED, bool RING>
+template <typename T, int D, bool PLANNED, bool RING, bool STREAM>
 static int launch_thin_variant(const char* who, SpmmParams p, hipStream_t st) {
     using G = ThinGeom<D, PLANNED, RING>;
     static_assert(G::LDS_BYTES <= 80 * 1024, "two workgroups per compute unit");
@@ -436,7 +443,7 @@ static int launch_thin_variant(const char* who, SpmmParams p, hipStream_t st) {
     p.total = (int)blocks;
     static uint64_t reserved = 0;
     // (d = 128 with rings: a third set would spill)
-    auto kern = spmm_thin_kernel<T, D, D == 128 ? (RING ? 2 : 3) : 4, PLANNED, RING>;
+    auto kern = spmm_thin_kernel<T, D, D == 128 ? (RING ? 2 : 3) : 4, PLANNED, RING, STREAM>;
     if (int rc = reserve_dynamic_lds(&reserved, reinterpret_cast<const void*>(kern), G::LDS_BYTES, who)) return rc;
     const int grid = ((p.total + 7) / 8) * 8;
     kern<<<grid, 512, G::LDS_BYTES, st>>>(p);
@@ -457,9 +464,16 @@ int launch_spmm_thin(const char* who, const SpmmParams& p, int in_dtype, hipStre
     bool ring = (reinterpret_cast<uintptr_t>(p.p) & 15) == 0 && p.T % 8 == 0 && p.T >= 256;
     for (int k = 0; k < p.n_seg; ++k)
         if (p.seg[k].slot_offset % 8 != 0) ring = false;
+    // a compressed matrix too large for the 256 MB last-level cache streams past the L2, where V stays (config 4's 537 MB:
+    // -9 % with non-temporal loads; config 2's 134 MB, which repeated launches find in that cache: +5 %)
+    const bool stream = (int64_t)p.B * p.H * p.L * p.T * 2 > ((int64_t)192 << 20);
     auto go = [&](auto t, auto d_c, auto planned_c) {
-        if (ring) return launch_thin_variant<decltype(t), decltype(d_c)::value, decltype(planned_c)::value, true>(who, p, st);
-        return launch_thin_variant<decltype(t), decltype(d_c)::value, decltype(planned_c)::value, false>(who, p, st);
+        using TT = decltype(t);
+        constexpr int DD = decltype(d_c)::value;
+        constexpr bool PL = decltype(planned_c)::value;
+        if (ring && stream) return launch_thin_variant<TT, DD, PL, true, true>(who, p, st);
+        if (ring) return launch_thin_variant<TT, DD, PL, true, false>(who, p, st);
+        return launch_thin_variant<TT, DD, PL, false, false>(who, p, st);
     };
     auto by_plan = [&](auto t, auto d_c) { return go(t, d_c, std::true_type{}); };
     auto by_d = [&](auto t) {
