@@ -172,7 +172,7 @@ int splat_spmm(const void* p, const void* v, int64_t v_sb, int64_t v_sh, int64_t
 
 /* splat_spmm with the mask's plan table (`plan` as in splat_sddmm_planned).  For 16-bit types, 64 or 128 output columns and
  * launches of at least 512 row blocks this runs a kernel of thin wavefronts (16 rows, four per SIMD) that starts from the
- * table: -11 % at B=2 H=32 L=8192 d=128 T=512, -15 % at B=4 H=16 L=4096 d=64 T=256, -30 % on rows of 64 slots; masks
+ * table: -20 % at B=2 H=32 L=8192 d=128 T=512, -15 % at B=4 H=16 L=4096 d=64 T=256, -30 % on rows of 64 slots; masks
  * whose rows all start on multiples of 8 positions of their block's walk (blocked masks) are better served by splat_spmm
  * (the Python launcher looks that up in the table once and picks).  Other shapes ignore the plan.  Same results as
  * splat_spmm up to the order of the float32 additions.  Replaces the same reference code (rspmm_launcher,
