@@ -337,6 +337,48 @@ def test_sddmm_refuses_a_plan_that_is_too_small_and_ignores_one_it_has_no_use_fo
     assert torch.equal(a, b)
 
 
+def test_the_unfused_launchers_under_stream_capture(dev):
+    """A launcher whose first qualifying call happens under stream capture must not build its plan table there (that
+    synchronises): it runs without one, and a capture after an eager call uses the table that call left.  Replays equal
+    the eager results."""
+    mask = O.create_causal_windowed_mask(1024, 255)
+    L, d, B, H = 1024, 64, 8, 8
+    q, k, v = O.make_inputs(47, B, H, L, d, torch.bfloat16)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    kT = kd.transpose(2, 3)
+    outs = []
+    for warm in (False, True):
+        acsr = A.create_acsr(mask, 16, dev)
+        T = acsr[5]
+        scores = torch.full((B, H, L, T), SENTINEL, dtype=torch.bfloat16, device=dev)
+        o = torch.zeros(B, H, L, d, dtype=torch.bfloat16, device=dev)
+
+        def run():
+            r_sddmm.rsddmm_launcher(qd, kT, scores, acsr[0], acsr[1], acsr[2], acsr[3], T, acsr[4], (1, 1), None, None, 16, 16,
+                                    scale=d ** -0.5)
+            r_softmax.rsoftmax_launcher(scores, scores, acsr[0], acsr[1], acsr[2], acsr[3], T, 256, acsr[4], (1, 1), 16)
+            r_spmm.rspmm_launcher(scores, vd, o, acsr[0], acsr[1], acsr[2], acsr[3], acsr[6], acsr[7], T, acsr[4], (1, 1, 1), 16, 16)
+        if warm:
+            run()
+            assert hasattr(acsr[3], "splat_plans")
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                run()
+        torch.cuda.current_stream(dev).wait_stream(side)
+        assert warm or not hasattr(acsr[3], "splat_plans")
+        o.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        outs.append(o.clone())
+    want = O.dense_masked_attention(q, k.transpose(2, 3), v, np.asarray(mask), d ** -0.5)
+    for got in outs:
+        assert float((got.float().cpu() - want).abs().max()) <= 2 * TOL[torch.bfloat16]
+
+
 def test_sddmm_two_aligned_segments_in_a_launch_of_many_row_blocks(dev):
     """Two segments per row whose slots both start on 16-byte boundaries (local window 384 + every 8th earlier column: the
     second segment's slots start at offset 384 of a row of 464): the thin-wavefront kernel walks one segment after the

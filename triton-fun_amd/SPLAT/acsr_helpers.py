@@ -471,6 +471,12 @@ class ACSRSegments:
             plans[key] = (table, aligned)
         return plans[key][0]
 
+    def has_plan(self, L: int, device) -> bool:
+        """Whether ``plan`` would return a table it already holds (no kernel, no synchronisation)."""
+        dev = _hip.resolve_device(device)
+        holder = self._plan_holder if self._plan_holder is not None else self
+        return (int(L), len(self), tuple(self.offsets), dev.index) in getattr(holder, "splat_plans", {})
+
     def plan_is_aligned(self, L: int, device) -> bool:
         """Whether every row of the plan for ``L`` rows starts on a multiple of 8 positions (see ``plan``)."""
         self.plan(L, device)

@@ -119,7 +119,10 @@ def rsddmm_launcher(x: torch.Tensor, y: torch.Tensor, output: torch.Tensor,
         _hip.require_device_tensor(lse, "lse")
         if lse.dtype != torch.float32 or tuple(lse.shape) != (B, H, L) or not lse.is_contiguous() or lse.device != dev:
             raise _hip.SplatError(f"lse must be a contiguous float32 tensor of shape {(B, H, L)} on {dev}")
-    if plan is None and _takes_a_plan(x, output, y, B, H, L, d, trailing_dim, segs):
+    # (building the table synchronises once, which a stream under capture must not do: such a call uses a table only if an
+    # earlier call has left one)
+    if plan is None and _takes_a_plan(x, output, y, B, H, L, d, trailing_dim, segs) \
+            and (segs.has_plan(L, dev) or not torch.cuda.is_current_stream_capturing()):
         plan = segs.plan(L, dev)
     if plan is not None and plan is not False:
         _hip.require_device_tensor(plan, "plan")

@@ -62,7 +62,9 @@ def rspmm_launcher(x: torch.Tensor, y: torch.Tensor, output: torch.Tensor,
     dev = x.device
     arr = _hip.seg_array(segs.seg_args(), L, T)
     if plan is None and x.dtype in (torch.float16, torch.bfloat16) and output.dtype == x.dtype and n_out in (64, 128) \
-            and B * H * ((L + 127) // 128) >= 512 and not segs.plan_is_aligned(L, dev):
+            and B * H * ((L + 127) // 128) >= 512 \
+            and (segs.has_plan(L, dev) or not torch.cuda.is_current_stream_capturing()) \
+            and not segs.plan_is_aligned(L, dev):  # (no table is built under stream capture: building synchronises)
         plan = segs.plan(L, dev)
     if plan is not None and plan is not False:
         _hip.require_device_tensor(plan, "plan")
