@@ -231,6 +231,8 @@ MANY_BLOCKS = {
     # d = 128, long rows: steps of 32 keys, whole lines; row-stride grouping
     "dilated512_d128": (lambda: O.create_dilated_mask(1024, 512, 2), 128),
     "blocked512_d128": (lambda: O.create_blocked_mask(1024, 256), 128),
+    # row-stride grouping with a sequence length that fills neither the last row block nor the last group of two
+    "dilated128_L1000_d64": (lambda: O.create_dilated_mask(1000, 256, 2), 64),
     # every row its own span (an empty row, a single-column row): uniform plans whose wavefronts never drop the tests
     "ragged304_d128": (lambda: _random_rows_mask(1024, 31, [1], 304), 128),
     "ragged96_d64": (lambda: _random_rows_mask(1024, 32, [1], 96), 64),
