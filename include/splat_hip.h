@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define SPLAT_VERSION 700 /* major*10000 + minor*100 + patch; 0.2.0 added the planned forward, 0.3.0 splat_spmm_t, 0.4.0 splat_attention_fwd_stats, splat_sddmm_probs, 0.5.0 splat_attention_fwd_noalloc, 0.6.0 moved the two measurement aids out (libsplat_bench.so, splat_bench.h), 0.7.0 added splat_sddmm_planned, splat_spmm_planned */
+#define SPLAT_VERSION 800 /* major*10000 + minor*100 + patch; 0.2.0 added the planned forward, 0.3.0 splat_spmm_t, 0.4.0 splat_attention_fwd_stats, splat_sddmm_probs, 0.5.0 splat_attention_fwd_noalloc, 0.6.0 moved the two measurement aids out (libsplat_bench.so, splat_bench.h), 0.7.0 added splat_sddmm_planned, splat_spmm_planned, 0.8.0 splat_spmm_t_planned */
 
 /* element types of q/k/v/score/output buffers */
 #define SPLAT_F32 0
@@ -285,6 +285,20 @@ int splat_spmm_t(const void* p, const void* x, int64_t x_sb, int64_t x_sh, int64
                  const splat_acsr_seg* segs /* host */, const splat_acsr_seg* segs_t /* host */, int32_t n_seg,
                  int32_t B, int32_t H, int32_t L, int32_t Lt, int32_t n_out, int32_t T, int32_t in_dtype,
                  int32_t out_dtype, void* stream);
+/* splat_spmm_t with the plan table of the TRANSPOSED mask (splat_attention_plan on `segs_t` with Lt rows; plan_bytes >=
+ * splat_attention_plan_bytes(segs_t, n_seg, Lt), 16-byte aligned, device memory).  For 16-bit types of one kind for p, x
+ * and out, n_out = 64 or 128, 16-byte aligned x rows, every segment with a first_col array, T >= 8 and launches of at
+ * least 512 blocks of 128 output rows this runs a kernel of thin wavefronts (16 output rows each, four per SIMD) that
+ * starts from the table and keeps the tile loop's loads independent of one another: -31 % at B=2 H=32 L=8192 n_out=128
+ * T=512 (dilated), -28 % at B=4 H=16 L=4096 n_out=64 T=256, -33 % on blocks of 512.  It is built for rows whose column
+ * step equals the stride by which the transposed mask's rows are grouped (1 for windows and blocks, the dilation for
+ * dilated windows); rows of another step are walked a second time entry by entry, which the general kernel does better
+ * (the Python launcher picks by the metadata's largest step).  Other shapes ignore the plan.  Same results as
+ * splat_spmm_t.  No counterpart in the reference (it has no backward pass). */
+int splat_spmm_t_planned(const void* p, const void* x, int64_t x_sb, int64_t x_sh, int64_t x_sl, void* out,
+                         const splat_acsr_seg* segs /* host */, const splat_acsr_seg* segs_t /* host */, int32_t n_seg,
+                         int32_t B, int32_t H, int32_t L, int32_t Lt, int32_t n_out, int32_t T, int32_t in_dtype,
+                         int32_t out_dtype, const void* plan_t, int64_t plan_bytes, void* stream);
 int splat_compressed_transpose(const void* src, void* dst, const splat_acsr_seg* segs /* host */,
                                const splat_acsr_seg* segs_t /* host */, int32_t n_seg, int64_t BH,
                                int32_t L, int32_t T, int32_t Lt, int32_t Tt, int32_t dtype, void* stream);

@@ -238,6 +238,79 @@ def test_transposed_product(dev, make, dense, dtype, n_out):
     assert float((out.double() - out2.double()).abs().max().cpu()) <= tol
 
 
+def _staircase_mask(L, seed, width):
+    """Rows and columns both intervals of differing lengths (some empty): the lower and the upper column bound do not
+    decrease from one row to the next."""
+    rng = np.random.default_rng(seed)
+    lo = np.sort(rng.integers(0, L, L))
+    hi = np.maximum.accumulate(np.minimum(np.maximum(np.sort(rng.integers(0, L + width, L)), lo), lo + width))
+    m = np.zeros((L, L), np.uint8)
+    for r in range(L):
+        m[r, lo[r]:min(hi[r], L)] = 1
+    return m
+
+
+MANY_BLOCKS_T = {
+    # name: (segment masks, B*H, n_out, the plan table passed by hand)
+    # the sequence fills neither the last block of columns nor the last tile of rows
+    "causal127_L1000_n128": (lambda: [O.create_causal_windowed_mask(1000, 127)], 64, 128, False),
+    "window63_L1000_n64": (lambda: [O.create_windowed_mask(1000, 63)], 64, 64, False),
+    # blocks of columns grouped by a stride of 2 (a power of two) and of 3
+    "dilated256x2_n128": (lambda: [O.create_dilated_mask(1024, 256, 2)], 64, 128, False),
+    "dilated100x3_L1000_n64": (lambda: [O.create_dilated_mask(1000, 100, 3)], 64, 64, False),
+    "blocked256_n128": (lambda: [O.create_blocked_mask(1024, 256)], 64, 128, False),
+    # 26 tiles of rows per block of columns: more than the 16 whose row maps are prepared at a time
+    "causal1500_L2048_n64": (lambda: [O.create_causal_windowed_mask(2048, 1500)], 32, 64, False),
+    "staircase_n128": (lambda: [_staircase_mask(1024, 7, 300)], 64, 128, False),
+    # rows of another column step than the blocks' (the far field): the launcher would pick the general kernel, so the table
+    # is passed by hand; the kernel of thin wavefronts walks such rows a second time
+    "strided32_16_two_segments_n64": (lambda: O.create_strided_segment_masks(1024, 32, 16), 64, 64, True),
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", list(MANY_BLOCKS_T))
+def test_transposed_product_16_bit_in_launches_of_many_blocks(dev, case, dtype):
+    """16-bit transposed product with 64 / 128 output columns and at least 512 blocks of 128 output rows: with the plan
+    table of the transposed mask the kernel of thin wavefronts runs and must agree with the dense product and with the
+    general kernel (plan=False); dead slots hold NaN and must not reach the output."""
+    make, BH, n_out, by_hand = MANY_BLOCKS_T[case]
+    dms = [np.asarray(m) for m in make()]
+    L = dms[0].shape[0]
+    segs = A.create_acsr_segments(dms, 16, dev)
+    segs_t = transposed_segments(dms, 16, dev)
+    g = torch.Generator(device=dev).manual_seed(61)
+    full = torch.randn(1, BH, L, L, generator=g, device=dev).to(dtype)
+    x = torch.randn(1, BH, L, n_out, generator=g, device=dev).to(dtype)
+    src = torch.cat([O.compress(full, O.create_acsr(m, 16), first_col=O.row_extents(m)[0], fill=float("nan")) for m in dms], dim=-1)
+    assert src.shape[-1] == segs.T
+    live = torch.from_numpy(sum(m.astype(np.int64) for m in dms) > 0).to(dev)
+    want = torch.where(live, full.float(), torch.zeros((), device=dev)).transpose(2, 3) @ x.float()
+    del full
+    # exact products of 16-bit values summed in float32: what is left is the output's own rounding (2^-9 / 2^-12 of a value)
+    tol = {torch.float16: 1e-3, torch.bfloat16: 8e-3}[dtype] * float(want.abs().max())
+    outs = []
+    for plan in (segs_t.plan(L, dev) if by_hand else None, False):
+        out = torch.full((1, BH, L, n_out), 7.0, dtype=dtype, device=dev)
+        rspmm_t_launcher(src, x, out, segs, segs_t, plan=plan)
+        assert torch.isfinite(out).all()
+        assert float((out.float() - want).abs().max()) <= tol
+        outs.append(out)
+    assert segs_t.has_plan(L, dev)  # the first call built it (or the test did)
+    assert float((outs[0].float() - outs[1].float()).abs().max()) <= tol
+
+
+def test_transposed_product_refuses_a_plan_that_is_too_small(dev):
+    pat = [A.causal_windowed_pattern(1024, 100)]
+    segs, segs_t = A.create_acsr_segments(pat, 16, dev), transposed_segments(pat, 16, dev)
+    p = torch.zeros(8, 8, 1024, segs.T, device=dev, dtype=torch.bfloat16)
+    x = torch.zeros(8, 8, 1024, 64, device=dev, dtype=torch.bfloat16)
+    out = torch.zeros_like(x)
+    plan = segs_t.plan(1024, dev)
+    with pytest.raises(Exception, match="plan holds"):
+        rspmm_t_launcher(p, x, out, segs, segs_t, plan=plan[:plan.numel() // 2])
+
+
 def test_transposed_product_arguments_are_checked(dev):
     segs = A.create_acsr_segments([A.causal_windowed_pattern(64, 8)], 16, dev)
     segs_t = transposed_segments([A.causal_windowed_pattern(64, 8)], 16, dev)

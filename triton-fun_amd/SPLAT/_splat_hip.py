@@ -64,6 +64,8 @@ _SIGNATURES = {
     "splat_softmax_bwd": (ctypes.c_int, [_vp, _vp, _vp, ctypes.POINTER(AcsrSeg), _i32, _i64, _i32, _i32, _f32, _i32, _vp]),
     "splat_spmm_t": (ctypes.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, ctypes.POINTER(AcsrSeg), ctypes.POINTER(AcsrSeg), _i32, _i32,
                                    _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
+    "splat_spmm_t_planned": (ctypes.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, ctypes.POINTER(AcsrSeg), ctypes.POINTER(AcsrSeg), _i32,
+                                            _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _i64, _vp]),
     "splat_compressed_transpose": (ctypes.c_int, [_vp, _vp, ctypes.POINTER(AcsrSeg), ctypes.POINTER(AcsrSeg), _i32, _i64, _i32,
                                                   _i32, _i32, _i32, _i32, _vp]),
     "splat_attention_plan_bytes": (ctypes.c_int64, [ctypes.POINTER(AcsrSeg), _i32, _i32]),

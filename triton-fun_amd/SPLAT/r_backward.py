@@ -105,12 +105,24 @@ def compressed_transpose_launcher(src: torch.Tensor, dst: torch.Tensor, segments
     return dst
 
 
+def _rows_step_like_the_blocks(segments: ACSRSegments, segments_t: ACSRSegments) -> bool:
+    """Whether the kernel of thin wavefronts is the faster one for these masks: it reads a row's entries at a block of
+    output rows as consecutive slots when the row's column step equals the stride by which the transposed mask's rows are
+    grouped into blocks (1 for windows and blocks, the dilation for dilated windows); rows of another step (the far field
+    of a strided pattern) it walks a second time, entry by entry, which the general kernel does better."""
+    strides = {int(getattr(t[3], "splat_row_stride", 1)) for t in segments_t.tuples}
+    rs = strides.pop() if len(strides) == 1 else 1
+    return segments.max_step <= 1 or segments.max_step == rs
+
+
 def rspmm_t_launcher(p: torch.Tensor, x: torch.Tensor, out: torch.Tensor, segments: ACSRSegments,
-                     segments_t: ACSRSegments) -> torch.Tensor:
+                     segments_t: ACSRSegments, plan: torch.Tensor | None | bool = None) -> torch.Tensor:
     """out[.., j, :] = sum over the rows i that keep column j of p[.., i, slot of j in row i] * x[.., i, :], i.e. the
     product with the transposed compressed matrix: p [B, H, L, T] contiguous in the layout of ``segments``, x
     [B, H, L, n] with unit stride along n, out [B, H, Lt, n] contiguous; ``segments_t`` the ACSR of the transposed
-    segment masks."""
+    segment masks.  ``plan``: the plan table of the transposed mask (``segments_t.plan(Lt, device)``), which selects the
+    kernel of thin wavefronts where the library has one (16-bit types, n = 64 / 128, at least 512 blocks of 128 output
+    rows); None builds it on the first such call and keeps it with the metadata, False runs without."""
     for name, t in (("p", p), ("x", x), ("out", out)):
         _hip.require_device_tensor(t, name)
         if t.dim() != 4:
@@ -128,10 +140,25 @@ def rspmm_t_launcher(p: torch.Tensor, x: torch.Tensor, out: torch.Tensor, segmen
     dev = p.device
     a, b = _hip.seg_array(segments.seg_args(), L, T), _hip.seg_array(segments_t.seg_args(), Lt)
     xs = x.stride()
+    if plan is None and p.dtype in (torch.float16, torch.bfloat16) and out.dtype == p.dtype and n in (64, 128) \
+            and B * H * ((Lt + 127) // 128) >= 512 and _rows_step_like_the_blocks(segments, segments_t) \
+            and (segments_t.has_plan(Lt, dev) or not torch.cuda.is_current_stream_capturing()):
+        plan = segments_t.plan(Lt, dev)  # (no table is built under stream capture: building synchronises)
     with torch.cuda.device(dev):
-        rc = _hip.lib().splat_spmm_t(p.data_ptr(), x.data_ptr(), xs[0], xs[1], xs[2], out.data_ptr(), a, b, len(segments), B, H,
-                                     L, Lt, n, T, _hip.dtype_code(p.dtype), _hip.dtype_code(out.dtype), _hip.stream_ptr(dev))
-    _hip.check(rc, "splat_spmm_t")
+        if plan is not None and plan is not False:
+            _hip.require_device_tensor(plan, "plan")
+            if plan.device != dev:
+                raise _hip.SplatError(f"the plan lives on {plan.device}, the tensors on {dev}")
+            rc = _hip.lib().splat_spmm_t_planned(p.data_ptr(), x.data_ptr(), xs[0], xs[1], xs[2], out.data_ptr(), a, b,
+                                                 len(segments), B, H, L, Lt, n, T, _hip.dtype_code(p.dtype),
+                                                 _hip.dtype_code(out.dtype), plan.data_ptr(),
+                                                 plan.numel() * plan.element_size(), _hip.stream_ptr(dev))
+            _hip.check(rc, "splat_spmm_t_planned")
+        else:
+            rc = _hip.lib().splat_spmm_t(p.data_ptr(), x.data_ptr(), xs[0], xs[1], xs[2], out.data_ptr(), a, b, len(segments),
+                                         B, H, L, Lt, n, T, _hip.dtype_code(p.dtype), _hip.dtype_code(out.dtype),
+                                         _hip.stream_ptr(dev))
+            _hip.check(rc, "splat_spmm_t")
     return out
 
 

@@ -331,55 +331,6 @@ static int launch_spmm(SpmmParams p, hipStream_t st) {
 // its compressed row (consecutive slots when the row's column step is rs and its phase the block's) into an LDS tile
 // [i][m], zero where row i does not keep the column, and read back as the A operand with the transposing LDS read,
 // exactly as the x tile [i][feature] is read as the B operand.
-struct SpmmTParams {
-    const void* p;   // [BH, L, T] compressed, rows of the mask
-    const void* x;   // [B, H, L, n_out] by strides, unit stride along the features
-    void* out;       // [BH, Lt, n_out] contiguous
-    int64_t x_sb, x_sh, x_sl;
-    int B, H, L, Lt, n_out, T;
-    int out_dtype, out_vec, x_vec;
-    int n_seg;
-    SegPtrs seg[SPLAT_MAX_SEGMENTS];    // the mask: which columns row i keeps, and where
-    SegPtrs seg_t[SPLAT_MAX_SEGMENTS];  // the transposed mask: which rows column j meets
-    int n_row_blocks, total, n_col_chunks;
-    int row_stride;  // of the transposed mask's ACSR
-    int64_t p_elems;  // elements of p
-};
-
-// Row i's entries seen from a block of columns first + rs*m, m = 0..127.
-struct BlockRow {
-    RowWin w;  // unit step (lin == 1): live iff 0 <= m - lo < cnt, slot m - lo; lin > 1 (rs == 1 only): affine test in
-               // columns as in dense plans; lin == 0: the row fits neither and is tested per entry from its map
-    RowMap m;
-};
-__device__ __forceinline__ BlockRow block_row(const RowMap& m, int first, int rs) {
-    BlockRow b;
-    b.m = m;
-    b.w.lo = 0, b.w.cnt = 0, b.w.lin = 1;
-    if (m.cnt <= 0) return b;
-    const int d0 = m.a - first;
-    if (rs == 1) {
-        b.w.lo = d0;
-        b.w.lin = (m.cnt > 1) ? m.lin : 1;
-        b.w.cnt = b.w.lin * (m.cnt - 1) + 1;
-    } else if ((m.cnt == 1 || m.lin == rs) && d0 % rs == 0) {
-        b.w.lo = d0 / rs;
-        b.w.cnt = m.cnt;
-    } else {
-        b.w.lin = 0;
-    }
-    return b;
-}
-// the general test: entry of the row at column j, or zero
-template <typename T>
-__device__ __forceinline__ T entry_at_column(const T* row, const RowMap& m, int j) {
-    const int u = j - m.a;
-    if (u < 0 || m.cnt <= 0) return (T)0.f;
-    if (u == 0) return row[0];
-    if (m.cnt == 1 || u % m.lin != 0 || u / m.lin >= m.cnt) return (T)0.f;
-    return row[u / m.lin];
-}
-
 template <typename T, int DVT>
 __global__ __launch_bounds__(256, 2) void spmm_t_kernel(const SpmmTParams p) {
     constexpr int ES = sizeof(T);
@@ -649,10 +600,10 @@ extern "C" int splat_spmm_planned(const void* pp, const void* v, int64_t v_sb, i
                        out_dtype, plan, plan_bytes, stream);
 }
 
-extern "C" int splat_spmm_t(const void* pp, const void* x, int64_t x_sb, int64_t x_sh, int64_t x_sl, void* out,
-                            const splat_acsr_seg* segs, const splat_acsr_seg* segs_t, int32_t n_seg, int32_t B, int32_t H,
-                            int32_t L, int32_t Lt, int32_t n_out, int32_t T, int32_t in_dtype, int32_t out_dtype, void* stream) {
-    const char* who = "splat_spmm_t";
+static int spmm_t_common(const char* who, const void* pp, const void* x, int64_t x_sb, int64_t x_sh, int64_t x_sl, void* out,
+                         const splat_acsr_seg* segs, const splat_acsr_seg* segs_t, int32_t n_seg, int32_t B, int32_t H,
+                         int32_t L, int32_t Lt, int32_t n_out, int32_t T, int32_t in_dtype, int32_t out_dtype, const void* plan_t,
+                         int64_t plan_bytes, void* stream) {
     if (!pp || !x || !out || !segs || !segs_t) return fail(SPLAT_E_NULL, "%s: null pointer argument", who);
     if (B <= 0 || H <= 0 || L <= 0 || Lt <= 0 || n_out <= 0 || T <= 0)
         return fail(SPLAT_E_SHAPE, "%s: need B, H, L, Lt, n_out, T > 0 (got %d, %d, %d, %d, %d, %d)", who, B, H, L, Lt, n_out, T);
@@ -677,10 +628,37 @@ extern "C" int splat_spmm_t(const void* pp, const void* x, int64_t x_sb, int64_t
     p.x_vec = ((reinterpret_cast<uintptr_t>(x) & 15) == 0 && x_sb % epc == 0 && x_sh % epc == 0 && x_sl % epc == 0) ? 1 : 0;
     const int es_out = out_dtype == SPLAT_F32 ? 4 : 2;
     p.out_vec = ((reinterpret_cast<uintptr_t>(out) & 15) == 0 && ((int64_t)n_out * es_out) % 16 == 0) ? 1 : 0;
+    p.plan_t = nullptr;
+    if (plan_t) {
+        if ((reinterpret_cast<uintptr_t>(plan_t) & 15) != 0) return fail(SPLAT_E_ALIGN, "%s: the plan must be 16-byte aligned", who);
+        const int64_t need = splat_attention_plan_bytes(segs_t, n_seg, Lt);
+        if (need <= 0 || plan_bytes < need)
+            return fail(SPLAT_E_SHAPE, "%s: the plan holds %lld bytes, the transposed mask needs %lld", who, (long long)plan_bytes,
+                        (long long)need);
+        p.plan_t = static_cast<const PlanRec*>(plan_t);  // the variant with gathered walks comes first
+    }
     hipStream_t st = (hipStream_t)stream;
+    begin_launch();
+    if (const int rc = launch_spmm_t_thin(who, p, in_dtype, st)) return rc < 0 ? rc : check_launch(who);
     switch (in_dtype) {
         case SPLAT_F32: return launch_spmm_t<float>(p, st);
         case SPLAT_F16: return launch_spmm_t<f16>(p, st);
         default: return launch_spmm_t<bf16>(p, st);
     }
+}
+
+extern "C" int splat_spmm_t(const void* pp, const void* x, int64_t x_sb, int64_t x_sh, int64_t x_sl, void* out,
+                            const splat_acsr_seg* segs, const splat_acsr_seg* segs_t, int32_t n_seg, int32_t B, int32_t H,
+                            int32_t L, int32_t Lt, int32_t n_out, int32_t T, int32_t in_dtype, int32_t out_dtype, void* stream) {
+    return spmm_t_common("splat_spmm_t", pp, x, x_sb, x_sh, x_sl, out, segs, segs_t, n_seg, B, H, L, Lt, n_out, T, in_dtype,
+                         out_dtype, nullptr, 0, stream);
+}
+
+extern "C" int splat_spmm_t_planned(const void* pp, const void* x, int64_t x_sb, int64_t x_sh, int64_t x_sl, void* out,
+                                    const splat_acsr_seg* segs, const splat_acsr_seg* segs_t, int32_t n_seg, int32_t B,
+                                    int32_t H, int32_t L, int32_t Lt, int32_t n_out, int32_t T, int32_t in_dtype,
+                                    int32_t out_dtype, const void* plan_t, int64_t plan_bytes, void* stream) {
+    if (!plan_t) return fail(SPLAT_E_NULL, "splat_spmm_t_planned: null plan");
+    return spmm_t_common("splat_spmm_t_planned", pp, x, x_sb, x_sh, x_sl, out, segs, segs_t, n_seg, B, H, L, Lt, n_out, T,
+                         in_dtype, out_dtype, plan_t, plan_bytes, stream);
 }

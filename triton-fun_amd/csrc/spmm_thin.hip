@@ -37,43 +37,6 @@ struct ThinGeom {
     static constexpr int LDS_BYTES = PLANNED ? PLAN_AT : PLAN_AT + (int)sizeof(PlanScratch<BM>) + SPLAT_MAX_SEGMENTS * (int)sizeof(SegPlan);
 };
 
-// Physical 16-byte chunk of logical chunk c of V tile row `row`: the 64-byte block index is XORed with the row's low bits
-// (4 consecutive rows -> the 4 quadrants of the 256-byte bank space; for 128-byte rows two rows share a quadrant pair),
-// and the halves of a block swap places in every second group of 8 rows.  Its own inverse.
-template <int ROWB>
-__device__ __forceinline__ constexpr int v_chunk(int row, int c) {
-    const int blk = ROWB >= 256 ? (row & 3) : ((row >> 1) & 1);
-    return (((c >> 2) ^ blk) << 2) | ((c & 3) ^ (((row >> 3) & 1) << 1));
-}
-
-// x shifted by k 16-bit elements towards higher element indices (k >= 0) or lower ones (k < 0), zeros moving in
-__device__ __forceinline__ u32x4 shift_elements(u32x4 x, int k) {
-    const uint64_t lo = (uint64_t)x[0] | ((uint64_t)x[1] << 32), hi = (uint64_t)x[2] | ((uint64_t)x[3] << 32);
-    uint64_t rl, rh;
-    if (k >= 0) {
-        const int s = 16 * k;  // 0..128
-        if (s == 0) {
-            rl = lo, rh = hi;
-        } else if (s < 64) {
-            rl = lo << s, rh = (hi << s) | (lo >> (64 - s));
-        } else if (s < 128) {
-            rl = 0, rh = lo << (s - 64);
-        } else {
-            rl = 0, rh = 0;
-        }
-    } else {
-        const int s = -16 * k;
-        if (s < 64) {
-            rl = (lo >> s) | (hi << (64 - s)), rh = hi >> s;
-        } else if (s < 128) {
-            rl = hi >> (s - 64), rh = 0;
-        } else {
-            rl = 0, rh = 0;
-        }
-    }
-    return u32x4{(uint32_t)rl, (uint32_t)(rl >> 32), (uint32_t)rh, (uint32_t)(rh >> 32)};
-}
-
 // NB: register sets for probabilities in flight: requested NB steps (rings) or NB - 1 steps (straight from memory) ahead
 // RING: probabilities as whole aligned lines through per-row rings in LDS instead of per lane straight from memory;
 // STREAM: those lines with non-temporal loads
