@@ -585,8 +585,9 @@ def _spmm_case(mask, n_out, dtype, B=8, H=8, seed=51):
 @pytest.mark.parametrize("case", list(MANY_BLOCKS))
 def test_spmm_16_bit_in_launches_of_many_row_blocks(dev, case, dtype):
     """16-bit SpMM with 64 / 128 output columns and at least 512 row blocks: with the mask's plan table (the default unless
-    every row starts on a multiple of 8 positions) the kernel of thin wavefronts runs -- probabilities straight from
-    memory or through per-row rings, spans that end inside half steps, rows that are empty or hold one column, rows with
+    the rows are long and every one starts on a multiple of 8 positions) the kernels that start from it run -- rows of
+    fewer than 256 slots through a workgroup-wide tile, longer ones through per-row rings or, where they start on 16-byte
+    boundaries, straight from memory; spans that end inside half steps, rows that are empty or hold one column, rows with
     differing steps -- and must agree with the dense product; dead slots hold NaN and must not reach the output; the
     general kernel (plan=False) must agree too."""
     make, d = MANY_BLOCKS[case]

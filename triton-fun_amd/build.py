@@ -15,7 +15,7 @@ LIB_DIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIB_DIR, "libsplat_hip.so")
 BENCH_LIB = os.path.join(LIB_DIR, "libsplat_bench.so")
 
-SOURCES = ["api_common.cpp", "acsr_build.hip", "softmax.hip", "sddmm.hip", "sddmm_lines.hip", "spmm.hip", "spmm_thin.hip", "spmm_t_thin.hip", "attention.hip", "backward.hip", "attention_bwd.hip", "transpose.hip"]
+SOURCES = ["api_common.cpp", "acsr_build.hip", "softmax.hip", "sddmm.hip", "sddmm_lines.hip", "spmm.hip", "spmm_thin.hip", "spmm_tile.hip", "spmm_t_thin.hip", "attention.hip", "backward.hip", "attention_bwd.hip", "transpose.hip"]
 # the measurement aids: a library of their own, so that the operator ABI holds operators only
 BENCH_SOURCES = ["api_common.cpp", "bench_probes.hip"]
 # packed fp32 VALU forms are switched off for every device compile

@@ -1,4 +1,4 @@
-// Kernel arguments of the SpMM kernels (spmm.hip: every shape; spmm_thin.hip, spmm_t_thin.hip: 16-bit types, 64 / 128
+// Kernel arguments of the SpMM kernels (spmm.hip: every shape; spmm_thin.hip, spmm_tile.hip, spmm_t_thin.hip: 16-bit types, 64 / 128
 // output columns).
 #pragma once
 #include "acsr_plan.hpp"
@@ -24,6 +24,8 @@ struct SpmmParams {
 // Launches the kernel of thin wavefronts when the problem has its shape (see spmm_thin.hip); returns 1 when it did, 0
 // when the general kernel has to run, a negative code on errors.  `p` is complete except for the launch geometry.
 int launch_spmm_thin(const char* who, const SpmmParams& p, int in_dtype, hipStream_t st);
+// The same for rows that are short or not aligned (see spmm_tile.hip; launch_spmm_thin hands them over).
+int launch_spmm_tile(const char* who, const SpmmParams& p, int in_dtype, hipStream_t st);
 
 // ---- shared by the kernels of thin wavefronts ----
 // Physical 16-byte chunk of logical chunk c of V tile row `row`: the 64-byte block index is XORed with the row's low bits

@@ -1,16 +1,17 @@
-// SpMM on ACSR for the common fast shape: 16-bit probabilities, V and output of one type, 64 or 128 output columns,
-// 16-byte alignment, at least 512 row blocks in the launch.
+// SpMM on ACSR for 16-bit launches of many row blocks with long rows: probabilities, V and output of one type, 64 or 128
+// output columns, 16-byte alignment, at least 512 row blocks, rows of at least 256 slots that start on 16-byte boundaries
+// of the buffer, the mask's plan table.  (Shorter or unaligned rows: spmm_tile.hip.)
 //
 // A workgroup of 8 wavefronts owns 128 rows of one (batch, head); wavefront w owns rows 16w..16w+15 and accumulates
 // O^T = V^T P^T with 16x16x32 MFMAs (rows = output columns, columns = queries: a lane owns one query row).  Thin
 // wavefronts stay below 128 registers, so that four of them share a SIMD and cover each other's waits.
 //
 // The B operand needs, per lane, 8 consecutive key positions of the lane's own row: with a uniform plan these are 8
-// consecutive compressed slots, one 16-byte load (any alignment) straight from the compressed row into registers, a
-// step ahead; nothing of the compressed matrix passes through LDS.  Where the 32 positions of a half step are not inside
-// the span of every row of the wavefront, a lane loads the 8 slots at its row's nearer end instead (inside the row,
-// whatever lies beyond is never read) and shifts and masks them in registers.  Other plans walk dense columns and gather
-// element by element under the row's affine test.
+// consecutive compressed slots.  A wavefront fetches its rows' slots as whole aligned 128-byte lines (non-temporal where the
+// compressed matrix is larger than the last-level cache), two steps ahead through registers into per-row rings of two
+// lines in LDS, and every fragment is the funnel shift of two aligned 16-byte chunks of the lane's ring.  A wavefront
+// whose rows all start on multiples of 8 positions (blocked masks) skips the rings: its fragments are aligned 16-byte
+// loads straight from memory.  Other plans walk dense columns and gather element by element under the row's affine test.
 //
 // V tiles of 64 keys go through registers into one of two LDS stages (written a step ahead, one barrier per step), 64-byte
 // blocks and their halves permuted so that the transposing reads of the A operand -- a lane block reads 4 key rows x
@@ -23,7 +24,7 @@
 
 namespace splat {
 
-template <int D, bool PLANNED, bool RING>
+template <int D>
 struct ThinGeom {
     static constexpr int BM = 128;
     static constexpr int ROWB = D * 2;            // bytes per V row
@@ -33,28 +34,24 @@ struct ThinGeom {
     static constexpr int TILE_BYTES = 2 * STAGE > BM * O_ROW ? 2 * STAGE : BM * O_ROW;
     static constexpr int R_ROW = 128 * 2 + 16;     // bytes per row of the probability rings: two lines of 64 slots
     static constexpr int RING_AT = TILE_BYTES;
-    static constexpr int PLAN_AT = RING_AT + (RING ? BM * R_ROW : 0);
-    static constexpr int LDS_BYTES = PLANNED ? PLAN_AT : PLAN_AT + (int)sizeof(PlanScratch<BM>) + SPLAT_MAX_SEGMENTS * (int)sizeof(SegPlan);
+    static constexpr int LDS_BYTES = RING_AT + BM * R_ROW;
 };
 
 // NB: register sets for probabilities in flight: requested NB steps (rings) or NB - 1 steps (straight from memory) ahead
-// RING: probabilities as whole aligned lines through per-row rings in LDS instead of per lane straight from memory;
-// STREAM: those lines with non-temporal loads
-template <typename T, int D, int NB, bool PLANNED, bool RING, bool STREAM>
+// STREAM: the rings' lines with non-temporal loads
+template <typename T, int D, int NB, bool STREAM>
 __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
-    using G = ThinGeom<D, PLANNED, RING>;
+    using G = ThinGeom<D>;
     constexpr int R_ROW = G::R_ROW;
     constexpr int BM = G::BM, ROWB = G::ROWB, STAGE = G::STAGE, O_ROW = G::O_ROW;
     constexpr int CPR = ROWB / 16;        // 16-byte chunks per V row
     constexpr int NI = kBN * CPR / 512;   // chunks of a V tile per thread
     constexpr int DT = D / 16;            // 16-column blocks of the output
-    static_assert(NI >= 1 && G::PLAN_AT % 16 == 0, "tile shape");
+    static_assert(NI >= 1 && G::RING_AT % 16 == 0, "tile shape");
 
     extern __shared__ __attribute__((aligned(1024))) char smem[];
     char* const s_v = smem;
     char* const s_rings = smem + G::RING_AT;
-    PlanScratch<BM>* const s_ps = reinterpret_cast<PlanScratch<BM>*>(smem + G::PLAN_AT);
-    SegPlan* const s_plan = reinterpret_cast<SegPlan*>(s_ps + 1);
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -73,7 +70,6 @@ __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
     const int64_t v_rowb = p.v_sl * 2;
     const T* pb = (const T*)p.p + (int64_t)bh * L * p.T;
 
-    if constexpr (!PLANNED) plan_segments<BM>(p.seg, p.n_seg, r0, rs, L, true, s_plan, s_ps, tid);
     const PlanRec* const pt = p.plan;
     const int n_rb = p.n_row_blocks;
 
@@ -108,11 +104,9 @@ __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
 
     for (int sg = 0; sg < p.n_seg; ++sg) {
         SegPlan pl;
-        if constexpr (PLANNED) {
+        {
             const PlanRec r = plan_uniform_load(pt + plan_seg_at(p.n_seg, rb, sg));
             pl = SegPlan{r[0], r[1], r[2], r[3]};
-        } else {
-            pl = s_plan[sg];
         }
         const int n_steps = pl.n_tiles;
         if (n_steps == 0) continue;  // workgroup-uniform
@@ -120,22 +114,18 @@ __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
         const bool uniform = pl.uniform != 0;
 
         RowWin mine;
-        if constexpr (PLANNED) {
+        {
             // (counts are clamped to the slots the segment owns in this buffer, like the ones read from the metadata)
             const PlanRec r = pt[plan_row_at(n_rb, p.n_seg, rb, sg, my_rr)];
             const int64_t most = uniform ? (int64_t)p.seg[sg].max_cnt : (int64_t)r[2] * (p.seg[sg].max_cnt - 1) + 1;
             mine = RowWin{r[0], (int)min((int64_t)r[1], most), r[2]};
-        } else {
-            mine = make_row_win(cached_row_map<BM>(s_ps, sg, my_rr), pl);
         }
         if (my_r >= L) mine.cnt = 0;
         WaveSpan span;
-        if constexpr (PLANNED) {
+        {
             // the table holds the spans of 32 rows: wider than this wavefront's 16, which only makes the tests below pass less often
             const PlanRec r = plan_uniform_load(pt + plan_span_at(n_rb, p.n_seg, rb, sg, wave >> 1));
             span = WaveSpan{r[0], r[1], r[2], r[3]};
-        } else {
-            span = wave_span(mine, uniform);
         }
         const int lmin = span.lo_min, hmax = span.hi_max;
         const T* const prow = pb + (int64_t)min(my_r, L - 1) * p.T + off;
@@ -146,7 +136,7 @@ __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
         // has all of them.
         auto act = [&](int pos0) { return !(pos0 + 32 <= lmin || pos0 >= hmax); };
         auto full = [&](int pos0) { return pos0 >= span.lo_max && pos0 + 32 <= span.hi_min; };
-        // ---- RING: the rows whose lines this lane fetches (8 lanes per row, 8 rows per instruction: two instructions
+        // ---- rings: the rows whose lines this lane fetches (8 lanes per row, 8 rows per instruction: two instructions
         // cover the wavefront's 16 rows; the two rows of 16 consecutive lanes are 8 apart, half the banks apart in the ring)
         // Step t needs slots 64 t - lo .. + 63 of a row, which lie in lines t + la and t + la + 1 (la = -ceil(lo / 64), a
         // line = 64 slots from the row's first): line t + la + 1 is requested NB steps ahead, written into the ring (line
@@ -154,22 +144,15 @@ __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
         int f_rr[2], f_la[2], f_cnt[2];
         const T* f_row[2];
         const int f_piece = lane & 7;
-        if constexpr (RING) {
 #pragma unroll
-            for (int c = 0; c < 2; ++c) {
-                f_rr[c] = 16 * wave + 4 * c + (lane >> 4) + 8 * ((lane >> 3) & 1);
-                RowWin w;
-                if constexpr (PLANNED) {
-                    const PlanRec r = pt[plan_row_at(n_rb, p.n_seg, rb, sg, f_rr[c])];
-                    w = RowWin{r[0], min(r[1], p.seg[sg].max_cnt), r[2]};
-                } else {
-                    w = make_row_win(cached_row_map<BM>(s_ps, sg, f_rr[c]), pl);
-                }
-                const int r = r0 + rs * f_rr[c];
-                f_la[c] = -((w.lo + 63) >> 6);
-                f_cnt[c] = (r < L && uniform) ? w.cnt : 0;
-                f_row[c] = pb + (int64_t)min(r, L - 1) * p.T + off;
-            }
+        for (int c = 0; c < 2; ++c) {
+            f_rr[c] = 16 * wave + 4 * c + (lane >> 4) + 8 * ((lane >> 3) & 1);
+            const PlanRec rec = pt[plan_row_at(n_rb, p.n_seg, rb, sg, f_rr[c])];
+            const RowWin w = RowWin{rec[0], min(rec[1], p.seg[sg].max_cnt), rec[2]};
+            const int r = r0 + rs * f_rr[c];
+            f_la[c] = -((w.lo + 63) >> 6);
+            f_cnt[c] = (r < L && uniform) ? w.cnt : 0;
+            f_row[c] = pb + (int64_t)min(r, L - 1) * p.T + off;
         }
         // the 16 bytes of line t + la + 1 this lane fetches for row c (zeros where the line has nothing of the row)
         auto load_line = [&](int t, int c) {
@@ -291,7 +274,7 @@ __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
         // ---- prologue: V tile 0 into stage 0, V tile 1 and the probabilities of the first steps requested
         // Rings pay where rows start inside a 16-byte chunk of their positions' grid; a wavefront whose rows all start on
         // one (blocked masks) reads its aligned chunks straight from memory.  Wavefront-uniform: the rings are private.
-        const bool ring = RING && uniform && __any((mine.lo & 7) != 0 && mine.cnt > 0);
+        const bool ring = uniform && __any((mine.lo & 7) != 0 && mine.cnt > 0);
         u32x4 vreg[NI];
         u32x4 praw[NB][2];  // [step modulo NB][half (direct loads) or row (rings)]
         load_v(0, vreg);
@@ -337,9 +320,6 @@ __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
                 }
                 praw[ri][0] = load_line(s + NB, 0);
                 praw[ri][1] = load_line(s + NB, 1);
-            } else if (!RING) {
-                praw[rn][0] = load_p((s + NB - 1) * kBN);  // (nothing is read of steps past the last one: they are not active)
-                praw[rn][1] = load_p((s + NB - 1) * kBN + 32);
             }
 #pragma unroll
             for (int hf = 0; hf < 2; ++hf) {
@@ -353,7 +333,7 @@ __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
                     mma16(acc[dt], vf, pf);
                 }
             }
-            if (RING && !ring) {  // (kept out of the way of the ring path's schedule: after the products)
+            if (!ring) {  // (kept out of the way of the ring path's schedule: after the products; nothing is read of steps past the last one: they are not active)
                 praw[rn][0] = load_p((s + NB - 1) * kBN);
                 praw[rn][1] = load_p((s + NB - 1) * kBN + 32);
             }
@@ -362,7 +342,7 @@ __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
         // the unrolled steps make the stage (s % 2) and the register set (s % NB) compile-time constants
         // (straight from memory, a half step may look at what was requested for the next step; with rings that path only
         // serves wavefronts whose rows start on 16-byte boundaries, which never do)
-        static_assert(NB >= (RING ? 2 : 3), "register sets");
+        static_assert(NB >= 2, "register sets");
         constexpr int UNROLL = NB % 2 == 0 ? NB : 2 * NB;
         for (int s = 0; s < n_steps; s += UNROLL) {
             static_for<UNROLL>([&](auto u) {
@@ -395,9 +375,9 @@ __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
     }
 }
 
-template <typename T, int D, bool PLANNED, bool RING, bool STREAM>
+template <typename T, int D, bool STREAM>
 static int launch_thin_variant(const char* who, SpmmParams p, hipStream_t st) {
-    using G = ThinGeom<D, PLANNED, RING>;
+    using G = ThinGeom<D>;
     static_assert(G::LDS_BYTES <= 80 * 1024, "two workgroups per compute unit");
     p.n_row_blocks = count_row_blocks(p.L, G::BM, p.row_stride);
     p.n_col_chunks = 1;
@@ -405,8 +385,8 @@ static int launch_thin_variant(const char* who, SpmmParams p, hipStream_t st) {
     if (blocks > 0x7ffffff0) return 0;
     p.total = (int)blocks;
     static uint64_t reserved = 0;
-    // (d = 128 with rings: a third set would spill)
-    auto kern = spmm_thin_kernel<T, D, D == 128 ? (RING ? 2 : 3) : 4, PLANNED, RING, STREAM>;
+    // (d = 128: a third set would spill)
+    auto kern = spmm_thin_kernel<T, D, D == 128 ? 2 : 4, STREAM>;
     if (int rc = reserve_dynamic_lds(&reserved, reinterpret_cast<const void*>(kern), G::LDS_BYTES, who)) return rc;
     const int grid = ((p.total + 7) / 8) * 8;
     kern<<<grid, 512, G::LDS_BYTES, st>>>(p);
@@ -422,25 +402,19 @@ int launch_spmm_thin(const char* who, const SpmmParams& p, int in_dtype, hipStre
     for (int k = 0; k < p.n_seg; ++k)
         if (p.seg[k].max_cnt < 8) return 0;
     if ((int64_t)p.B * p.H * count_row_blocks(p.L, 128, p.row_stride) < 512) return 0;
-    // rings: rows of the compressed matrix start on 16-byte boundaries
-    // (and long: rows of one or two lines are better off without)
+    // rings: rows of the compressed matrix start on 16-byte boundaries and are long (rows of one or two lines are better
+    // off with the workgroup-wide tile of spmm_tile.hip, and so are rows anywhere else)
     bool ring = (reinterpret_cast<uintptr_t>(p.p) & 15) == 0 && p.T % 8 == 0 && p.T >= 256;
     for (int k = 0; k < p.n_seg; ++k)
         if (p.seg[k].slot_offset % 8 != 0) ring = false;
+    if (!ring) return launch_spmm_tile(who, p, in_dtype, st);
     // a compressed matrix too large for the 256 MB last-level cache streams past the L2, where V stays (config 4's 537 MB:
     // -9 % with non-temporal loads; config 2's 134 MB, which repeated launches find in that cache: +5 %)
     const bool stream = (int64_t)p.B * p.H * p.L * p.T * 2 > ((int64_t)192 << 20);
-    auto go = [&](auto t, auto d_c, auto planned_c) {
-        using TT = decltype(t);
-        constexpr int DD = decltype(d_c)::value;
-        constexpr bool PL = decltype(planned_c)::value;
-        if (ring && stream) return launch_thin_variant<TT, DD, PL, true, true>(who, p, st);
-        if (ring) return launch_thin_variant<TT, DD, PL, true, false>(who, p, st);
-        return launch_thin_variant<TT, DD, PL, false, false>(who, p, st);
-    };
-    auto by_plan = [&](auto t, auto d_c) { return go(t, d_c, std::true_type{}); };
     auto by_d = [&](auto t) {
-        return p.n_out == 128 ? by_plan(t, std::integral_constant<int, 128>{}) : by_plan(t, std::integral_constant<int, 64>{});
+        using TT = decltype(t);
+        if (p.n_out == 128) return stream ? launch_thin_variant<TT, 128, true>(who, p, st) : launch_thin_variant<TT, 128, false>(who, p, st);
+        return stream ? launch_thin_variant<TT, 64, true>(who, p, st) : launch_thin_variant<TT, 64, false>(who, p, st);
     };
     return in_dtype == SPLAT_BF16 ? by_d(bf16{}) : by_d(f16{});
 }
