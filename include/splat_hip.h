@@ -172,8 +172,8 @@ int splat_spmm(const void* p, const void* v, int64_t v_sb, int64_t v_sh, int64_t
 
 /* splat_spmm with the mask's plan table (`plan` as in splat_sddmm_planned).  For 16-bit types, 64 or 128 output columns and
  * launches of at least 512 row blocks this runs kernels of thin wavefronts (four per SIMD) that start from the table --
- * rows of at least 256 slots on 16-byte boundaries through per-row rings of aligned lines, shorter or unaligned rows
- * through a workgroup-wide tile: -20 % at B=2 H=32 L=8192 d=128 T=512, -23 % at B=4 H=16 L=4096 d=64 T=256, -40 % on rows
+ * rows of at least 256 slots on 16-byte boundaries in compressed matrices of more than 192 MB through per-row rings of
+ * aligned lines, everything else through a workgroup-wide tile: -20 % at B=2 H=32 L=8192 d=128 T=512, -23 % at B=4 H=16 L=4096 d=64 T=256, -40 % on rows
  * of 64 slots; masks of at least 256 slots per row whose rows all start on multiples of 8 positions of their block's walk
  * (blocked masks with large blocks) are better served by splat_spmm (the Python launcher looks that up in the table once
  * and picks).  Other shapes ignore the plan.  Same results as

@@ -649,6 +649,46 @@ def test_spmm_with_a_plan_forced_on_an_aligned_mask_and_two_segments(dev):
     assert float((got2 - want2).abs().max()) <= 2 * TOL[torch.float16]
 
 
+@pytest.mark.parametrize("case", ["dilated512x2_d128_bf16", "causal511_d64_f16", "blocked512_d128_bf16"])
+def test_spmm_rings_on_a_compressed_matrix_larger_than_the_last_level_cache(dev, case):
+    """Rows of at least 256 slots on 16-byte boundaries and more than 192 MB of probabilities (here 268 MB) take the kernel of
+    per-row rings, whose lines are loaded non-temporally; on a blocked mask (the table passed by hand: the launcher would
+    pick the general kernel) its wavefronts read aligned chunks straight from memory.  Against the general kernel over the
+    whole output and against the dense product for two (batch, head) pairs; dead slots hold NaN."""
+    make, d, dtype = {"dilated512x2_d128_bf16": (lambda: O.create_dilated_mask(4096, 512, 2), 128, torch.bfloat16),
+                      "causal511_d64_f16": (lambda: O.create_causal_windowed_mask(4096, 511), 64, torch.float16),
+                      "blocked512_d128_bf16": (lambda: O.create_blocked_mask(4096, 256), 128, torch.bfloat16)}[case]
+    mask = make()
+    L, B, H = mask.shape[0], 8, 8
+    acsr_np = O.create_acsr(mask, 16)
+    cols, valid = O.slot_columns(acsr_np, first_col=O.row_extents(mask)[0])
+    T = cols.shape[-1]
+    assert T == 512 and B * H * L * T * 2 > (192 << 20)
+    lv = torch.from_numpy(valid).to(dev)
+    g = torch.Generator(device=dev).manual_seed(71)
+    pr = torch.rand(B, H, L, T, generator=g, device=dev)
+    pr = pr / torch.where(lv, pr, torch.zeros((), device=dev)).sum(-1, keepdim=True).clamp(min=1e-9)
+    pr = torch.where(lv, pr, torch.full((), float("nan"), device=dev)).to(dtype)
+    v = torch.randn(B, H, L, d, generator=g, device=dev).to(dtype)
+    acsr = A.create_acsr(mask, 16, dev)
+    segs = A.ACSRSegments.single(acsr[0], acsr[1], acsr[2], acsr[3], acsr[4], T)
+    outs = []
+    for plan in (segs.plan(L, dev), False):
+        out = torch.full((B, H, L, d), 7.0, dtype=dtype, device=dev)
+        r_spmm.rspmm_launcher(pr, v, out, acsr[0], acsr[1], acsr[2], acsr[3], acsr[6], acsr[7], T, acsr[4],
+                              (1, 1, 1), 16, 16, plan=plan)
+        assert torch.isfinite(out).all()
+        outs.append(out.float())
+    assert float((outs[0] - outs[1]).abs().max()) <= TOL[dtype]
+    rows_i, slots_i = np.nonzero(valid)
+    ri, si = torch.from_numpy(rows_i).to(dev), torch.from_numpy(slots_i).to(dev)
+    ci = torch.from_numpy(cols[rows_i, slots_i].astype(np.int64)).to(dev)
+    for b, h in ((0, 0), (B - 1, H - 1)):
+        dense = torch.zeros(L, L, device=dev)
+        dense[ri, ci] = pr[b, h].float()[ri, si]
+        assert float((outs[0][b, h] - dense @ v[b, h].float()).abs().max()) <= TOL[dtype]
+
+
 def test_comparison_sweeps_run_and_agree_with_dense(dev):
     """The sweep harness (successor of the reference's comparison.py:76-106) at toy size: one record per doubling of
     the sparsity parameter, nnz as the pattern's closed form, fused forward equal to dense attention with the same mask."""

@@ -1,14 +1,15 @@
-// SpMM on ACSR for 16-bit launches of many row blocks with long rows: probabilities, V and output of one type, 64 or 128
-// output columns, 16-byte alignment, at least 512 row blocks, rows of at least 256 slots that start on 16-byte boundaries
-// of the buffer, the mask's plan table.  (Shorter or unaligned rows: spmm_tile.hip.)
+// SpMM on ACSR for 16-bit launches of many row blocks with long rows and a compressed matrix larger than the last-level
+// cache: probabilities, V and output of one type, 64 or 128 output columns, 16-byte alignment, at least 512 row blocks,
+// rows of at least 256 slots that start on 16-byte boundaries of the buffer, more than 192 MB of probabilities, the mask's
+// plan table.  (Everything else with a plan table: spmm_tile.hip.)
 //
 // A workgroup of 8 wavefronts owns 128 rows of one (batch, head); wavefront w owns rows 16w..16w+15 and accumulates
 // O^T = V^T P^T with 16x16x32 MFMAs (rows = output columns, columns = queries: a lane owns one query row).  Thin
 // wavefronts stay below 128 registers, so that four of them share a SIMD and cover each other's waits.
 //
 // The B operand needs, per lane, 8 consecutive key positions of the lane's own row: with a uniform plan these are 8
-// consecutive compressed slots.  A wavefront fetches its rows' slots as whole aligned 128-byte lines (non-temporal where the
-// compressed matrix is larger than the last-level cache), two steps ahead through registers into per-row rings of two
+// consecutive compressed slots.  A wavefront fetches its rows' slots as whole aligned 128-byte lines (non-temporal: they
+// stream past the L2, where V stays), two steps ahead through registers into per-row rings of two
 // lines in LDS, and every fragment is the funnel shift of two aligned 16-byte chunks of the lane's ring.  A wavefront
 // whose rows all start on multiples of 8 positions (blocked masks) skips the rings: its fragments are aligned 16-byte
 // loads straight from memory.  Other plans walk dense columns and gather element by element under the row's affine test.
@@ -38,8 +39,7 @@ struct ThinGeom {
 };
 
 // NB: register sets for probabilities in flight: requested NB steps (rings) or NB - 1 steps (straight from memory) ahead
-// STREAM: the rings' lines with non-temporal loads
-template <typename T, int D, int NB, bool STREAM>
+template <typename T, int D, int NB>
 __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
     using G = ThinGeom<D>;
     constexpr int R_ROW = G::R_ROW;
@@ -159,11 +159,8 @@ __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
             u32x4 raw = {0u, 0u, 0u, 0u};
             const int slot = 64 * (t + f_la[c] + 1) + 8 * f_piece;
             if (slot >= 0 && slot < f_cnt[c]) {  // 16-byte aligned
-                // a compressed matrix too large for the last-level cache streams past the L2, where V stays
-                if constexpr (STREAM)
-                    raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(f_row[c] + slot));
-                else
-                    raw = *reinterpret_cast<const u32x4*>(f_row[c] + slot);
+                // (this kernel's compressed matrices are too large for the last-level cache: they stream past the L2, where V stays)
+                raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(f_row[c] + slot));
             }
             return raw;
         };
@@ -375,7 +372,7 @@ __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
     }
 }
 
-template <typename T, int D, bool STREAM>
+template <typename T, int D>
 static int launch_thin_variant(const char* who, SpmmParams p, hipStream_t st) {
     using G = ThinGeom<D>;
     static_assert(G::LDS_BYTES <= 80 * 1024, "two workgroups per compute unit");
@@ -386,7 +383,7 @@ static int launch_thin_variant(const char* who, SpmmParams p, hipStream_t st) {
     p.total = (int)blocks;
     static uint64_t reserved = 0;
     // (d = 128: a third set would spill)
-    auto kern = spmm_thin_kernel<T, D, D == 128 ? 2 : 4, STREAM>;
+    auto kern = spmm_thin_kernel<T, D, D == 128 ? 2 : 4>;
     if (int rc = reserve_dynamic_lds(&reserved, reinterpret_cast<const void*>(kern), G::LDS_BYTES, who)) return rc;
     const int grid = ((p.total + 7) / 8) * 8;
     kern<<<grid, 512, G::LDS_BYTES, st>>>(p);
@@ -402,19 +399,19 @@ int launch_spmm_thin(const char* who, const SpmmParams& p, int in_dtype, hipStre
     for (int k = 0; k < p.n_seg; ++k)
         if (p.seg[k].max_cnt < 8) return 0;
     if ((int64_t)p.B * p.H * count_row_blocks(p.L, 128, p.row_stride) < 512) return 0;
-    // rings: rows of the compressed matrix start on 16-byte boundaries and are long (rows of one or two lines are better
-    // off with the workgroup-wide tile of spmm_tile.hip, and so are rows anywhere else)
-    bool ring = (reinterpret_cast<uintptr_t>(p.p) & 15) == 0 && p.T % 8 == 0 && p.T >= 256;
+    // Rings: rows of the compressed matrix start on 16-byte boundaries, are long, and the matrix is too large for the 256 MB
+    // last-level cache, so that whole lines fetched with non-temporal loads stream past the L2, where V stays (config 4's
+    // 537 MB: 0.184 ms against 0.218 for the workgroup-wide tile of spmm_tile.hip).  A matrix that repeated launches find in
+    // that cache (config 2's 134 MB), rows of one or two lines and rows anywhere else are better off with the tile (-7 to
+    // -10 %).
+    bool ring = (reinterpret_cast<uintptr_t>(p.p) & 15) == 0 && p.T % 8 == 0 && p.T >= 256 &&
+                (int64_t)p.B * p.H * p.L * p.T * 2 > ((int64_t)192 << 20);
     for (int k = 0; k < p.n_seg; ++k)
         if (p.seg[k].slot_offset % 8 != 0) ring = false;
     if (!ring) return launch_spmm_tile(who, p, in_dtype, st);
-    // a compressed matrix too large for the 256 MB last-level cache streams past the L2, where V stays (config 4's 537 MB:
-    // -9 % with non-temporal loads; config 2's 134 MB, which repeated launches find in that cache: +5 %)
-    const bool stream = (int64_t)p.B * p.H * p.L * p.T * 2 > ((int64_t)192 << 20);
     auto by_d = [&](auto t) {
         using TT = decltype(t);
-        if (p.n_out == 128) return stream ? launch_thin_variant<TT, 128, true>(who, p, st) : launch_thin_variant<TT, 128, false>(who, p, st);
-        return stream ? launch_thin_variant<TT, 64, true>(who, p, st) : launch_thin_variant<TT, 64, false>(who, p, st);
+        return p.n_out == 128 ? launch_thin_variant<TT, 128>(who, p, st) : launch_thin_variant<TT, 64>(who, p, st);
     };
     return in_dtype == SPLAT_BF16 ? by_d(bf16{}) : by_d(f16{});
 }
