@@ -208,46 +208,26 @@ __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
 #pragma unroll
             for (int i = 0; i < NI; ++i) *reinterpret_cast<u32x4*>(s_v + stage * STAGE + v_lds[i]) = reg[i];
         };
-        // A 16-byte load that starts on an odd 2-byte boundary takes twice as long as one on a 4-byte boundary.  A lane
-        // whose slots start there loads from one element earlier and takes the element it lacks, the last of its 8, from
-        // the lane that holds the next 8 positions of the row (16 lanes on, or lane % 16 of the next half step): `odd`.
-        const bool odd = ((reinterpret_cast<uintptr_t>(prow) >> 1) + (unsigned)(8 * g4 - mine.lo)) & 1u;
-        // The 8 entries at positions pos0 + 8 g4 .. + 7 of this lane's row as they come from memory (uniform plans): the
-        // slots themselves (from an even boundary) where the half step is full, else the 8 slots of the row nearest to them.
+        // Straight from memory (wavefronts whose rows all start on multiples of 8 positions: every piece is 16-byte aligned): the
+        // 8 entries at positions pos0 + 8 g4 .. + 7 of this lane's row as they come from memory -- the slots themselves where
+        // the half step is full, else the 8 slots of the row nearest to them.
         auto load_p = [&](int pos0) {
             u32x4 raw = {0u, 0u, 0u, 0u};
             if (!uniform || !act(pos0)) return raw;
             const int u = pos0 + 8 * g4 - mine.lo;
             if (full(pos0)) {
-                __builtin_memcpy(&raw, prow + (u - (odd ? 1 : 0)), 16);
+                __builtin_memcpy(&raw, prow + u, 16);
             } else {
                 const int uc = min(max(u, 0), max(min(mine.cnt - 8, row_last8), 0));
                 __builtin_memcpy(&raw, prow + uc, 16);
             }
             return raw;
         };
-        // ... and as the B operand wants them: entry e is slot u + e, zero outside the row's span (`next0`: what load_p
-        // returned for the next half step)
-        auto fix_p = [&](u32x4 raw, const u32x4& next0, int pos0) {
+        // ... and as the B operand wants them: entry e is slot u + e, zero outside the row's span
+        auto fix_p = [&](u32x4 raw, int pos0) {
             Frag<T> f;
             if (uniform) {
-                if (full(pos0)) {
-                    if (__any(odd)) {
-                        uint32_t x4;
-                        if (full(pos0 + 32)) {  // wavefront-uniform
-                            const uint32_t mine0 = g4 == 0 ? next0[0] : raw[0];  // what the lane 16 lanes back takes
-                            x4 = (uint32_t)__shfl((int)mine0, (lane + 16) & 63);
-                        } else {  // the next half step was not loaded that way: the element itself
-                            const int u = pos0 + 8 * g4 - mine.lo;
-                            x4 = *reinterpret_cast<const uint16_t*>(prow + u + 7);
-                        }
-                        const uint32_t sh = odd ? 16u : 0u;
-                        raw[0] = __builtin_amdgcn_alignbit(raw[1], raw[0], sh);
-                        raw[1] = __builtin_amdgcn_alignbit(raw[2], raw[1], sh);
-                        raw[2] = __builtin_amdgcn_alignbit(raw[3], raw[2], sh);
-                        raw[3] = __builtin_amdgcn_alignbit(x4, raw[3], sh);
-                    }
-                } else if (!full(pos0)) {
+                if (!full(pos0)) {
                     const int u = pos0 + 8 * g4 - mine.lo;
                     const int uc = min(max(u, 0), max(min(mine.cnt - 8, row_last8), 0));
                     raw = shift_elements(raw, uc - u);
@@ -322,7 +302,7 @@ __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
             for (int hf = 0; hf < 2; ++hf) {
                 const int pos0 = s * kBN + 32 * hf;
                 if (!act(pos0)) continue;  // wavefront-uniform
-                const Frag<T> pf = ring ? ring_frag(pos0) : fix_p(praw[ri][hf], hf == 0 ? praw[ri][1] : praw[(ri + 1) % NB][0], pos0);
+                const Frag<T> pf = ring ? ring_frag(pos0) : fix_p(praw[ri][hf], pos0);
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
                     const char* a = s_v + v_off[dt] + (par * STAGE + 32 * hf * ROWB);
@@ -337,8 +317,6 @@ __global__ __launch_bounds__(512, 4) void spmm_thin_kernel(const SpmmParams p) {
             lds_barrier();
         };
         // the unrolled steps make the stage (s % 2) and the register set (s % NB) compile-time constants
-        // (straight from memory, a half step may look at what was requested for the next step; with rings that path only
-        // serves wavefronts whose rows start on 16-byte boundaries, which never do)
         static_assert(NB >= 2, "register sets");
         constexpr int UNROLL = NB % 2 == 0 ? NB : 2 * NB;
         for (int s = 0; s < n_steps; s += UNROLL) {
