@@ -460,7 +460,7 @@ def main() -> int:
         ms_c0 = sum(pr) / len(pr)
         extras["backward_cfg4"] = {"ms": round(ms_f, 4), "tflops_nnz": round(fl4 / ms_f / 1e9, 2),
                                    "x_fused_forward": round(ms_f / extras["fused_cfg4"]["ms"], 2),
-                                   "kernel": "splat_attention_bwd: row sums + three launches of attn_bwd_kernel, no compressed matrix",
+                                   "kernel": "splat_attention_bwd: three launches of attn_bwd_kernel (the first also computes the row sums of dO * O), no compressed matrix",
                                    "composed_ms_with_forward_lse": round(ms_c, 3), "composed_ms": round(ms_c0, 3)}
         del out4, lse4
         del attn4, g4, q4, k4, v4

@@ -12,8 +12,9 @@
 //   dK    keys     queries    K, V             Q        dO       the same with the mask's transpose
 //   dV    keys     queries    K                Q        dO       S^T = X A^T; P;                 acc^T += Y^T P^T
 //
-// dQ walks the mask's own plan, dK and dV the plan of the transposed mask (keys as rows).  lse and D belong to the
-// queries: one value per lane in dQ, one per tile position otherwise (64 floats each per tile, copied into LDS beside
+// dQ walks the mask's own plan, dK and dV the plan of the transposed mask (keys as rows).  The dQ launch comes first: its
+// lanes hold their dO rows, so it also computes D (one more read of the lane's O row) and stores it for the other two.  lse
+// and D belong to the queries: one value per lane in dQ, one per tile position otherwise (64 floats each per tile, copied into LDS beside
 // the tiles).  The X tile of dQ / dK is read row-wise (16-byte fragments for S^T) and through the transposing read
 // (for acc^T), hence the swizzle that serves both (tile_copy.hpp: dual_chunk).  Probabilities come straight from the
 // statistic: no running maximum, no rescale, no second pass.  16-bit types, d = 64 or 128, rows of every operand
@@ -34,7 +35,10 @@ struct BwdParams {
     void* out;      // dQ, dK, dV
     int64_t a_sb, a_sh, a_sl, b_sb, b_sh, b_sl, x_sb, x_sh, x_sl, y_sb, y_sh, y_sl, o_sb, o_sh, o_sl;
     const float* lse;    // [B*H, L], natural log, per query
-    const float* delta;  // [B*H, L], D per query
+    const float* delta;  // [B*H, L], D per query (dK, dV: written by the dQ launch before them on the stream)
+    const void* o;       // dQ only: the forward's output, from which that launch computes D = rowsum(dO * O) ...
+    int64_t oo_sb, oo_sh, oo_sl;
+    float* delta_w;      // ... and where it stores it
     int B, H, L;
     float scale, scale_log2e;
     int n_seg, n_row_blocks, total, row_stride;
@@ -94,7 +98,19 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_kernel(const BwdParams p) {
     float row_lse2 = 0.f, row_delta = 0.f;  // dQ: the lane's own query
     if constexpr (!POS_STATS) {
         row_lse2 = lse_b[my_row] * 1.4426950408889634f;
-        row_delta = del_b[my_row];
+        // D = rowsum(dO * O) of the lane's row (the two lanes of a row hold half of it each), kept for this launch and stored
+        // for the dK and dV launches that follow it on the stream
+        const T* orow = (const T*)p.o + b * p.oo_sb + h * p.oo_sh + (int64_t)my_row * p.oo_sl;
+        float s = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const Frag<T> of = global_frag<T>(orow + 16 * ks + 8 * g);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s = fmaf((float)bf[ks].v[e], (float)of.v[e], s);
+        }
+        s += __shfl_xor(s, 32);
+        row_delta = s;
+        if (g == 0 && r0 + rs * (wave * 32 + lm) < L) p.delta_w[(int64_t)bh * L + my_row] = s;
     }
 
     // ---- plan ----
@@ -508,27 +524,6 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_kernel(const BwdParams p) {
     }
 }
 
-// D[bh, r] = sum over d of dO[b, h, r, :] * O[b, h, r, :]; d / 8 lanes per row, 16 bytes per lane and operand
-template <typename T, int D>
-__global__ __launch_bounds__(256) void attn_bwd_delta_kernel(const T* dout, int64_t g_sb, int64_t g_sh, int64_t g_sl, const T* out,
-                                                             int64_t o_sb, int64_t o_sh, int64_t o_sl, float* delta, int H, int L,
-                                                             int64_t n_rows) {
-    constexpr int LPR = D / 8;  // lanes per row
-    const int sub = threadIdx.x % LPR;
-    const int64_t row_raw = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPR;
-    const int64_t row = row_raw < n_rows ? row_raw : n_rows - 1;  // surplus lanes shadow the last row and store nothing
-    const int r = (int)(row % L);
-    const int bh = (int)(row / L);
-    const Frag<T> gv = global_frag<T>(dout + (bh / H) * g_sb + (bh % H) * g_sh + (int64_t)r * g_sl + 8 * sub);
-    const Frag<T> ov = global_frag<T>(out + (bh / H) * o_sb + (bh % H) * o_sh + (int64_t)r * o_sl + 8 * sub);
-    float s = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) s += (float)gv.v[e] * (float)ov.v[e];
-#pragma unroll
-    for (int o = LPR / 2; o > 0; o >>= 1) s += __shfl_xor(s, o);
-    if (sub == 0 && row_raw < n_rows) delta[row] = s;
-}
-
 template <typename T, int D, int MODE>
 static int launch_bwd(BwdParams p, hipStream_t st) {
     begin_launch();
@@ -588,24 +583,9 @@ extern "C" int splat_attention_bwd(const void* q, int64_t q_sb, int64_t q_sh, in
                     (long long)plan_t_bytes);
     hipStream_t st = (hipStream_t)stream;
 
-    // D = rowsum(dO * O)
-    {
-        begin_launch();
-        const int64_t n_rows = (int64_t)B * H * L;
-        const unsigned grid = (unsigned)((n_rows * (d / 8) + 255) / 256);
-        auto run = [&](auto tag) {
-            typedef decltype(tag) E;
-            if (d == 64)
-                attn_bwd_delta_kernel<E, 64><<<grid, 256, 0, st>>>((const E*)dout, g_sb, g_sh, g_sl, (const E*)out, o_sb, o_sh, o_sl, delta, H, L, n_rows);
-            else
-                attn_bwd_delta_kernel<E, 128><<<grid, 256, 0, st>>>((const E*)dout, g_sb, g_sh, g_sl, (const E*)out, o_sb, o_sh, o_sl, delta, H, L, n_rows);
-        };
-        if (dtype == SPLAT_F16) run(f16{}); else run(bf16{});
-        if (int rc = check_launch(who)) return rc;
-    }
-
     BwdParams base;
     base.lse = lse; base.delta = delta;
+    base.o = nullptr; base.oo_sb = base.oo_sh = base.oo_sl = 0; base.delta_w = nullptr;
     base.B = B; base.H = H; base.L = L;
     base.scale = scale; base.scale_log2e = scale * 1.4426950408889634f;
     // dQ: rows = queries, the mask's own plan
@@ -618,6 +598,7 @@ extern "C" int splat_attention_bwd(const void* q, int64_t q_sb, int64_t q_sh, in
     pq.n_seg = n_seg; pq.row_stride = common_row_stride(segs, n_seg);
     pq.n_row_blocks = count_row_blocks(L, kPlanBM, pq.row_stride); pq.total = B * H * pq.n_row_blocks;
     pq.plan = static_cast<const PlanRec*>(plan);
+    pq.o = out; pq.oo_sb = o_sb; pq.oo_sh = o_sh; pq.oo_sl = o_sl; pq.delta_w = delta;  // D = rowsum(dO * O): computed and stored by this launch
     // dK, dV: rows = keys, the transposed mask's plan
     BwdParams pk = base;
     pk.a = k; pk.a_sb = k_sb; pk.a_sh = k_sh; pk.a_sl = k_sl;
