@@ -101,16 +101,20 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_kernel(const BwdParams p) {
         // D = rowsum(dO * O) of the lane's row (the two lanes of a row hold half of it each), kept for this launch and stored
         // for the dK and dV launches that follow it on the stream
         const T* orow = (const T*)p.o + b * p.oo_sb + h * p.oo_sh + (int64_t)my_row * p.oo_sl;
+        Frag<T> of[KS];  // (all requested before any is used: the accumulators' registers are still free here)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) of[ks] = global_frag<T>(orow + 16 * ks + 8 * g);
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(of[ks].v));
+#endif
         float s = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            const Frag<T> of = global_frag<T>(orow + 16 * ks + 8 * g);
+        for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) s = fmaf((float)bf[ks].v[e], (float)of.v[e], s);
-        }
+            for (int e = 0; e < 8; ++e) s = fmaf((float)bf[ks].v[e], (float)of[ks].v[e], s);
         s += __shfl_xor(s, 32);
-        row_delta = s;
-        if (g == 0 && r0 + rs * (wave * 32 + lm) < L) p.delta_w[(int64_t)bh * L + my_row] = s;
+        row_delta = s;  // (stored after the tile loop: a store in flight would be waited for with the first tile's copies)
     }
 
     // ---- plan ----
@@ -495,6 +499,10 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_kernel(const BwdParams p) {
     // every wavefront has finished reading the last tile before the stages are reused for the output
     wait_loads<0>();
     __syncthreads();
+
+    if constexpr (!POS_STATS) {
+        if (g == 0 && r0 + rs * (wave * 32 + lm) < L) p.delta_w[(int64_t)bh * L + my_row] = row_delta;
+    }
 
     // ---- epilogue: out = acc^T transposed through LDS, whole rows per store ----
     {
