@@ -360,8 +360,10 @@ static int launch_thin_variant(const char* who, SpmmParams p, hipStream_t st) {
     if (blocks > 0x7ffffff0) return 0;
     p.total = (int)blocks;
     static uint64_t reserved = 0;
-    // (d = 128: a third set would spill)
-    auto kern = spmm_thin_kernel<T, D, D == 128 ? 2 : 4>;
+    // (two register sets: more request the lines earlier, which buys nothing -- loads return in order, and the wait for a
+    // step's V rows covers every line requested before them -- and costs registers: d = 64 with 3 / 4 / 6 sets is 2 / 5 / 20 %
+    // slower, d = 128 spills with 3)
+    auto kern = spmm_thin_kernel<T, D, 2>;
     if (int rc = reserve_dynamic_lds(&reserved, reinterpret_cast<const void*>(kern), G::LDS_BYTES, who)) return rc;
     const int grid = ((p.total + 7) / 8) * 8;
     kern<<<grid, 512, G::LDS_BYTES, st>>>(p);
