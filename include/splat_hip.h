@@ -142,7 +142,7 @@ int splat_sddmm_probs(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, c
 /* splat_sddmm (lse == NULL) or splat_sddmm_probs (lse != NULL) with the mask's plan table: `plan` is what
  * splat_attention_plan wrote for the same segments and L (its per-block column ranges and per-row windows are those of
  * every tiled kernel here, not only the fused one).  The kernel for 16-bit types, d = 64 / 128 and launches of at least
- * 512 row blocks then starts its copies after two scalar loads instead of deriving the plan from the ACSR arrays
+ * 256 row blocks (or rows of at most 256 slots) then starts its copies after two scalar loads instead of deriving the plan from the ACSR arrays
  * (-7 % at B=2 H=32 L=8192 d=128 T=512, -18 % at B=4 H=16 L=4096 d=64 T=256); other shapes ignore the plan.  Same
  * results bit for bit.  A plan built from other metadata gives wrong scores but no access outside the buffers.
  * Replaces the same reference code as splat_sddmm (rsddmm_launcher, r_sddmm.py:153-188). */
@@ -170,8 +170,8 @@ int splat_spmm(const void* p, const void* v, int64_t v_sb, int64_t v_sh, int64_t
                int32_t L, int32_t n_keys, int32_t n_out, int32_t T, int32_t in_dtype,
                int32_t out_dtype, void* stream);
 
-/* splat_spmm with the mask's plan table (`plan` as in splat_sddmm_planned).  For 16-bit types, 64 or 128 output columns and
- * launches of at least 512 row blocks this runs kernels of thin wavefronts (four per SIMD) that start from the table --
+/* splat_spmm with the mask's plan table (`plan` as in splat_sddmm_planned).  For 16-bit types and 64 or 128 output columns
+ * this runs kernels of thin wavefronts (four per SIMD) that start from the table --
  * rows of at least 256 slots on 16-byte boundaries in compressed matrices of more than 192 MB through per-row rings of
  * aligned lines, everything else through a workgroup-wide tile: -20 % at B=2 H=32 L=8192 d=128 T=512, -23 % at B=4 H=16 L=4096 d=64 T=256, -40 % on rows
  * of 64 slots; masks of at least 256 slots per row whose rows all start on multiples of 8 positions of their block's walk
@@ -289,8 +289,8 @@ int splat_spmm_t(const void* p, const void* x, int64_t x_sb, int64_t x_sh, int64
                  int32_t out_dtype, void* stream);
 /* splat_spmm_t with the plan table of the TRANSPOSED mask (splat_attention_plan on `segs_t` with Lt rows; plan_bytes >=
  * splat_attention_plan_bytes(segs_t, n_seg, Lt), 16-byte aligned, device memory).  For 16-bit types of one kind for p, x
- * and out, n_out = 64 or 128, 16-byte aligned x rows, every segment with a first_col array, T >= 8 and launches of at
- * least 512 blocks of 128 output rows this runs a kernel of thin wavefronts (16 output rows each, four per SIMD) that
+ * and out, n_out = 64 or 128, 16-byte aligned x rows, every segment with a first_col array and T >= 8
+ * this runs a kernel of thin wavefronts (four per SIMD) that
  * starts from the table and keeps the tile loop's loads independent of one another: -31 % at B=2 H=32 L=8192 n_out=128
  * T=512 (dilated), -28 % at B=4 H=16 L=4096 n_out=64 T=256, -33 % on blocks of 512.  It is built for rows whose column
  * step equals the stride by which the transposed mask's rows are grouped (1 for windows and blocks, the dilation for

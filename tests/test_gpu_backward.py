@@ -271,7 +271,7 @@ MANY_BLOCKS_T = {
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("case", list(MANY_BLOCKS_T))
 def test_transposed_product_16_bit_in_launches_of_many_blocks(dev, case, dtype):
-    """16-bit transposed product with 64 / 128 output columns and at least 512 blocks of 128 output rows: with the plan
+    """16-bit transposed product with 64 / 128 output columns, here in launches of 512 blocks of 128 output rows: with the plan
     table of the transposed mask the kernel of thin wavefronts runs and must agree with the dense product and with the
     general kernel (plan=False); dead slots hold NaN and must not reach the output."""
     make, BH, n_out, by_hand = MANY_BLOCKS_T[case]

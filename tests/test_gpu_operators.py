@@ -245,7 +245,7 @@ MANY_BLOCKS = {
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("case", list(MANY_BLOCKS))
 def test_sddmm_16_bit_in_launches_of_many_row_blocks(dev, case, dtype):
-    """16-bit SDDMM with d = 64 / 128, aligned rows and at least 512 row blocks runs the kernel of thin wavefronts
+    """16-bit SDDMM with d = 64 / 128 and aligned rows (here in launches of 512 row blocks) runs the kernel of thin wavefronts
     (K through an LDS-DMA ring, scores through per-row rings, stores of whole or half lines): every variant it has, on
     uniform and non-uniform plans, against the oracle; dead slots untouched."""
     make, d = MANY_BLOCKS[case]
@@ -584,7 +584,7 @@ def _spmm_case(mask, n_out, dtype, B=8, H=8, seed=51):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("case", list(MANY_BLOCKS))
 def test_spmm_16_bit_in_launches_of_many_row_blocks(dev, case, dtype):
-    """16-bit SpMM with 64 / 128 output columns and at least 512 row blocks: with the mask's plan table (the default unless
+    """16-bit SpMM with 64 / 128 output columns, here in launches of 512 row blocks: with the mask's plan table (the default unless
     the rows are long and every one starts on a multiple of 8 positions) the kernels that start from it run -- rows of
     fewer than 256 slots through a workgroup-wide tile, longer ones through per-row rings or, where they start on 16-byte
     boundaries, straight from memory; spans that end inside half steps, rows that are empty or hold one column, rows with

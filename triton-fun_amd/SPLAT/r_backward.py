@@ -121,8 +121,7 @@ def rspmm_t_launcher(p: torch.Tensor, x: torch.Tensor, out: torch.Tensor, segmen
     product with the transposed compressed matrix: p [B, H, L, T] contiguous in the layout of ``segments``, x
     [B, H, L, n] with unit stride along n, out [B, H, Lt, n] contiguous; ``segments_t`` the ACSR of the transposed
     segment masks.  ``plan``: the plan table of the transposed mask (``segments_t.plan(Lt, device)``), which selects the
-    kernel of thin wavefronts where the library has one (16-bit types, n = 64 / 128, at least 512 blocks of 128 output
-    rows); None builds it on the first such call and keeps it with the metadata, False runs without."""
+    kernel of thin wavefronts where the library has one (16-bit types, n = 64 / 128); None builds it on the first such call and keeps it with the metadata, False runs without."""
     for name, t in (("p", p), ("x", x), ("out", out)):
         _hip.require_device_tensor(t, name)
         if t.dim() != 4:
@@ -141,7 +140,7 @@ def rspmm_t_launcher(p: torch.Tensor, x: torch.Tensor, out: torch.Tensor, segmen
     a, b = _hip.seg_array(segments.seg_args(), L, T), _hip.seg_array(segments_t.seg_args(), Lt)
     xs = x.stride()
     if plan is None and p.dtype in (torch.float16, torch.bfloat16) and out.dtype == p.dtype and n in (64, 128) \
-            and B * H * ((Lt + 127) // 128) >= 512 and _rows_step_like_the_blocks(segments, segments_t) \
+            and _rows_step_like_the_blocks(segments, segments_t) \
             and (segments_t.has_plan(Lt, dev) or not torch.cuda.is_current_stream_capturing()):
         plan = segments_t.plan(Lt, dev)  # (no table is built under stream capture: building synchronises)
     with torch.cuda.device(dev):

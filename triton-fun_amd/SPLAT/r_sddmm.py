@@ -66,12 +66,13 @@ def _strides4(t: torch.Tensor, name: str):
 
 def _takes_a_plan(x, output, y, B: int, H: int, L: int, d: int, T: int, segs: ACSRSegments) -> bool:
     """Whether this launch runs the kernel that reads a plan table (the library decides by the same rules and ignores the
-    plan otherwise): 16-bit types, d = 64 / 128, rows of K contiguous, 16-byte alignment, at least 512 row blocks."""
+    plan otherwise): 16-bit types, d = 64 / 128, rows of K contiguous, 16-byte alignment, and at least 256 row blocks or rows
+    of at most 256 slots (fewer blocks of longer rows are better off with the general kernel's split of the key range)."""
     if x.dtype not in (torch.float16, torch.bfloat16) or output.dtype != x.dtype or d not in (64, 128):
         return False
     if y.stride(2) != 1 or T % 8 != 0 or any(off % 8 for off in segs.offsets):
         return False
-    return B * H * ((L + 127) // 128) >= 512
+    return B * H * ((L + 127) // 128) >= 256 or T <= 256
 
 
 def rsddmm_launcher(x: torch.Tensor, y: torch.Tensor, output: torch.Tensor,
@@ -89,7 +90,7 @@ def rsddmm_launcher(x: torch.Tensor, y: torch.Tensor, output: torch.Tensor,
     [B, H, L], contiguous: every row's log of its sum of exp(scale * score), as the fused forward hands it out) the
     stored value is exp(scale * score - lse[row]), the row's softmax probability, instead of the score.
     ``plan``: the mask's plan table (``ACSRSegments.plan``); by default the launches that use one (16-bit types, d = 64 or
-    128, at least 512 row blocks of 128 rows) build it on their first call and keep it with the metadata, ``False``
+    128, at least 256 row blocks of 128 rows or rows of at most 256 slots) build it on their first call and keep it with the metadata, ``False``
     launches without one.  The results are the same bit for bit.
     Returns (output, sTod_linear_transformations, sTod_translations, nnzs)."""
     for name, t in (("x", x), ("y", y), ("output", output)):

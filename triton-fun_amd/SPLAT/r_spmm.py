@@ -37,7 +37,7 @@ def rspmm_launcher(x: torch.Tensor, y: torch.Tensor, output: torch.Tensor,
     ``span_loop_start/end`` (the reference's per-row-block key range) are accepted unchanged; the HIP
     kernel derives each workgroup's key range from the row maps themselves.
     ``plan``: the mask's plan table (``ACSRSegments.plan``), which selects the kernels that start from it where the library
-    has them (16-bit types, 64 or 128 output columns, at least 512 row blocks of 128 rows); by default such launches build
+    has them (16-bit types, 64 or 128 output columns); by default such launches build
     the table on their first call, keep it with the metadata and use it unless the rows have at least 256 slots and every
     one of them starts on a multiple of 8 positions (blocked masks with large blocks: the general kernel is faster
     there); ``False`` always runs the general kernel.  The kernels agree up to the order of the float32 additions.
@@ -62,7 +62,6 @@ def rspmm_launcher(x: torch.Tensor, y: torch.Tensor, output: torch.Tensor,
     dev = x.device
     arr = _hip.seg_array(segs.seg_args(), L, T)
     if plan is None and x.dtype in (torch.float16, torch.bfloat16) and output.dtype == x.dtype and n_out in (64, 128) \
-            and B * H * ((L + 127) // 128) >= 512 \
             and (segs.has_plan(L, dev) or not torch.cuda.is_current_stream_capturing()) \
             and not (T >= 256 and segs.plan_is_aligned(L, dev)):  # (no table is built under stream capture: building synchronises)
         plan = segs.plan(L, dev)

@@ -261,6 +261,7 @@ __device__ __forceinline__ int win_phase(const RowWin& w) {
 //   row  [segment][row block][row k]     RowWin + phase (row k of the block is row first + stride * k)
 typedef int PlanRec __attribute__((ext_vector_type(4)));
 constexpr int kPlanBM = 128;  // rows per row block of the fused kernel
+
 __host__ __device__ inline int64_t plan_variant_recs(int n_rb, int n_seg) { return (int64_t)n_rb * n_seg * (5 + kPlanBM); }
 __host__ __device__ inline int64_t plan_seg_at(int n_seg, int rb, int sg) { return (int64_t)rb * n_seg + sg; }
 __host__ __device__ inline int64_t plan_span_at(int n_rb, int n_seg, int rb, int sg, int wave) {

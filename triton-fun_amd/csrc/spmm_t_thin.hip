@@ -1,6 +1,6 @@
 // Transposed SpMM on ACSR (out[bh, j, :] = sum over the rows i that keep column j of p[bh, i, slot of j] * x[bh, i, :]) for
-// the common fast shape: 16-bit probabilities, x and output of one type, 64 or 128 output columns, 16-byte alignment, at
-// least 512 row blocks in the launch, and the plan table of the transposed mask.
+// the common fast shape: 16-bit probabilities, x and output of one type, 64 or 128 output columns, 16-byte alignment, and
+// the plan table of the transposed mask.
 //
 // A workgroup of 8 wavefronts owns 128 columns j = first + rs*m of the mask (rows of the output); a wavefront owns 32 of
 // them and half of the features and accumulates out^T = x^T P with 16x16x32 MFMAs (rows = output features, columns =
@@ -384,7 +384,6 @@ int launch_spmm_t_thin(const char* who, const SpmmTParams& p, int in_dtype, hipS
     // (every row's first column is read as such, whatever the row's count)
     for (int k = 0; k < p.n_seg; ++k)
         if (!p.seg[k].first_col) return 0;
-    if ((int64_t)p.B * p.H * count_row_blocks(p.Lt, 128, p.row_stride) < 512) return 0;
     auto by_d = [&](auto t) {
         using TT = decltype(t);
         return p.n_out == 128 ? launch_thin_t_variant<TT, 128>(who, p, st) : launch_thin_t_variant<TT, 64>(who, p, st);

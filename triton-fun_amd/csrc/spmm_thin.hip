@@ -1,5 +1,5 @@
-// SpMM on ACSR for 16-bit launches of many row blocks with long rows and a compressed matrix larger than the last-level
-// cache: probabilities, V and output of one type, 64 or 128 output columns, 16-byte alignment, at least 512 row blocks,
+// SpMM on ACSR for 16-bit launches with long rows and a compressed matrix larger than the last-level
+// cache: probabilities, V and output of one type, 64 or 128 output columns, 16-byte alignment,
 // rows of at least 256 slots that start on 16-byte boundaries of the buffer, more than 192 MB of probabilities, the mask's
 // plan table.  (Everything else with a plan table: spmm_tile.hip.)
 //
@@ -378,7 +378,6 @@ int launch_spmm_thin(const char* who, const SpmmParams& p, int in_dtype, hipStre
     // a lane reads 16 bytes at a time from inside its row's share of a segment
     for (int k = 0; k < p.n_seg; ++k)
         if (p.seg[k].max_cnt < 8) return 0;
-    if ((int64_t)p.B * p.H * count_row_blocks(p.L, 128, p.row_stride) < 512) return 0;
     // Rings: rows of the compressed matrix start on 16-byte boundaries, are long, and the matrix is too large for the 256 MB
     // last-level cache, so that whole lines fetched with non-temporal loads stream past the L2, where V stays (config 4's
     // 537 MB: 0.184 ms against 0.218 for the workgroup-wide tile of spmm_tile.hip).  A matrix that repeated launches find in

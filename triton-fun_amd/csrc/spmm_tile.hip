@@ -1,6 +1,6 @@
-// SpMM on ACSR for 16-bit launches of many row blocks whose rows are short or do not start on 16-byte boundaries (the
-// cases spmm_thin.hip's rings do not take): probabilities, V and output of one type, 64 or 128 output columns, at least
-// 512 row blocks, the mask's plan table.
+// SpMM on ACSR for 16-bit launches with the mask's plan table, except those that spmm_thin.hip's rings take (long rows on
+// 16-byte boundaries in a compressed matrix larger than the last-level cache): probabilities, V and output of one type, 64 or
+// 128 output columns.
 //
 // A workgroup of 8 wavefronts owns 128 rows of one (batch, head) and walks their key positions in steps of 64 as the
 // table lists them.  Per step the whole workgroup loads every row's 64 entries (8 pieces of 8 consecutive slots, 16 bytes
@@ -296,7 +296,6 @@ int launch_spmm_tile(const char* who, const SpmmParams& p, int in_dtype, hipStre
     if (p.T < 8) return 0;
     for (int k = 0; k < p.n_seg; ++k)
         if (p.seg[k].max_cnt < 8) return 0;
-    if ((int64_t)p.B * p.H * count_row_blocks(p.L, 128, p.row_stride) < 512) return 0;
     auto by_d = [&](auto t) {
         using TT = decltype(t);
         return p.n_out == 128 ? launch_tile_variant<TT, 128>(who, p, st) : launch_tile_variant<TT, 64>(who, p, st);
