@@ -300,6 +300,42 @@ def test_transposed_product_16_bit_in_launches_of_many_blocks(dev, case, dtype):
     assert float((outs[0].float() - outs[1].float()).abs().max()) <= tol
 
 
+def test_transposed_product_at_config_4_by_column_sums_and_linearity(dev):
+    """Config 4's full shape (B=2 H=32 L=8192, dilated 512/2, bf16, 128 features; 537 MB of probabilities): with x = 1 every
+    feature of output row j is the sum of column j of the compressed matrix, which a scatter-add over the slots' columns
+    gives without any dense matrix; and the product is linear in x."""
+    B, H, L, d = 2, 32, 8192, 128
+    pat = [A.dilated_pattern(L, 512, 2)]
+    segs, segs_t = A.create_acsr_segments(pat, 16, dev), transposed_segments(pat, 16, dev)
+    T = segs.T
+    dm = O.create_dilated_mask(L, 512, 2)
+    cols, valid = O.slot_columns(O.create_acsr(dm, 16), first_col=O.row_extents(dm)[0])
+    lv = torch.from_numpy(valid).to(dev)
+    ci = torch.from_numpy(np.where(valid, cols, 0)).to(dev)
+    g = torch.Generator(device=dev).manual_seed(81)
+    p = torch.rand(B, H, L, T, generator=g, device=dev)
+    p = torch.where(lv, p, torch.full((), float("nan"), device=dev)).to(torch.bfloat16)
+    want = torch.zeros(B * H, L, device=dev)
+    want.scatter_add_(1, ci.reshape(1, -1).expand(B * H, -1), torch.nan_to_num(p.float()).reshape(B * H, -1))
+    ones = torch.ones(B, H, L, d, device=dev, dtype=torch.bfloat16)
+    out = torch.full((B, H, L, d), 7.0, dtype=torch.bfloat16, device=dev)
+    rspmm_t_launcher(p, ones, out, segs, segs_t)
+    assert segs_t.has_plan(L, dev)
+    got = out.float().reshape(B * H, L, d)
+    assert float((got - want[..., None]).abs().max()) <= 8e-3 * float(want.max())
+    # linearity: (x1 + 2 x2) with values that bf16 adds exactly
+    x1 = torch.randint(-4, 5, (B, H, L, d), generator=g, device=dev).to(torch.bfloat16)
+    x2 = torch.randint(-4, 5, (B, H, L, d), generator=g, device=dev).to(torch.bfloat16)
+    o1, o2, o3 = [torch.empty(B, H, L, d, dtype=torch.float32, device=dev) for _ in range(3)]
+    # (float32 outputs take the general kernel: the two kernels against each other at full size)
+    rspmm_t_launcher(p, x1, o1, segs, segs_t)
+    rspmm_t_launcher(p, x2, o2, segs, segs_t)
+    o3b = torch.empty(B, H, L, d, dtype=torch.bfloat16, device=dev)
+    rspmm_t_launcher(p, x1 + 2 * x2, o3b, segs, segs_t)
+    lin = o1 + 2 * o2
+    assert float((o3b.float() - lin).abs().max()) <= 8e-3 * float(lin.abs().max())
+
+
 def test_transposed_product_refuses_a_plan_that_is_too_small(dev):
     pat = [A.causal_windowed_pattern(1024, 100)]
     segs, segs_t = A.create_acsr_segments(pat, 16, dev), transposed_segments(pat, 16, dev)
