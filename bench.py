@@ -330,6 +330,17 @@ def main() -> int:
             # the reference's own layout of K: [B, H, d, L] contiguous (rows that step over columns cost a transpose of K)
             kTc = kTc.contiguous()
             extras[name]["ms_kT_contiguous"] = round(min(time_batch(run, 60, 60) for _ in range(2)), 4)
+            if name in ("fused_cfg2", "fused_cfg3"):
+                # the fused backward at d = 64 (two launches: dQ, then dK and dV from one walk), from the forward's output
+                # and row statistic
+                xc = [qc, kc.transpose(2, 3), vc]
+                oc, lc = at.forward_with_stats(xc)
+                oc, lc = oc.clone(), lc.clone()
+                gc = torch.randn_like(qc)
+                at.backward_pass(xc, gc, lc, oc, fused=True)  # builds the transposed mask's ACSR and plan
+                ms_b = min(time_batch(lambda: at.backward_pass(xc, gc, lc, oc, fused=True), 20, 5) for _ in range(3))
+                extras["backward_" + name[6:]] = {"ms": round(ms_b, 4), "x_fused_forward": round(ms_b / ms, 2)}
+                del xc, oc, lc, gc
             del at, qc, kc, vc, kTc
         # the literal reference layout: K^T contiguous [B, H, d, L]
         kT_c = kT_view.contiguous()
@@ -460,7 +471,7 @@ def main() -> int:
         ms_c0 = sum(pr) / len(pr)
         extras["backward_cfg4"] = {"ms": round(ms_f, 4), "tflops_nnz": round(fl4 / ms_f / 1e9, 2),
                                    "x_fused_forward": round(ms_f / extras["fused_cfg4"]["ms"], 2),
-                                   "kernel": "splat_attention_bwd: three launches of attn_bwd_kernel (the first also computes the row sums of dO * O), no compressed matrix",
+                                   "kernel": "splat_attention_bwd: three launches of attn_bwd_kernel at d = 128 (dQ, which also computes the row sums of dO * O; dK; dV), no compressed matrix",
                                    "composed_ms_with_forward_lse": round(ms_c, 3), "composed_ms": round(ms_c0, 3)}
         del out4, lse4
         del attn4, g4, q4, k4, v4

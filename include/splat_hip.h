@@ -305,7 +305,7 @@ int splat_compressed_transpose(const void* src, void* dst, const splat_acsr_seg*
                                const splat_acsr_seg* segs_t /* host */, int32_t n_seg, int64_t BH,
                                int32_t L, int32_t T, int32_t Lt, int32_t Tt, int32_t dtype, void* stream);
 
-/* The same backward pass in three launches of one kernel and without any compressed matrix in memory (no counterpart in
+/* The same backward pass in three launches of one kernel (two at d = 64) and without any compressed matrix in memory (no counterpart in
  * the reference, which is forward only: r_attention.py:77-100).  q, k, v, out (the forward's output) and dout (the
  * upstream gradient) are [B, H, L, d] views with unit stride along d (k is K itself, rows contiguous, not K^T);
  * lse [B, H, L] is the row statistic of splat_attention_fwd_stats for the same inputs; delta [B, H, L] float32 is

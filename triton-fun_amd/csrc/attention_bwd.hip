@@ -3,7 +3,7 @@
 // With S = scale * Q K^T on the live columns, P = exp(S - lse) (lse: the forward's row statistic), O = P V and the
 // upstream gradient dO:  D = rowsum(dO * O),  dP = dO V^T,  dS = P * (dP - D),
 //     dQ = scale * dS K        dK = scale * dS^T Q        dV = P^T dO.
-// One kernel, three modes, built like the forward (attention.hip): a workgroup of 4 wavefronts owns 128 "rows", one
+// One kernel, four modes (d = 128: dQ, dK, dV, 8 products; d = 64: dQ, dK+dV, 7), built like the forward (attention.hip): a workgroup of 4 wavefronts owns 128 "rows", one
 // lane one row (two lanes share it), and walks 64-position tiles of the rows' spans as the mask's plan table lists
 // them; per tile two operand tiles X and Y arrive in LDS through the asynchronous copy ring.
 //
@@ -11,6 +11,7 @@
 //   dQ    queries  keys       Q, dO            K        V        S^T = X A^T; P; dP^T = Y B^T; dS; acc^T += X^T dS^T
 //   dK    keys     queries    K, V             Q        dO       the same with the mask's transpose
 //   dV    keys     queries    K                Q        dO       S^T = X A^T; P;                 acc^T += Y^T P^T
+//   dK+dV keys     queries    K, V             Q        dO       as dK, and acc2^T += Y^T P^T    (d = 64: both accumulators fit)
 //
 // dQ walks the mask's own plan, dK and dV the plan of the transposed mask (keys as rows).  The dQ launch comes first: its
 // lanes hold their dO rows, so it also computes D (one more read of the lane's O row) and stores it for the other two.  lse
@@ -25,7 +26,7 @@ namespace splat {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-enum { kBwdDQ = 0, kBwdDK = 1, kBwdDV = 2 };
+enum { kBwdDQ = 0, kBwdDK = 1, kBwdDV = 2, kBwdDKV = 3 };
 
 struct BwdParams {
     const void* a;  // register operand A, one row per lane: Q (dQ), K (dK, dV)
@@ -33,6 +34,7 @@ struct BwdParams {
     const void* x;  // tile operand X: K (dQ), Q (dK, dV)
     const void* y;  // tile operand Y: V (dQ), dO (dK, dV)
     void* out;      // dQ, dK, dV
+    void* out2;     // dK + dV in one launch: dV (same strides as out)
     int64_t a_sb, a_sh, a_sl, b_sb, b_sh, b_sl, x_sb, x_sh, x_sl, y_sb, y_sh, y_sl, o_sb, o_sh, o_sl;
     const float* lse;    // [B*H, L], natural log, per query
     const float* delta;  // [B*H, L], D per query (dK, dV: written by the dQ launch before them on the stream)
@@ -61,6 +63,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_kernel(const BwdParams p) {
     constexpr int NDMA = 2 * NI;
     constexpr bool POS_STATS = MODE != kBwdDQ;  // lse / D per tile position instead of per lane
     constexpr bool THREE = MODE != kBwdDV;      // the dP and dS steps
+    constexpr bool BOTH = MODE == kBwdDKV;      // dK and dV from one walk: a second accumulator, fed with P^T and Y^T
 
     extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -212,11 +215,16 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_kernel(const BwdParams p) {
         xr_addr[ks] = smem_base + RING + dual_off(lm, (16 * ks + 8 * g) * ES);
         if constexpr (THREE) yr_addr[ks] = smem_base + RING + TILE + dual_off(lm, (16 * ks + 8 * g) * ES);
     }
-    constexpr int TR_BASE = RING + (THREE ? 0 : TILE);  // dQ, dK: transposed reads of X; dV: of Y
+    constexpr int TR_BASE = RING + (THREE ? 0 : TILE);  // dQ, dK: transposed reads of X; dV: of Y; dK + dV: of both
+    uint32_t ty_addr[BOTH ? DT : 1], ty_addr8[BOTH ? DT : 1];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
         tr_addr[dt] = smem_base + TR_BASE + dual_off(4 * g + tr_row, (32 * dt + tr_col) * ES);
         tr_addr8[dt] = smem_base + TR_BASE + dual_off(4 * g + tr_row + 8, (32 * dt + tr_col) * ES);
+        if constexpr (BOTH) {
+            ty_addr[dt] = tr_addr[dt] + TILE;
+            ty_addr8[dt] = tr_addr8[dt] + TILE;
+        }
     }
     uint32_t st_addr = smem_base + 16 * g;  // lse of positions 4g.. of the stage; D is BN*4 bytes further
 
@@ -235,11 +243,14 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_kernel(const BwdParams p) {
         issue_stats(ppl, pf_tile, 0);
         advance_fetch();
     }
-    f32x16 acc[DT];
+    f32x16 acc[DT], acc2[BOTH ? DT : 1];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int j = 0; j < 16; ++j) acc[dt][j] = 0.f;
+        for (int j = 0; j < 16; ++j) {
+            acc[dt][j] = 0.f;
+            if constexpr (BOTH) acc2[dt][j] = 0.f;
+        }
 
     int cur_seg = -1, cur_tile = 0;
     RowWin win = {0, 0, 1};
@@ -420,6 +431,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_kernel(const BwdParams p) {
                     for (int j = 0; j < 16; ++j) s_acc[j] = fast_exp2(fmaf(s_acc[j], c2, -row_lse2));
                 }
                 Frag<T> pf[2];  // the second product's B operand: 16 positions each
+                Frag<T> pp[BOTH ? 2 : 1];  // dK + dV: the probabilities themselves, dV's B operand
                 if constexpr (THREE) {
                     // ---- dP^T = Y rows . B^T ----
                     f32x16 dp;
@@ -447,6 +459,10 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_kernel(const BwdParams p) {
 #pragma unroll
                         for (int j = 0; j < 16; ++j) pf[j >> 3].v[j & 7] = (T)(s_acc[j] * (dp[j] - row_delta) * p.scale);
                     }
+                    if constexpr (BOTH) {
+#pragma unroll
+                        for (int j = 0; j < 16; ++j) pp[j >> 3].v[j & 7] = (T)s_acc[j];
+                    }
                 } else {
 #pragma unroll
                     for (int j = 0; j < 16; ++j) pf[j >> 3].v[j & 7] = (T)s_acc[j];
@@ -463,6 +479,17 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_kernel(const BwdParams p) {
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int dt = 0; dt < DT; ++dt) mma32(acc[dt], tf[dt], pf[t]);
+                    if constexpr (BOTH) {
+                        // ---- acc2^T += Y^T . P^T ----
+#pragma unroll
+                        for (int dt = 0; dt < DT; ++dt) {
+                            const int roff = (32 * nt + 16 * t) * ROWB;
+                            tf[dt] = frag_from_tr<T>(lds_load_tr16(ty_addr[dt] + roff), lds_load_tr16(ty_addr8[dt] + roff));
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int dt = 0; dt < DT; ++dt) mma32(acc2[dt], tf[dt], pp[t]);
+                    }
                 }
             }
             if (2 * KS < NDMA && spread) {
@@ -493,6 +520,10 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_kernel(const BwdParams p) {
         for (int dt = 0; dt < DT; ++dt) {
             tr_addr[dt] += delta_b;
             tr_addr8[dt] += delta_b;
+            if constexpr (BOTH) {
+                ty_addr[dt] += delta_b;
+                ty_addr8[dt] += delta_b;
+            }
         }
         st_addr += stage_it == 0 ? -STATS : STATS;
     }
@@ -504,31 +535,36 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_kernel(const BwdParams p) {
         if (g == 0 && r0 + rs * (wave * 32 + lm) < L) p.delta_w[(int64_t)bh * L + my_row] = row_delta;
     }
 
-    // ---- epilogue: out = acc^T transposed through LDS, whole rows per store ----
+    // ---- epilogue: out = acc^T transposed through LDS, whole rows per store (each wavefront through a stretch of its own) ----
     {
         constexpr int OROW = D * ES + 16;
         static_assert(4 * 32 * OROW <= RING + 2 * STAGE, "staging space");
         char* stg = smem + wave * (32 * OROW);
+        auto store_rows = [&](const f32x16 (&a)[DT], T* dst) {
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
+            for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-            for (int jj = 0; jj < 4; ++jj) {
-                typedef T vec4 __attribute__((ext_vector_type(4)));
-                vec4 o;
+                for (int jj = 0; jj < 4; ++jj) {
+                    typedef T vec4 __attribute__((ext_vector_type(4)));
+                    vec4 o;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) o[i] = (T)acc[dt][4 * jj + i];
-                *reinterpret_cast<vec4*>(stg + lm * OROW + (32 * dt + 8 * jj + 4 * g) * ES) = o;
+                    for (int i = 0; i < 4; ++i) o[i] = (T)a[dt][4 * jj + i];
+                    *reinterpret_cast<vec4*>(stg + lm * OROW + (32 * dt + 8 * jj + 4 * g) * ES) = o;
+                }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            constexpr int OCPR = D * ES / 16;
+#pragma unroll
+            for (int i = 0; i < 32 * OCPR / 64; ++i) {
+                const int flat = i * 64 + lane;
+                const int row = flat / OCPR, c = flat % OCPR;
+                const int r = r0 + rs * (wave * 32 + row);
+                const u32x4 val = *reinterpret_cast<const u32x4*>(stg + row * OROW + c * 16);
+                if (r < L) __builtin_nontemporal_store(val, reinterpret_cast<u32x4*>(reinterpret_cast<char*>(dst + (int64_t)r * p.o_sl) + c * 16));
             }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        constexpr int OCPR = D * ES / 16;
-#pragma unroll
-        for (int i = 0; i < 32 * OCPR / 64; ++i) {
-            const int flat = i * 64 + lane;
-            const int row = flat / OCPR, c = flat % OCPR;
-            const int r = r0 + rs * (wave * 32 + row);
-            const u32x4 val = *reinterpret_cast<const u32x4*>(stg + row * OROW + c * 16);
-            if (r < L) __builtin_nontemporal_store(val, reinterpret_cast<u32x4*>(reinterpret_cast<char*>(ob + (int64_t)r * p.o_sl) + c * 16));
-        }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // (read out before the stretch is written again)
+        };
+        store_rows(acc, ob);
+        if constexpr (BOTH) store_rows(acc2, (T*)p.out2 + b * p.o_sb + h * p.o_sh);
     }
 }
 
@@ -547,9 +583,12 @@ static int launch_bwd(BwdParams p, hipStream_t st) {
 template <typename T>
 static int run_bwd(const BwdParams& dq, const BwdParams& dk, const BwdParams& dv, int d, hipStream_t st) {
     if (d == 64) {
+        // both accumulators of the keys' side fit the registers at d = 64 (204 of 256; at d = 128 they would need over 300):
+        // one walk, 4 products instead of 3 + 2, the scores and the exponentials once (config 2: 0.160 -> 0.133 ms)
         if (int rc = launch_bwd<T, 64, kBwdDQ>(dq, st)) return rc;
-        if (int rc = launch_bwd<T, 64, kBwdDK>(dk, st)) return rc;
-        return launch_bwd<T, 64, kBwdDV>(dv, st);
+        BwdParams dkv = dk;
+        dkv.out2 = dv.out;
+        return launch_bwd<T, 64, kBwdDKV>(dkv, st);
     }
     if (int rc = launch_bwd<T, 128, kBwdDQ>(dq, st)) return rc;
     if (int rc = launch_bwd<T, 128, kBwdDK>(dk, st)) return rc;
@@ -593,7 +632,7 @@ extern "C" int splat_attention_bwd(const void* q, int64_t q_sb, int64_t q_sh, in
 
     BwdParams base;
     base.lse = lse; base.delta = delta;
-    base.o = nullptr; base.oo_sb = base.oo_sh = base.oo_sl = 0; base.delta_w = nullptr;
+    base.o = nullptr; base.oo_sb = base.oo_sh = base.oo_sl = 0; base.delta_w = nullptr; base.out2 = nullptr;
     base.B = B; base.H = H; base.L = L;
     base.scale = scale; base.scale_log2e = scale * 1.4426950408889634f;
     // dQ: rows = queries, the mask's own plan
