@@ -413,6 +413,7 @@ class ACSRSegments:
             off += int(t[5])
         self.T = off
         self._plan_holder = None  # where plan() keeps its tables when not with this object
+        self._arrays = {}  # seg_array()'s results
 
     def __len__(self) -> int:
         return len(self.tuples)
@@ -451,7 +452,7 @@ class ACSRSegments:
             holder.splat_plans = plans
         key = (int(L), len(self), tuple(self.offsets), dev.index)
         if key not in plans:
-            arr = _hip.seg_array(self.seg_args(), L)
+            arr = self.seg_array(L)
             nbytes = int(_hip.lib().splat_attention_plan_bytes(arr, len(self), L))
             if nbytes <= 0:
                 raise _hip.SplatError(f"no plan for {len(self)} segments and L={L}")
@@ -486,6 +487,15 @@ class ACSRSegments:
 
     def seg_args(self) -> list[tuple]:
         return [(t[0], t[1], t[2], t[3], t[4], fc, off) for t, fc, off in zip(self.tuples, self.first_cols, self.offsets)]
+
+    def seg_array(self, rows: int, trailing_dim: int | None = None):
+        """The segments as the C ABI takes them (``_splat_hip.seg_array``), checked and built once per (rows, trailing
+        dimension) and kept: the metadata is taken to be immutable, and its tensors live as long as this object."""
+        key = (int(rows), None if trailing_dim is None else int(trailing_dim))
+        arr = self._arrays.get(key)
+        if arr is None:
+            arr = self._arrays[key] = _hip.seg_array(self.seg_args(), rows, trailing_dim)
+        return arr
 
     @staticmethod
     def single(dTos_lin, dTos_trans, sTod_lin, sTod_trans, nnzs, T) -> "ACSRSegments":

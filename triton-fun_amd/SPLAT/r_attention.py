@@ -81,7 +81,7 @@ def attention_launcher(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor, outpu
         output = torch.empty((B, H, L, d), dtype=target.dtype, device=target.device)
     qs, ks, vs, os_ = q.stride(), kT.stride(), v.stride(), output.stride()
     dev = q.device
-    arr = _hip.seg_array(segments.seg_args(), L)
+    arr = segments.seg_array(L)
     args = (q.data_ptr(), qs[0], qs[1], qs[2], kT.data_ptr(), ks[0], ks[1], ks[2], ks[3],
             v.data_ptr(), vs[0], vs[1], vs[2], output.data_ptr(), os_[0], os_[1], os_[2],
             arr, len(segments), B, H, L, d, float(scale), _hip.dtype_code(q.dtype))
@@ -200,7 +200,7 @@ class RegularAttention(nn.Module):
                 torch.cuda.current_stream(self._device).synchronize()
             return attention_launcher(q, k, v, self.rspmm_output, self.segments, self.scale, self._plan)
 
-        multi = self.segments if len(self.segments) > 1 else None
+        multi = self.segments  # (also for one segment: the object keeps what every call would otherwise rebuild and recheck)
         rsddmm_launcher(q, k, self.rsddmm_output,
                         self.dTos_linear_transformations, self.dTos_translations,
                         self.sTod_linear_transformations, self.sTod_translations,

@@ -74,7 +74,7 @@ def softmax_backward_launcher(p: torch.Tensor, dp: torch.Tensor, ds: torch.Tenso
     if T != segments.T:
         raise _hip.SplatError(f"trailing dimension {T} does not match the segments' {segments.T}")
     dev = p.device
-    arr = _hip.seg_array(segments.seg_args(), L, T)
+    arr = segments.seg_array(L, T)
     with torch.cuda.device(dev):
         rc = _hip.lib().splat_softmax_bwd(p.data_ptr(), dp.data_ptr(), ds.data_ptr(), arr, len(segments), B * H, L, T,
                                           float(scale), _hip.dtype_code(p.dtype), _hip.stream_ptr(dev))
@@ -97,7 +97,7 @@ def compressed_transpose_launcher(src: torch.Tensor, dst: torch.Tensor, segments
     if T != segments.T or Tt != segments_t.T:
         raise _hip.SplatError("trailing dimensions do not match the segments")
     dev = src.device
-    a, b = _hip.seg_array(segments.seg_args(), L, T), _hip.seg_array(segments_t.seg_args(), Lt, Tt)
+    a, b = segments.seg_array(L, T), segments_t.seg_array(Lt, Tt)
     with torch.cuda.device(dev):
         rc = _hip.lib().splat_compressed_transpose(src.data_ptr(), dst.data_ptr(), a, b, len(segments), B * H, L, T, Lt, Tt,
                                                    _hip.dtype_code(src.dtype), _hip.stream_ptr(dev))
@@ -137,7 +137,7 @@ def rspmm_t_launcher(p: torch.Tensor, x: torch.Tensor, out: torch.Tensor, segmen
     if T != segments.T or len(segments) != len(segments_t):
         raise _hip.SplatError("the segments do not fit p (trailing dimension, number of segments)")
     dev = p.device
-    a, b = _hip.seg_array(segments.seg_args(), L, T), _hip.seg_array(segments_t.seg_args(), Lt)
+    a, b = segments.seg_array(L, T), segments_t.seg_array(Lt)
     xs = x.stride()
     if plan is None and p.dtype in (torch.float16, torch.bfloat16) and out.dtype == p.dtype and n in (64, 128) \
             and _rows_step_like_the_blocks(segments, segments_t) \
@@ -229,8 +229,8 @@ def attention_backward_fused(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor,
         raise _hip.SplatError(f"lse must be a contiguous float32 tensor of shape {(B, H, L)}")
     delta = torch.empty((B, H, L), dtype=torch.float32, device=dev)
     dq, dk, dv = (torch.empty((B, H, L, d), dtype=dt, device=dev) for _ in range(3))
-    arr = _hip.seg_array(segments.seg_args(), L)
-    arr_t = _hip.seg_array(segments_t.seg_args(), L)
+    arr = segments.seg_array(L)
+    arr_t = segments_t.seg_array(L)
     args = []
     for t in (q, k, v, out, grad_out):
         args += [t.data_ptr(), t.stride(0), t.stride(1), t.stride(2)]

@@ -112,7 +112,7 @@ def rsddmm_launcher(x: torch.Tensor, y: torch.Tensor, output: torch.Tensor,
         raise _hip.SplatError(f"output must be a contiguous [B, H, L, T] = {(B, H, L, trailing_dim)} tensor")
     qs, ks = _strides4(x, "x"), _strides4(y, "y")
     dev = x.device
-    arr = _hip.seg_array(segs.seg_args(), L, trailing_dim)
+    arr = segs.seg_array(L, trailing_dim)
     args = (x.data_ptr(), qs[0], qs[1], qs[2], y.data_ptr(), ks[0], ks[1], ks[2], ks[3], output.data_ptr(), arr, len(segs),
             B, H, L, n_keys, d, trailing_dim, 1.0 if scale is None else float(scale), _hip.dtype_code(x.dtype),
             _hip.dtype_code(output.dtype))

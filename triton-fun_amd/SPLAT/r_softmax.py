@@ -50,7 +50,7 @@ def rsoftmax_launcher(x: torch.Tensor, output: torch.Tensor,
                                            acsr_trailing_dim_true)
     B, H, L, T = x.shape
     dev = x.device
-    arr = _hip.seg_array(segs.seg_args(), L, T)
+    arr = segs.seg_array(L, T)
     with torch.cuda.device(dev):
         rc = _hip.lib().splat_softmax(x.data_ptr(), output.data_ptr(), arr, len(segs), B * H, L, T,
                                       _hip.dtype_code(x.dtype), _hip.dtype_code(output.dtype), _hip.stream_ptr(dev))

@@ -60,7 +60,7 @@ def rspmm_launcher(x: torch.Tensor, y: torch.Tensor, output: torch.Tensor,
                                            sTod_linear_transformations, sTod_translations, nnzs, acsr_trailing_dim)
     vs = y.stride()
     dev = x.device
-    arr = _hip.seg_array(segs.seg_args(), L, T)
+    arr = segs.seg_array(L, T)
     if plan is None and x.dtype in (torch.float16, torch.bfloat16) and output.dtype == x.dtype and n_out in (64, 128) \
             and (segs.has_plan(L, dev) or not torch.cuda.is_current_stream_capturing()) \
             and not (T >= 256 and segs.plan_is_aligned(L, dev)):  # (no table is built under stream capture: building synchronises)
