@@ -153,6 +153,139 @@ def test_fused_backward_on_views_in_token_major_layout(dev, d, dtype):
         assert float((g.float().cpu() - w).abs().max()) <= TOL[dtype], nm
 
 
+def _even_rows_far_field(L, local, stride):
+    """Two segment masks: the causal window (i - local, i], and for even rows i the columns j <= i - local with
+    j % stride == stride - 1.  The far segment's transpose keeps one key in ``stride``, whose queries step by 2."""
+    i = np.arange(L)[:, None]
+    j = np.arange(L)[None, :]
+    near = ((j <= i) & (j > i - local)).astype(np.uint8)
+    far = ((j <= i - local) & (j % stride == stride - 1) & (i % 2 == 0)).astype(np.uint8)
+    return near, far
+
+
+@pytest.mark.parametrize("name,make,dense,B,H,L,d,dtype", [
+    ("strided 384/32/16", lambda: A.strided_patterns(384, 32, 16), lambda: sum(O.create_strided_segment_masks(384, 32, 16)),
+     1, 2, 384, 64, torch.float16),
+    ("strided 768/64/32, d = 128", lambda: A.strided_patterns(768, 64, 32), lambda: sum(O.create_strided_segment_masks(768, 64, 32)),
+     2, 2, 768, 128, torch.bfloat16),
+    ("strided 1000/48/40, ragged", lambda: A.strided_patterns(1000, 48, 40), lambda: sum(O.create_strided_segment_masks(1000, 48, 40)),
+     1, 3, 1000, 64, torch.bfloat16),
+    ("strided 3000/16/16: more than 128 listed keys", lambda: A.strided_patterns(3000, 16, 16),
+     lambda: sum(O.create_strided_segment_masks(3000, 16, 16)), 1, 1, 3000, 64, torch.float16),
+    ("far field of even rows only (columns step by 2), masks as arrays",
+     lambda: [torch.from_numpy(m) for m in _even_rows_far_field(640, 32, 16)], lambda: sum(_even_rows_far_field(640, 32, 16)),
+     1, 2, 640, 64, torch.float16),
+], ids=lambda x: x if isinstance(x, str) else None)
+def test_fused_backward_with_sparse_rows_of_the_transposed_mask_listed(dev, name, make, dense, B, H, L, d, dtype):
+    """Segments of the transposed mask that keep few keys with long columns (a strided pattern's far field), taken row by
+    row through splat_attention_bwd_keys: against the oracle's dense gradients, and within an ulp or two of the plain walk
+    of 128 consecutive keys (the listed keys' shares pass through one more rounding)."""
+    from r_backward import keys_side_schedule
+    scale = d ** -0.5
+    q, k, v = O.make_inputs(11 * L + d, B, H, L, d, dtype)
+    go = O.make_inputs(11 * L + d + 1, B, H, L, d, dtype)[0]
+    want = O.dense_masked_attention_grads(q, k.transpose(2, 3), v, np.asarray(dense()), scale, go)
+    attn = RegularAttention(B, L, H, d, make(), 16, 16, dev, dtype, scale=scale)
+    qd, kd, vd, god = [t.to(dev) for t in (q, k, v, go)]
+    x = [qd, kd.transpose(2, 3), vd]
+    out, lse = attn.forward_with_stats(x)
+    out, lse = out.clone(), lse.clone()
+    listed = [t.clone() for t in attn.backward_pass(x, god, lse, out, fused=True, sparse_rows=True)]
+    sched = keys_side_schedule(attn._segments_t, L, dev, B * H, always=True)
+    assert sched is not None and len(sched.main) == 1 and sched.keys.numel() > 0
+    plain = attn.backward_pass(x, god, lse, out, fused=True, sparse_rows=False)
+    for nm, g, w, pl in zip(("dq", "dk", "dv"), listed, want, plain):
+        assert torch.isfinite(g.float()).all(), nm
+        assert float((g.float().cpu() - w).abs().max()) <= TOL[dtype], nm
+        rel = (g.float() - pl.float()).abs() / pl.float().abs().clamp(min=1.0)
+        assert float(rel.max()) <= 2 * torch.finfo(dtype).eps, nm
+    assert torch.equal(listed[0], plain[0])   # dq does not depend on how the keys' side is walked
+
+
+def test_keys_side_schedule_lists_every_entry_of_the_sparse_rows_once(dev):
+    """The schedule's rows against the transposed segment they replace: per key, the stretches' progressions are disjoint
+    and their union is the key's column of queries; padding rows are empty; masks without a row-sparse segment, and walks
+    too short for the extra launch to pay, get no schedule."""
+    from r_backward import keys_side_schedule
+    L, local, stride = 2000, 48, 40
+    segs_t = transposed_segments(A.strided_patterns(L, local, stride), 16, dev)
+    assert keys_side_schedule(segs_t, L, dev, 4) is None            # columns of at most 31 tiles, one round: not worth it
+    sched = keys_side_schedule(segs_t, L, dev, 4, always=True)
+    assert sched is not None and len(sched.main) == 1 and sched.n_stretches > 1
+    far_t = sum(O.create_strided_segment_masks(L, local, stride)[1:]).T     # [key, query]
+    t = sched.rows.tuples[0]
+    lin, nnz, fcol = t[2].cpu().numpy(), t[4].cpu().numpy().astype(np.int64), sched.rows.first_cols[0].cpu().numpy()
+    key_of_row = sched.key_of_row.cpu().numpy()
+    seen = np.zeros_like(far_t, dtype=np.int64)
+    for r in range(sched.n_rows):
+        cols = fcol[r] + lin[r].astype(np.int64) * np.arange(nnz[r])
+        seen[key_of_row[r], cols] += 1
+        if r % sched.per_stretch >= sched.keys.numel():
+            assert nnz[r] == 0
+    assert np.array_equal(seen, far_t.astype(np.int64))
+    assert sorted(sched.keys.cpu().tolist()) == sorted(np.nonzero(far_t.sum(1))[0].tolist())
+    # config 3's shape takes the schedule by itself; a causal window has nothing to list
+    assert keys_side_schedule(transposed_segments(A.strided_patterns(8192, 128, 128), 16, dev), 8192, dev, 32) is not None
+    assert keys_side_schedule(transposed_segments([A.causal_windowed_pattern(4096, 255)], 16, dev), 4096, dev, 64, always=True) is None
+
+
+def test_fused_backward_at_config_3_by_comparison_of_the_two_walks(dev):
+    """Config 3's full shape (bf16, B=2 H=16 L=8192 d=64, local window 128 + every 128th key): the default takes the far
+    field's 63 keys row by row in 16 stretches of queries; same gradients as the plain walk within two ulps, and the
+    keys nobody lists are bit-identical."""
+    B, H, L, d, dtype = 2, 16, 8192, 64, torch.bfloat16
+    scale = d ** -0.5
+    attn = RegularAttention(B, L, H, d, A.strided_patterns(L, 128, 128), 16, 16, dev, dtype, scale=scale)
+    g = torch.Generator(device=dev).manual_seed(3)
+    q, k, v, go = (torch.randn(B, H, L, d, generator=g, device=dev).to(dtype) for _ in range(4))
+    x = [q, k.transpose(2, 3), v]
+    out, lse = attn.forward_with_stats(x)
+    out, lse = out.clone(), lse.clone()
+    got = [t.clone() for t in attn.backward_pass(x, go, lse, out, fused=True)]
+    plain = attn.backward_pass(x, go, lse, out, fused=True, sparse_rows=False)
+    from r_backward import keys_side_schedule
+    sched = keys_side_schedule(attn._segments_t, L, dev, B * H)
+    assert sched is not None and sched.keys.numel() == 63
+    assert torch.equal(got[0], plain[0])
+    listed = torch.zeros(L, dtype=torch.bool, device=dev)
+    listed[sched.keys] = True
+    for nm, a, b_ in zip(("dk", "dv"), got[1:], plain[1:]):
+        assert torch.equal(a[:, :, ~listed], b_[:, :, ~listed]), nm
+        diff = (a[:, :, listed].float() - b_[:, :, listed].float()).abs()
+        assert float((diff / b_[:, :, listed].float().abs().clamp(min=1.0)).max()) <= 2 * torch.finfo(dtype).eps, nm
+
+
+def test_keys_entry_point_checks_its_arguments(dev):
+    import _splat_hip as hip
+    L, d, B, H = 256, 64, 1, 1
+    segs_t = transposed_segments(A.strided_patterns(L, 16, 16), 16, dev)
+    from r_backward import keys_side_schedule
+    sched = keys_side_schedule(segs_t, L, dev, B * H, always=True)
+    R = sched.n_rows
+    t = torch.zeros(B, H, L, d, device=dev, dtype=torch.float16)
+    stat = torch.zeros(B, H, L, device=dev)
+    part = torch.zeros(2, B, H, R, d, device=dev, dtype=torch.float16)
+    plan = sched.rows.plan(R, dev)
+
+    def call(**kw):
+        a = dict(q=t.data_ptr(), k=t.data_ptr(), keys=sched.key_of_row.data_ptr(), plan_bytes=plan.numel(), n_rows=R, d=d,
+                 scale=0.125, sl=d)
+        a.update(kw)
+        rows = lambda ptr: [ptr, H * L * d, L * d, a["sl"]]
+        return hip.lib().splat_attention_bwd_keys(*rows(a["q"]), *rows(a["k"]), *rows(t.data_ptr()), *rows(t.data_ptr()),
+                                                  stat.data_ptr(), stat.data_ptr(), a["keys"], part[0].data_ptr(), part[1].data_ptr(),
+                                                  sched.rows.seg_array(R), 1, plan.data_ptr(), a["plan_bytes"], B, H, L, a["n_rows"],
+                                                  a["d"], a["scale"], hip.dtype_code(torch.float16), hip.stream_ptr(dev))
+    assert call() == 0
+    for kw, what in [(dict(q=None), "null"), (dict(keys=None), "null"), (dict(n_rows=0), "n_rows"), (dict(d=96), "head dim"),
+                     (dict(scale=0.0), "scale"), (dict(plan_bytes=plan.numel() - 16), "plan"), (dict(q=t.data_ptr() + 2), "aligned"),
+                     (dict(sl=d - 8), "row strides")]:
+        assert call(**kw) != 0, kw
+        msg = hip.lib().splat_last_error().decode()
+        assert what in msg, (kw, msg)
+    torch.cuda.synchronize()
+
+
 def test_fused_backward_arguments_are_checked(dev):
     from _splat_hip import SplatError
     L, d = 128, 64

@@ -236,13 +236,14 @@ class RegularAttention(nn.Module):
         return self.rspmm_output, self._lse
 
     def backward_pass(self, x, grad_out: torch.Tensor, lse: torch.Tensor | None = None, out: torch.Tensor | None = None,
-                      fused: bool | None = None):
+                      fused: bool | None = None, sparse_rows: bool | None = None):
         """Gradients (dq, dk, dv), each [B, H, L, d], of ``forward(x)`` for x = [q, kT, v] and the upstream gradient
         ``grad_out`` [B, H, L, d].  The ACSR of the transposed mask is built on first use; see ``r_backward``.  ``lse``
         and ``out``: the rows' statistic and the output of ``forward_with_stats`` for the same x.  Where the fused
         forward applies (16-bit dtype, d in {64, 128}) the gradients come from the fused backward kernel, which needs both
         (a forward is run here when one is missing); otherwise, or with ``fused=False``, from the operators composed over
-        compressed matrices, which ``lse`` spares the softmax pass."""
+        compressed matrices, which ``lse`` spares the softmax pass.  ``sparse_rows``: how the fused kernel takes segments
+        of the transposed mask that keep few keys with long columns (``r_backward.attention_backward_fused``)."""
         from r_backward import attention_backward, attention_backward_fused, transposed_segments
         q, kT, v = x
         if self._segments_t is None:
@@ -266,7 +267,7 @@ class RegularAttention(nn.Module):
             # once, so that later calls may run on any stream without ordering themselves after the plan kernels
             torch.cuda.current_stream(self._device).synchronize()
         return attention_backward_fused(q, kT, v, out, grad_out, lse, self.segments, self._segments_t, self._plan,
-                                        self._plan_t, self.scale)
+                                        self._plan_t, self.scale, sparse_rows)
 
 
 class _AttentionFunction(torch.autograd.Function):

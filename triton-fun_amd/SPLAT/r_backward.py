@@ -201,14 +201,120 @@ def attention_backward(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor, grad_
     return dq, dk, dv
 
 
+class KeysSideSchedule:
+    """How the fused backward walks a transposed mask some of whose segments keep only a few keys (rows), each with a long
+    column of queries: ``main`` holds the other segments (walked by 128 consecutive keys as usual), and the live rows of the
+    sparse segments are listed one per (key, stretch of queries): ``rows`` is their single-segment ACSR (``n_rows`` rows;
+    stretch c owns rows [c * per_stretch, (c + 1) * per_stretch), the keys in the same order in every stretch),
+    ``key_of_row`` the key each row belongs to (int32, 0 for padding rows, which are empty) and ``keys`` the
+    listed keys (int64, ``len(keys) <= per_stretch``)."""
+
+    def __init__(self, main: ACSRSegments, rows: ACSRSegments, key_of_row: torch.Tensor, keys: torch.Tensor,
+                 n_stretches: int, per_stretch: int):
+        self.main, self.rows, self.key_of_row, self.keys = main, rows, key_of_row, keys
+        self.n_stretches, self.per_stretch = n_stretches, per_stretch
+        self.n_rows = n_stretches * per_stretch
+
+
+# a segment of the transposed mask is listed row by row when at most one row in this many is live
+_SPARSE_ROWS_ONE_IN = 16
+# workgroups the listed rows are spread over (stretches x blocks of 128 listed rows x batch x heads): about two per slot
+_WORKGROUPS_WANTED = 512
+# the extra launch, the sum over the stretches and the scatter cost about 30 us: taken when the longest column's walk
+# (tiles of 64 queries, times the rounds in which the part runs the blocks of 128 keys) is longer than this many tiles
+_WORTH_TILES = 40
+
+
+def keys_side_schedule(segments_t: ACSRSegments, L: int, device, batch_heads: int,
+                       always: bool = False) -> KeysSideSchedule | None:
+    """The ``KeysSideSchedule`` of a transposed mask, or None when no segment of it is row-sparse (or all are, or a
+    sparse one lacks its rows' first columns), or when the walk it replaces is too short for the extra launch to pay
+    (unless ``always``).  A block of 128 consecutive keys of a strided pattern's far field holds
+    one live key with up to L queries: its workgroup walks up to L / 64 tiles for one row in 128, and the pass takes 5 x
+    what the rest of the mask needs.  Listed row by row and cut into stretches of queries, the same entries fill a few
+    workgroups each.  Built once per (L, device, number of stretches) and kept with ``segments_t`` (a host
+    synchronisation the first time: not under stream capture, where None is returned unless the schedule exists)."""
+    dev = _hip.resolve_device(device)
+    cache = segments_t.__dict__.setdefault("_keys_side", {})
+    facts = cache.get(("facts", L, dev.index))
+    if facts is None:
+        if torch.cuda.is_current_stream_capturing():
+            return None
+        sparse, first, step, cnt, key = [], [], [], [], []
+        for i, (t, fc) in enumerate(zip(segments_t.tuples, segments_t.first_cols)):
+            nnz = t[4]
+            live = torch.nonzero(nnz[:L] > 0).flatten()
+            if fc is None or live.numel() == 0 or live.numel() * _SPARSE_ROWS_ONE_IN > L:
+                continue
+            sparse.append(i)
+            n = nnz[live].to(torch.int64)
+            key.append(live)
+            first.append(fc[live].to(torch.int64))
+            step.append(torch.where(n > 1, t[2][live].to(torch.int64), torch.ones_like(n)).clamp(min=1))
+            cnt.append(n)
+        if not sparse or len(sparse) == len(segments_t):
+            facts = False
+        else:
+            first, step, cnt, key = (torch.cat(x) for x in (first, step, cnt, key))
+            last = first + step * (cnt - 1)
+            facts = (sparse, first, step, cnt, key, int(first.min()), int(last.max()), int((last - first).max()) // 64 + 1)
+        cache[("facts", L, dev.index)] = facts
+    if facts is False:
+        return None
+    sparse, first, step, cnt, key, p_min, p_max, longest_tiles = facts
+    rounds = -(-batch_heads * -(-L // 128) // 512)
+    if not always and longest_tiles * rounds < _WORTH_TILES:
+        return None
+    n_keys = key.numel()
+    per_stretch = -(-n_keys // 128) * 128
+    # stretches: enough workgroups to fill the part about twice, at least 8 tiles of 64 queries each
+    span = p_max - p_min + 1
+    want = max(1, round(_WORKGROUPS_WANTED / max(1, batch_heads * (per_stretch // 128))))
+    n_stretches = max(1, min(want, -(-span // 512)))
+    sched = cache.get((L, dev.index, n_stretches))
+    if sched is not None:
+        return sched
+    if torch.cuda.is_current_stream_capturing():
+        return None
+    width = -(-span // (n_stretches * 64)) * 64
+    lo = p_min + width * torch.arange(n_stretches, device=dev, dtype=torch.int64)[:, None]   # [stretches, 1]
+    hi = lo + width - 1
+    # the entries t of a row (columns first + step * t, t < cnt) that fall into [lo, hi]
+    t_lo = torch.div((lo - first[None, :]).clamp(min=0) + step[None, :] - 1, step[None, :], rounding_mode="floor")
+    t_hi = torch.minimum(torch.div(hi - first[None, :], step[None, :], rounding_mode="floor"), (cnt - 1)[None, :])
+    n = torch.where(hi >= first[None, :], (t_hi - t_lo + 1).clamp(min=0), torch.zeros_like(t_lo))
+    f = torch.where(n > 0, first[None, :] + step[None, :] * t_lo, torch.zeros_like(n))
+
+    def padded(x, fill, dtype):
+        out = torch.full((n_stretches, per_stretch), fill, dtype=dtype, device=dev)
+        out[:, :n_keys] = x.to(dtype)
+        return out.flatten().contiguous()
+    lin = padded(step[None, :].expand_as(n), 1, torch.float32)
+    fcol = padded(f, 0, torch.int32)
+    nnz = padded(n, 0, torch.float32)
+    trans = (fcol.to(torch.float32) / lin).contiguous()
+    rows = ACSRSegments([((1.0 / lin).contiguous(), (-trans).contiguous(), lin, trans, nnz, max(int(n.max()), 1), None, None)],
+                        [fcol])
+    main = ACSRSegments([t for i, t in enumerate(segments_t.tuples) if i not in sparse],
+                        [c for i, c in enumerate(segments_t.first_cols) if i not in sparse])
+    key_of_row = padded(key[None, :].expand(n_stretches, n_keys), 0, torch.int32)
+    sched = KeysSideSchedule(main, rows, key_of_row, key.contiguous(), n_stretches, per_stretch)
+    sched.main.plan(L, dev)
+    sched.rows.plan(sched.n_rows, dev)
+    cache[(L, dev.index, n_stretches)] = sched
+    return sched
+
+
 def attention_backward_fused(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor, out: torch.Tensor, grad_out: torch.Tensor,
                              lse: torch.Tensor, segments: ACSRSegments, segments_t: ACSRSegments, plan: torch.Tensor,
-                             plan_t: torch.Tensor, scale: float = 1.0):
+                             plan_t: torch.Tensor, scale: float = 1.0, sparse_rows: bool | None = None):
     """(dq, dk, dv) as ``attention_backward`` gives them, from three launches of one kernel and without a compressed
     matrix: ``out`` and ``lse`` are the output and the row statistic of the fused forward for the same inputs
     (``RegularAttention.forward_with_stats``), ``plan`` / ``plan_t`` the fused kernel's plans (``attention_plan``) of the
     mask's segments and of the transposed mask's.  16-bit dtypes, d in {64, 128}; operands whose rows are not contiguous
-    16-byte pieces (K^T-contiguous keys among them) are copied first."""
+    16-byte pieces (K^T-contiguous keys among them) are copied first.  Segments of the transposed mask that keep few keys
+    with long columns are taken row by row (``keys_side_schedule``; ``plan_t`` then goes unused) where that pays (``sparse_rows`` None), wherever
+    there are such segments (True) or never (False)."""
     B, H, L, d = q.shape
     dt, dev = q.dtype, q.device
     if dt not in (torch.float16, torch.bfloat16) or d not in (64, 128):
@@ -228,17 +334,40 @@ def attention_backward_fused(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor,
     if lse.dtype != torch.float32 or tuple(lse.shape) != (B, H, L) or not lse.is_contiguous():
         raise _hip.SplatError(f"lse must be a contiguous float32 tensor of shape {(B, H, L)}")
     delta = torch.empty((B, H, L), dtype=torch.float32, device=dev)
-    dq, dk, dv = (torch.empty((B, H, L, d), dtype=dt, device=dev) for _ in range(3))
+    dq = torch.empty((B, H, L, d), dtype=dt, device=dev)
+    dkv = torch.empty((2, B, H, L, d), dtype=dt, device=dev)
+    dk, dv = dkv[0], dkv[1]
+    sched = None if sparse_rows is False else keys_side_schedule(segments_t, L, dev, B * H, always=bool(sparse_rows))
+    if sched is not None:  # the row-sparse segments of the transposed mask go row by row, after the others
+        segments_t, plan_t = sched.main, sched.main.plan(L, dev)
     arr = segments.seg_array(L)
     arr_t = segments_t.seg_array(L)
-    args = []
-    for t in (q, k, v, out, grad_out):
-        args += [t.data_ptr(), t.stride(0), t.stride(1), t.stride(2)]
+
+    def strides3(*tensors):
+        a = []
+        for t in tensors:
+            a += [t.data_ptr(), t.stride(0), t.stride(1), t.stride(2)]
+        return a
+    args = strides3(q, k, v, out, grad_out)
     args += [lse.data_ptr(), delta.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
              arr, len(segments), plan.data_ptr(), plan.numel() * plan.element_size(),
              arr_t, len(segments_t), plan_t.data_ptr(), plan_t.numel() * plan_t.element_size(),
              B, H, L, d, float(scale), _hip.dtype_code(dt)]
     with torch.cuda.device(dev):
         rc = _hip.lib().splat_attention_bwd(*args, _hip.stream_ptr(dev))
-    _hip.check(rc, "splat_attention_bwd")
+        _hip.check(rc, "splat_attention_bwd")
+        if sched is not None:
+            R = sched.n_rows
+            part = torch.empty((2, B, H, R, d), dtype=dt, device=dev)
+            plan_r = sched.rows.plan(R, dev)
+            args = strides3(q, k, v, grad_out)
+            args += [lse.data_ptr(), delta.data_ptr(), sched.key_of_row.data_ptr(), part[0].data_ptr(), part[1].data_ptr(),
+                     sched.rows.seg_array(R), 1, plan_r.data_ptr(), plan_r.numel() * plan_r.element_size(),
+                     B, H, L, R, d, float(scale), _hip.dtype_code(dt)]
+            rc = _hip.lib().splat_attention_bwd_keys(*args, _hip.stream_ptr(dev))
+            _hip.check(rc, "splat_attention_bwd_keys")
+            # a key's shares (one per stretch) added up in fp32, then onto what the other segments gave it
+            n_keys = sched.keys.numel()
+            share = part.view(2, B, H, sched.n_stretches, sched.per_stretch, d)[:, :, :, :, :n_keys].sum(3, dtype=torch.float32)
+            dkv.index_add_(3, sched.keys, share.to(dt))
     return dq, dk, dv

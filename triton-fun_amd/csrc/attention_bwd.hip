@@ -20,6 +20,8 @@
 // (for acc^T), hence the swizzle that serves both (tile_copy.hpp: dual_chunk).  Probabilities come straight from the
 // statistic: no running maximum, no rescale, no second pass.  16-bit types, d = 64 or 128, rows of every operand
 // contiguous.
+#include <initializer_list>
+
 #include "attn_tile.hpp"
 
 namespace splat {
@@ -42,6 +44,8 @@ struct BwdParams {
     int64_t oo_sb, oo_sh, oo_sl;
     float* delta_w;      // ... and where it stores it
     int B, H, L;
+    int Lr;               // rows of the launch: L, or the number of rows of a rectangular keys' side (dK, dV of selected keys)
+    const int* row_map;   // [Lr] or null: the row of A / B that row r of the mask stands for (r itself when null)
     float scale, scale_log2e;
     int n_seg, n_row_blocks, total, row_stride;
     const PlanRec* plan;  // plan table of the mask (dQ) or of its transpose (dK, dV), first variant
@@ -89,7 +93,11 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_kernel(const BwdParams p) {
     const float* del_b = p.delta + (int64_t)bh * L;
 
     // ---- register operands: fragments of this lane's row, resident for the whole kernel ----
-    const int my_row = min(r0 + rs * (wave * 32 + lm), L - 1);
+    const int Lr = p.Lr;
+    int my_row = min(r0 + rs * (wave * 32 + lm), Lr - 1);
+    if constexpr (MODE != kBwdDQ) {
+        if (p.row_map) my_row = min(max(p.row_map[my_row], 0), L - 1);
+    }
     Frag<T> af[KS], bf[THREE ? KS : 1];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) af[ks] = global_frag<T>(ab + (int64_t)my_row * p.a_sl + 16 * ks + 8 * g);
@@ -532,7 +540,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_kernel(const BwdParams p) {
     __syncthreads();
 
     if constexpr (!POS_STATS) {
-        if (g == 0 && r0 + rs * (wave * 32 + lm) < L) p.delta_w[(int64_t)bh * L + my_row] = row_delta;
+        if (g == 0 && r0 + rs * (wave * 32 + lm) < Lr) p.delta_w[(int64_t)bh * L + my_row] = row_delta;
     }
 
     // ---- epilogue: out = acc^T transposed through LDS, whole rows per store (each wavefront through a stretch of its own) ----
@@ -559,7 +567,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_kernel(const BwdParams p) {
                 const int row = flat / OCPR, c = flat % OCPR;
                 const int r = r0 + rs * (wave * 32 + row);
                 const u32x4 val = *reinterpret_cast<const u32x4*>(stg + row * OROW + c * 16);
-                if (r < L) __builtin_nontemporal_store(val, reinterpret_cast<u32x4*>(reinterpret_cast<char*>(dst + (int64_t)r * p.o_sl) + c * 16));
+                if (r < Lr) __builtin_nontemporal_store(val, reinterpret_cast<u32x4*>(reinterpret_cast<char*>(dst + (int64_t)r * p.o_sl) + c * 16));
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // (read out before the stretch is written again)
         };
@@ -580,19 +588,75 @@ static int launch_bwd(BwdParams p, hipStream_t st) {
     return check_launch("splat_attention_bwd");
 }
 
+// The keys' side: dK and dV of the rows of the transposed mask that `dk` describes (dv: the same launch geometry).
 template <typename T>
-static int run_bwd(const BwdParams& dq, const BwdParams& dk, const BwdParams& dv, int d, hipStream_t st) {
+static int run_bwd_keys(const BwdParams& dk, const BwdParams& dv, int d, hipStream_t st) {
     if (d == 64) {
         // both accumulators of the keys' side fit the registers at d = 64 (204 of 256; at d = 128 they would need over 300):
         // one walk, 4 products instead of 3 + 2, the scores and the exponentials once (config 2: 0.160 -> 0.133 ms)
-        if (int rc = launch_bwd<T, 64, kBwdDQ>(dq, st)) return rc;
         BwdParams dkv = dk;
         dkv.out2 = dv.out;
         return launch_bwd<T, 64, kBwdDKV>(dkv, st);
     }
-    if (int rc = launch_bwd<T, 128, kBwdDQ>(dq, st)) return rc;
     if (int rc = launch_bwd<T, 128, kBwdDK>(dk, st)) return rc;
     return launch_bwd<T, 128, kBwdDV>(dv, st);
+}
+
+template <typename T>
+static int run_bwd(const BwdParams& dq, const BwdParams& dk, const BwdParams& dv, int d, hipStream_t st) {
+    if (int rc = d == 64 ? launch_bwd<T, 64, kBwdDQ>(dq, st) : launch_bwd<T, 128, kBwdDQ>(dq, st)) return rc;
+    return run_bwd_keys<T>(dk, dv, d, st);
+}
+
+struct Rows3 {
+    const void* ptr;
+    int64_t sb, sh, sl;
+};
+
+// Checks shared by the two entry points; `who` names the caller in messages.
+static int check_bwd_common(const char* who, int B, int H, int L, int d, float scale, int dtype, std::initializer_list<Rows3> rows,
+                            std::initializer_list<const void*> aligned16) {
+    if (B <= 0 || H <= 0 || L <= 0) return fail(SPLAT_E_SHAPE, "%s: need B, H, L > 0 (got %d, %d, %d)", who, B, H, L);
+    if (L > (1 << 23)) return fail(SPLAT_E_SHAPE, "%s: L is limited to 2^23 (got %d)", who, L);
+    if (d != 64 && d != 128) return fail(SPLAT_E_UNSUPPORTED, "%s: head dim must be 64 or 128 (got %d)", who, d);
+    if (dtype != SPLAT_F16 && dtype != SPLAT_BF16) return fail(SPLAT_E_UNSUPPORTED, "%s: 16-bit element types only (got dtype %d)", who, dtype);
+    if (!(scale > 0.f)) return fail(SPLAT_E_UNSUPPORTED, "%s: scale must be > 0 (got %g)", who, (double)scale);
+    auto mis = [&](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) != 0; };
+    for (const Rows3& r : rows) {
+        if (mis(r.ptr)) return fail(SPLAT_E_ALIGN, "%s: every tensor of rows must be 16-byte aligned", who);
+        if ((r.sb % 8) != 0 || (r.sh % 8) != 0 || (r.sl % 8) != 0)
+            return fail(SPLAT_E_ALIGN, "%s: every batch/head/row stride must be a multiple of 8 elements (16 bytes)", who);
+        if (r.sl < d) return fail(SPLAT_E_SHAPE, "%s: row strides must be >= d", who);
+    }
+    for (const void* ptr : aligned16)
+        if (mis(ptr)) return fail(SPLAT_E_ALIGN, "%s: the gradients and the plans must be 16-byte aligned", who);
+    return 0;
+}
+
+static BwdParams bwd_base(const float* lse, const float* delta, int B, int H, int L, float scale) {
+    BwdParams base;
+    base.lse = lse; base.delta = delta;
+    base.o = nullptr; base.oo_sb = base.oo_sh = base.oo_sl = 0; base.delta_w = nullptr; base.out2 = nullptr;
+    base.B = B; base.H = H; base.L = L; base.Lr = L; base.row_map = nullptr;
+    base.scale = scale; base.scale_log2e = scale * 1.4426950408889634f;
+    return base;
+}
+
+// dK (and, as a copy with b = null and out = dV, dV): rows = `Lk` keys, the plan of the (transposed) mask's `n_seg_t` segments
+// for those rows; outputs contiguous [B, H, Lk, d]
+static BwdParams bwd_keys_params(const BwdParams& base, Rows3 q, Rows3 k, Rows3 v, Rows3 g, void* dk, const splat_acsr_seg* segs_t,
+                                 int n_seg_t, const void* plan_t, int Lk, const int* row_map, int d) {
+    BwdParams pk = base;
+    pk.a = k.ptr; pk.a_sb = k.sb; pk.a_sh = k.sh; pk.a_sl = k.sl;
+    pk.b = v.ptr; pk.b_sb = v.sb; pk.b_sh = v.sh; pk.b_sl = v.sl;
+    pk.x = q.ptr; pk.x_sb = q.sb; pk.x_sh = q.sh; pk.x_sl = q.sl;
+    pk.y = g.ptr; pk.y_sb = g.sb; pk.y_sh = g.sh; pk.y_sl = g.sl;
+    pk.out = dk; pk.o_sb = (int64_t)base.H * Lk * d; pk.o_sh = (int64_t)Lk * d; pk.o_sl = d;
+    pk.Lr = Lk; pk.row_map = row_map;
+    pk.n_seg = n_seg_t; pk.row_stride = common_row_stride(segs_t, n_seg_t);
+    pk.n_row_blocks = count_row_blocks(Lk, kPlanBM, pk.row_stride); pk.total = base.B * base.H * pk.n_row_blocks;
+    pk.plan = static_cast<const PlanRec*>(plan_t);
+    return pk;
 }
 
 }  // namespace splat
@@ -609,32 +673,22 @@ extern "C" int splat_attention_bwd(const void* q, int64_t q_sb, int64_t q_sh, in
     const char* who = "splat_attention_bwd";
     if (!q || !k || !v || !out || !dout || !lse || !delta || !dq || !dk || !dv || !segs || !segs_t || !plan || !plan_t)
         return fail(SPLAT_E_NULL, "%s: null pointer argument", who);
-    if (B <= 0 || H <= 0 || L <= 0) return fail(SPLAT_E_SHAPE, "%s: need B, H, L > 0 (got %d, %d, %d)", who, B, H, L);
-    if (L > (1 << 23)) return fail(SPLAT_E_SHAPE, "%s: L is limited to 2^23 (got %d)", who, L);
-    if (d != 64 && d != 128) return fail(SPLAT_E_UNSUPPORTED, "%s: head dim must be 64 or 128 (got %d)", who, d);
-    if (dtype != SPLAT_F16 && dtype != SPLAT_BF16) return fail(SPLAT_E_UNSUPPORTED, "%s: 16-bit element types only (got dtype %d)", who, dtype);
-    if (!(scale > 0.f)) return fail(SPLAT_E_UNSUPPORTED, "%s: scale must be > 0 (got %g)", who, (double)scale);
-    auto mis = [&](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) != 0; };
-    if (mis(q) || mis(k) || mis(v) || mis(out) || mis(dout) || mis(dq) || mis(dk) || mis(dv) || mis(plan) || mis(plan_t))
-        return fail(SPLAT_E_ALIGN, "%s: q, k, v, out, dout, dq, dk, dv and the plans must be 16-byte aligned", who);
+    const Rows3 rq{q, q_sb, q_sh, q_sl}, rk{k, k_sb, k_sh, k_sl}, rv{v, v_sb, v_sh, v_sl}, ro{out, o_sb, o_sh, o_sl}, rg{dout, g_sb, g_sh, g_sl};
+    if (int rc = check_bwd_common(who, B, H, L, d, scale, dtype, {rq, rk, rv, ro, rg}, {dq, dk, dv, plan, plan_t})) return rc;
     if ((reinterpret_cast<uintptr_t>(lse) & 3) != 0 || (reinterpret_cast<uintptr_t>(delta) & 3) != 0)
         return fail(SPLAT_E_ALIGN, "%s: lse and delta must be 4-byte aligned", who);
-    for (int64_t s : {q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, o_sb, o_sh, o_sl, g_sb, g_sh, g_sl})
-        if ((s % 8) != 0) return fail(SPLAT_E_ALIGN, "%s: every batch/head/row stride must be a multiple of 8 elements (16 bytes)", who);
-    if (q_sl < d || k_sl < d || v_sl < d || o_sl < d || g_sl < d) return fail(SPLAT_E_SHAPE, "%s: row strides must be >= d", who);
     SegPtrs tmp[SPLAT_MAX_SEGMENTS];
     if (int rc = fill_segs(who, segs, n_seg, tmp, -1)) return rc;
     if (int rc = fill_segs(who, segs_t, n_seg_t, tmp, -1)) return rc;
     if (plan_bytes < splat_attention_plan_bytes(segs, n_seg, L) || plan_t_bytes < splat_attention_plan_bytes(segs_t, n_seg_t, L))
         return fail(SPLAT_E_SHAPE, "%s: a plan is smaller than its mask needs (%lld and %lld bytes given)", who, (long long)plan_bytes,
                     (long long)plan_t_bytes);
+    if ((int64_t)B * H * std::max(count_row_blocks(L, kPlanBM, common_row_stride(segs, n_seg)),
+                                  count_row_blocks(L, kPlanBM, common_row_stride(segs_t, n_seg_t))) > 0x7ffffff0)
+        return fail(SPLAT_E_SHAPE, "%s: too many row blocks", who);
     hipStream_t st = (hipStream_t)stream;
 
-    BwdParams base;
-    base.lse = lse; base.delta = delta;
-    base.o = nullptr; base.oo_sb = base.oo_sh = base.oo_sl = 0; base.delta_w = nullptr; base.out2 = nullptr;
-    base.B = B; base.H = H; base.L = L;
-    base.scale = scale; base.scale_log2e = scale * 1.4426950408889634f;
+    const BwdParams base = bwd_base(lse, delta, B, H, L, scale);
     // dQ: rows = queries, the mask's own plan
     BwdParams pq = base;
     pq.a = q; pq.a_sb = q_sb; pq.a_sh = q_sh; pq.a_sl = q_sl;
@@ -647,17 +701,41 @@ extern "C" int splat_attention_bwd(const void* q, int64_t q_sb, int64_t q_sh, in
     pq.plan = static_cast<const PlanRec*>(plan);
     pq.o = out; pq.oo_sb = o_sb; pq.oo_sh = o_sh; pq.oo_sl = o_sl; pq.delta_w = delta;  // D = rowsum(dO * O): computed and stored by this launch
     // dK, dV: rows = keys, the transposed mask's plan
-    BwdParams pk = base;
-    pk.a = k; pk.a_sb = k_sb; pk.a_sh = k_sh; pk.a_sl = k_sl;
-    pk.b = v; pk.b_sb = v_sb; pk.b_sh = v_sh; pk.b_sl = v_sl;
-    pk.x = q; pk.x_sb = q_sb; pk.x_sh = q_sh; pk.x_sl = q_sl;
-    pk.y = dout; pk.y_sb = g_sb; pk.y_sh = g_sh; pk.y_sl = g_sl;
-    pk.out = dk; pk.o_sb = pq.o_sb; pk.o_sh = pq.o_sh; pk.o_sl = d;
-    pk.n_seg = n_seg_t; pk.row_stride = common_row_stride(segs_t, n_seg_t);
-    pk.n_row_blocks = count_row_blocks(L, kPlanBM, pk.row_stride); pk.total = B * H * pk.n_row_blocks;
-    pk.plan = static_cast<const PlanRec*>(plan_t);
+    const BwdParams pk = bwd_keys_params(base, rq, rk, rv, rg, dk, segs_t, n_seg_t, plan_t, L, nullptr, d);
     BwdParams pv = pk;
     pv.b = nullptr;
     pv.out = dv;
     return dtype == SPLAT_F16 ? run_bwd<f16>(pq, pk, pv, d, st) : run_bwd<bf16>(pq, pk, pv, d, st);
+}
+
+extern "C" int splat_attention_bwd_keys(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* k, int64_t k_sb,
+                                        int64_t k_sh, int64_t k_sl, const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sl,
+                                        const void* dout, int64_t g_sb, int64_t g_sh, int64_t g_sl, const float* lse,
+                                        const float* delta, const int32_t* key_of_row, void* dk_rows, void* dv_rows,
+                                        const splat_acsr_seg* segs_t, int32_t n_seg_t, const void* plan_t, int64_t plan_t_bytes,
+                                        int32_t B, int32_t H, int32_t L, int32_t n_rows, int32_t d, float scale, int32_t dtype,
+                                        void* stream) {
+    const char* who = "splat_attention_bwd_keys";
+    if (!q || !k || !v || !dout || !lse || !delta || !key_of_row || !dk_rows || !dv_rows || !segs_t || !plan_t)
+        return fail(SPLAT_E_NULL, "%s: null pointer argument", who);
+    const Rows3 rq{q, q_sb, q_sh, q_sl}, rk{k, k_sb, k_sh, k_sl}, rv{v, v_sb, v_sh, v_sl}, rg{dout, g_sb, g_sh, g_sl};
+    if (int rc = check_bwd_common(who, B, H, L, d, scale, dtype, {rq, rk, rv, rg}, {dk_rows, dv_rows, plan_t})) return rc;
+    if (n_rows <= 0 || n_rows > (1 << 23)) return fail(SPLAT_E_SHAPE, "%s: need 0 < n_rows <= 2^23 (got %d)", who, n_rows);
+    if ((reinterpret_cast<uintptr_t>(lse) & 3) != 0 || (reinterpret_cast<uintptr_t>(delta) & 3) != 0 ||
+        (reinterpret_cast<uintptr_t>(key_of_row) & 3) != 0)
+        return fail(SPLAT_E_ALIGN, "%s: lse, delta and key_of_row must be 4-byte aligned", who);
+    SegPtrs tmp[SPLAT_MAX_SEGMENTS];
+    if (int rc = fill_segs(who, segs_t, n_seg_t, tmp, -1)) return rc;
+    if (plan_t_bytes < splat_attention_plan_bytes(segs_t, n_seg_t, n_rows))
+        return fail(SPLAT_E_SHAPE, "%s: the plan is smaller than %d rows of this mask need (%lld bytes given)", who, n_rows,
+                    (long long)plan_t_bytes);
+    if ((int64_t)B * H * count_row_blocks(n_rows, kPlanBM, common_row_stride(segs_t, n_seg_t)) > 0x7ffffff0)
+        return fail(SPLAT_E_SHAPE, "%s: too many row blocks", who);
+    const BwdParams base = bwd_base(lse, delta, B, H, L, scale);
+    const BwdParams pk = bwd_keys_params(base, rq, rk, rv, rg, dk_rows, segs_t, n_seg_t, plan_t, n_rows, key_of_row, d);
+    BwdParams pv = pk;
+    pv.b = nullptr;
+    pv.out = dv_rows;
+    hipStream_t st = (hipStream_t)stream;
+    return dtype == SPLAT_F16 ? run_bwd_keys<f16>(pk, pv, d, st) : run_bwd_keys<bf16>(pk, pv, d, st);
 }
