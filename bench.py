@@ -331,14 +331,14 @@ def main() -> int:
             kTc = kTc.contiguous()
             extras[name]["ms_kT_contiguous"] = round(min(time_batch(run, 60, 60) for _ in range(2)), 4)
             if name in ("fused_cfg2", "fused_cfg3"):
-                # the fused backward at d = 64 (two launches: dQ, then dK and dV from one walk), from the forward's output
-                # and row statistic
+                # the fused backward at d = 64 (two launches: dQ, then dK and dV from one walk; config 3 adds the launch
+                # that takes the transposed far field's 63 keys row by row), from the forward's output and row statistic
                 xc = [qc, kc.transpose(2, 3), vc]
                 oc, lc = at.forward_with_stats(xc)
                 oc, lc = oc.clone(), lc.clone()
                 gc = torch.randn_like(qc)
                 at.backward_pass(xc, gc, lc, oc, fused=True)  # builds the transposed mask's ACSR and plan
-                ms_b = min(time_batch(lambda: at.backward_pass(xc, gc, lc, oc, fused=True), 20, 5) for _ in range(3))
+                ms_b = min(time_batch(lambda: at.backward_pass(xc, gc, lc, oc, fused=True), 40, 20) for _ in range(4))
                 extras["backward_" + name[6:]] = {"ms": round(ms_b, 4), "x_fused_forward": round(ms_b / ms, 2)}
                 del xc, oc, lc, gc
             del at, qc, kc, vc, kTc

@@ -366,8 +366,9 @@ def attention_backward_fused(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor,
                      B, H, L, R, d, float(scale), _hip.dtype_code(dt)]
             rc = _hip.lib().splat_attention_bwd_keys(*args, _hip.stream_ptr(dev))
             _hip.check(rc, "splat_attention_bwd_keys")
-            # a key's shares (one per stretch) added up in fp32, then onto what the other segments gave it
+            # a key's shares (one per stretch) added up (the reduction accumulates in fp32 and rounds once), then onto what
+            # the other segments gave it
             n_keys = sched.keys.numel()
-            share = part.view(2, B, H, sched.n_stretches, sched.per_stretch, d)[:, :, :, :, :n_keys].sum(3, dtype=torch.float32)
-            dkv.index_add_(3, sched.keys, share.to(dt))
+            share = part.view(2, B, H, sched.n_stretches, sched.per_stretch, d)[:, :, :, :, :n_keys].sum(3)
+            dkv.index_add_(3, sched.keys, share)
     return dq, dk, dv
