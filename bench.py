@@ -321,6 +321,9 @@ def main() -> int:
             byt = 4.0 * Bc * Hc * Lc * dc * qc.element_size()
             kTc = kc.transpose(2, 3)
             run = lambda: at([qc, kTc, vc])
+            # (launches of 0.02-0.05 ms: the clock, which drops while the host builds the next case, needs some 40 ms of
+            # them to come back: 0.051, 0.045, 0.043, 0.042, 0.041, 0.040 ms in six batches of 120 at config 2, then 0.0395)
+            settle(run)
             ms = min(time_batch(run, 60, 60) for _ in range(3))
             peak = FP32_MFMA_PEAK_TFLOPS if dt == torch.float32 else MFMA_PEAK_TFLOPS
             extras[name] = {"ms": round(ms, 4), "tflops_nnz": round(fl / ms / 1e9, 2),
@@ -329,6 +332,7 @@ def main() -> int:
                             "pct_of_hbm_floor_rate": round(100 * byt / HBM_PEAK_GBPS / 1e6 / ms, 2)}
             # the reference's own layout of K: [B, H, d, L] contiguous (rows that step over columns cost a transpose of K)
             kTc = kTc.contiguous()
+            settle(run)
             extras[name]["ms_kT_contiguous"] = round(min(time_batch(run, 60, 60) for _ in range(2)), 4)
             if name in ("fused_cfg2", "fused_cfg3"):
                 # the fused backward at d = 64 (two launches: dQ, then dK and dV from one walk; config 3 adds the launch
@@ -338,7 +342,8 @@ def main() -> int:
                 oc, lc = oc.clone(), lc.clone()
                 gc = torch.randn_like(qc)
                 at.backward_pass(xc, gc, lc, oc, fused=True)  # builds the transposed mask's ACSR and plan
-                ms_b = min(time_batch(lambda: at.backward_pass(xc, gc, lc, oc, fused=True), 40, 20) for _ in range(4))
+                settle(lambda: at.backward_pass(xc, gc, lc, oc, fused=True))
+                ms_b = min(time_batch(lambda: at.backward_pass(xc, gc, lc, oc, fused=True), 40, 20) for _ in range(3))
                 extras["backward_" + name[6:]] = {"ms": round(ms_b, 4), "x_fused_forward": round(ms_b / ms, 2)}
                 del xc, oc, lc, gc
             del at, qc, kc, vc, kTc
@@ -375,6 +380,7 @@ def main() -> int:
             rc = hip.lib().splat_acsr_build(mask.data_ptr(), L, L, mask.stride(0), 16, *[t.data_ptr() for t in f32 + spans + ext],
                                             summ.data_ptr(), hip.stream_ptr(dev))
             hip.check(rc, "splat_acsr_build")
+        settle(build_kernels)
         _, per_k = time_launches(build_kernels, 10, 2)
         ms_k = sum(per_k) / len(per_k)
         ms_cold = time_cold_launches(build_kernels, flush, 10)
@@ -449,6 +455,7 @@ def main() -> int:
         p3 = torch.empty_like(s3)
         sg0 = segs3.tuples[0]
         run_soft3 = lambda: r_softmax.rsoftmax_launcher(s3, p3, sg0[0], sg0[1], sg0[2], sg0[3], T3, 256, sg0[4], (1, 1), 16, segments=segs3)
+        settle(run_soft3)
         ms = min(time_batch(run_soft3, 40, 10) for _ in range(3))
         byt3 = 2 * live3 * B3 * H3 * 2
         extras["softmax_cfg3"] = {"ms": round(ms, 4), "T": T3, "gbps_algorithmic": round(byt3 / ms / 1e6, 1),
