@@ -347,6 +347,28 @@ def main() -> int:
                 extras["backward_" + name[6:]] = {"ms": round(ms_b, 4), "x_fused_forward": round(ms_b / ms, 2)}
                 del xc, oc, lc, gc
             del at, qc, kc, vc, kTc
+        # the d = 64 tile loop alone (both products out of LDS, one exponential per score, a barrier per tile: no loads, no
+        # masks, no beginnings and ends of workgroups) in the kernel's wavefront shape and in thin wavefronts: what configs
+        # 2 and 3 could reach if their workgroups had nothing but tiles to do
+        import bench_probes as BP
+        loop_data = (0.5 * torch.randn(32768, dtype=torch.float32)).to(torch.bfloat16).to(dev)
+        loop_wgs, loop_tiles = 256 * 3 * 3, 64
+        loop = {}
+        for shape, label in BP.SOFTMAX_LOOP_SHAPES.items():
+            loop_out = torch.empty(loop_wgs * BP.SOFTMAX_LOOP_THREADS[shape], dtype=torch.float32, device=dev)
+            for with_exp in (1, 0):
+                probe = lambda s=shape, e=with_exp, o=loop_out: BP.check(BP.lib().splat_bench_softmax_loop_probe(
+                    loop_data.data_ptr(), loop_data.numel() * 2, o.data_ptr(), o.numel() * 4, s, e, loop_wgs, loop_tiles,
+                    hip.stream_ptr(dev)), "splat_bench_softmax_loop_probe")
+                settle(probe)
+                ms_l = min(time_batch(probe, 20, 5) for _ in range(3))
+                tf = BP.lib().splat_bench_softmax_loop_probe_flops(loop_wgs, loop_tiles) / (ms_l * 1e-3) / 1e12
+                loop[("with" if with_exp else "without") + "_exponentials, " + label] = {
+                    "workgroup_tiles_per_us": round(loop_wgs * loop_tiles / ms_l / 1e3, 1), "tflops": round(tf, 1),
+                    "pct_mfma_peak": round(100 * tf / MFMA_PEAK_TFLOPS, 2)}
+            del loop_out
+        extras["tile_loop_d64"] = loop
+        del loop_data
         # the literal reference layout: K^T contiguous [B, H, d, L]
         kT_c = kT_view.contiguous()
         _, per_c = time_launches(lambda: attn([qd, kT_c, vd]), max(5, args.steps // 2), max(3, args.warmup // 2))

@@ -2,7 +2,7 @@
  * splat_bench.h -- C ABI of libsplat_bench.so: measurement aids for bench.py.
  *
  * Nothing here has a counterpart in the reference (spikerheado1234/triton-fun) and nothing on the operator path
- * calls it: the operator ABI a maintainer binds is include/splat_hip.h.  These are the two ceilings bench.py quotes the
+ * calls it: the operator ABI a maintainer binds is include/splat_hip.h.  These are the ceilings bench.py quotes the
  * kernels against, built from the same sources and with the same flags as the operators.
  *
  * Conventions as in splat_hip.h: device pointers, `stream` a hipStream_t passed as void*, calls only enqueue work and
@@ -18,7 +18,7 @@
 extern "C" {
 #endif
 
-#define SPLAT_BENCH_VERSION 100
+#define SPLAT_BENCH_VERSION 200
 
 int splat_bench_version(void);
 const char* splat_bench_last_error(void);
@@ -44,6 +44,18 @@ int splat_bench_stream_copy(const void* src, void* dst, int64_t bytes, void* str
 int splat_bench_mfma_lds_probe(const void* data, int64_t data_bytes, void* out, int64_t out_bytes, int32_t shape,
                                int32_t workgroups, int32_t tiles, void* stream);
 int64_t splat_bench_mfma_lds_probe_flops(int32_t shape, int32_t workgroups, int32_t tiles);
+
+/* The fused forward's tile loop at d = 64 in bf16 with its exponentials and nothing else around it: per 64-key tile both
+ * products out of LDS tiles and, per score, one multiply-add, one exponential, one add into the row sum and one
+ * conversion (the loop's work once every row has its reference), one workgroup barrier per tile; no global loads, no
+ * masks.  `shape` 0: 32 query rows per wavefront (32x32x16 MFMA, 256 threads per workgroup); 1: 16 rows per wavefront
+ * (16x16x32 MFMA, 512 threads).  Both are launched with 53 KiB of LDS, so that three workgroups share a compute unit:
+ * 3 and 6 wavefronts per SIMD.  `exponentials` 0 replaces the exponential and the sum by a multiplication.  data, out
+ * and the limits as for splat_bench_mfma_lds_probe; splat_bench_softmax_loop_probe_flops gives the matrix operations of
+ * one call (128 rows x 64 keys x 64 x 4 per workgroup and tile). */
+int splat_bench_softmax_loop_probe(const void* data, int64_t data_bytes, void* out, int64_t out_bytes, int32_t shape,
+                                   int32_t exponentials, int32_t workgroups, int32_t tiles, void* stream);
+int64_t splat_bench_softmax_loop_probe_flops(int32_t workgroups, int32_t tiles);
 
 #ifdef __cplusplus
 }

@@ -767,6 +767,35 @@ def test_mfma_lds_probe_runs_and_checks_its_arguments(dev, shape):
     assert BP.lib().splat_bench_mfma_lds_probe_flops(3, wgs, tiles) == 0
 
 
+@pytest.mark.parametrize("exponentials", [1, 0])
+@pytest.mark.parametrize("shape", [0, 1])
+def test_softmax_loop_probe_runs_and_checks_its_arguments(dev, shape, exponentials):
+    """splat_bench_softmax_loop_probe, the d = 64 tile loop with its exponentials that bench.py quotes configs 2 and 3
+    against: every workgroup computes the same finite figures from the same data, two calls agree, nothing is written past
+    the workgroups' floats, and short buffers are refused."""
+    import _splat_hip as hip
+    import bench_probes as BP
+    data = (0.5 * torch.randn(32768, generator=torch.Generator().manual_seed(6))).to(torch.bfloat16).to(dev)
+    wgs, tiles, nt = 5, 3, BP.SOFTMAX_LOOP_THREADS[shape]
+    out = torch.full((wgs * nt + 8,), 7.0, dtype=torch.float32, device=dev)
+    fn = BP.lib().splat_bench_softmax_loop_probe
+    call = lambda d, o: fn(d.data_ptr(), d.numel() * 2, o.data_ptr(), wgs * nt * 4, shape, exponentials, wgs, tiles, hip.stream_ptr(dev))
+    BP.check(call(data, out), "splat_bench_softmax_loop_probe")
+    res = out[:wgs * nt].view(wgs, nt)
+    assert torch.isfinite(res).all() and float(res.abs().max()) > 0
+    assert torch.equal(res, res[0].expand_as(res))
+    assert torch.all(out[wgs * nt:] == 7.0)
+    again = torch.empty_like(out)
+    BP.check(call(data, again), "splat_bench_softmax_loop_probe")
+    assert torch.equal(again[:wgs * nt], out[:wgs * nt])
+    assert fn(data.data_ptr(), 65535, out.data_ptr(), wgs * nt * 4, shape, exponentials, wgs, tiles, None) == -2
+    assert fn(data.data_ptr(), 65536, out.data_ptr(), wgs * nt * 4 - 1, shape, exponentials, wgs, tiles, None) == -2
+    assert fn(data.data_ptr(), 65536, out.data_ptr(), wgs * nt * 4, shape, exponentials, 0, tiles, None) == -2
+    assert fn(data.data_ptr() + 2, 65536, out.data_ptr(), wgs * nt * 4, shape, exponentials, wgs, tiles, None) == -4
+    assert fn(data.data_ptr(), 65536, out.data_ptr(), wgs * nt * 4, 2, exponentials, wgs, tiles, None) == -5
+    assert BP.lib().splat_bench_softmax_loop_probe_flops(wgs, tiles) == wgs * tiles * 128 * 64 * 64 * 4
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("L,d", [(64, 64), (1000, 128), (333, 64), (77, 40), (130, 7), (1, 128)])
 def test_key_transpose(dev, L, d, dtype):

@@ -15,12 +15,17 @@ _SIGNATURES = {
     "splat_bench_stream_copy": (ctypes.c_int, [_vp, _vp, _i64, _vp]),
     "splat_bench_mfma_lds_probe": (ctypes.c_int, [_vp, _i64, _vp, _i64, _i32, _i32, _i32, _vp]),
     "splat_bench_mfma_lds_probe_flops": (ctypes.c_int64, [_i32, _i32, _i32]),
+    "splat_bench_softmax_loop_probe": (ctypes.c_int, [_vp, _i64, _vp, _i64, _i32, _i32, _i32, _i32, _vp]),
+    "splat_bench_softmax_loop_probe_flops": (ctypes.c_int64, [_i32, _i32]),
 }
 EXPORTS = tuple(_SIGNATURES)
 PROBE_SHAPES = {0: "32x32x16, 32 rows per wavefront, 2 wavefronts per SIMD",
                 1: "32x32x16, 64 rows per wavefront, 1 wavefront per SIMD",
                 2: "16x16x32, 16 rows per wavefront, 4 wavefronts per SIMD"}
 PROBE_THREADS = {0: 256, 1: 256, 2: 512}
+SOFTMAX_LOOP_SHAPES = {0: "32x32x16, 32 rows per wavefront, 3 wavefronts per SIMD",
+                       1: "16x16x32, 16 rows per wavefront, 6 wavefronts per SIMD"}
+SOFTMAX_LOOP_THREADS = {0: 256, 1: 512}
 
 _lib = None
 

@@ -221,6 +221,184 @@ __global__ __launch_bounds__(512, 4) void mfma_lds_probe_thin_kernel(const bf16*
     out[(int64_t)blockIdx.x * blockDim.x + tid] = sum;
 }
 
+// The fused forward's tile loop at d = 64 with its exponentials: per 64-key tile both products out of LDS tiles and, per
+// score, one multiply-add, one exponential, one add into the row sum and one conversion (what the kernel's loop does once
+// every row has its reference); a workgroup barrier per tile, no loads, no masks.  Two shapes: 32 query rows per wavefront
+// (32 x 32 x 16 MFMA, 4 wavefronts per workgroup) and 16 (16 x 16 x 32 MFMA, 8 wavefronts per workgroup), both launched
+// with 53 KiB of LDS so that three workgroups share a compute unit (3 and 6 wavefronts per SIMD).
+constexpr int kSD = 64, kSROWB = kSD * 2, kSKB = kPBN * kSROWB, kSSTAGE = 2 * kSKB, kSLDS = 53 * 1024;
+
+template <bool EXP>
+__global__ __launch_bounds__(256, 3) void softmax_loop_probe_wide_kernel(const bf16* data, float* out, int tiles) {
+    constexpr int KS = kSD / 16, DT = kSD / 32, NT = kPBN / 32;
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, lm = lane & 31, g = lane >> 5;
+    for (int i = tid; i < 2 * kSSTAGE / 16; i += 256) reinterpret_cast<u32x4*>(smem)[i] = reinterpret_cast<const u32x4*>(data)[i];
+    Frag<bf16> qf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = global_frag<bf16>(data + (tid & 127) * kSD + 16 * ks + 8 * g);
+    __syncthreads();
+    const uint32_t smem_base = lds_address(smem);
+    const int tr_row = (lane & 15) >> 2, tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    uint32_t k_addr[KS], v_addr[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+        v_addr[dt] = smem_base + kSKB + (4 * g + tr_row) * kSROWB + ((dt ^ swz64<kSROWB>(4 * g + tr_row)) * 64) + tr_col * 2;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) k_addr[ks] = smem_base + lds_off<kSROWB, true>(lm, (16 * ks + 8 * g) * 2);
+    f32x16 o_acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) o_acc[dt][j] = 0.f;
+    float l_run = 0.f;
+    const float m2 = 3.0f + 0.01f * lane;
+    int stage = 0;
+    for (int it = 0; it < tiles; ++it) {
+        __syncthreads();  // (where the real loop hands a stage over)
+        f32x16 s_acc[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) s_acc[nt][j] = 0.f;
+        constexpr int NFR = NT * KS;
+        Frag<bf16> kfr[NFR];
+#pragma unroll
+        for (int i = 0; i < NFR; ++i)
+            kfr[i].v = __builtin_bit_cast(typename Frag<bf16>::vec, lds_load128(k_addr[i % KS] + 32 * (i / KS) * kSROWB));
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < NFR; ++i) mma32(s_acc[i / KS], kfr[i], qf[i % KS]);
+        Frag<bf16> pf[NT][2];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                float pv;
+                if (EXP) {
+                    pv = fast_exp2(fmaf(s_acc[nt][j], 0.18f, -m2));
+                    l_run += pv;
+                } else {
+                    pv = s_acc[nt][j] * 0.0884f;
+                }
+                pf[nt][j >> 3].v[j & 7] = (bf16)pv;
+            }
+        auto load_v = [&](int nt, int t, int dt) {
+            const uint32_t a0 = v_addr[dt] + (32 * nt + 16 * t) * kSROWB;
+            return frag_from_tr<bf16>(lds_load_tr16(a0), lds_load_tr16(a0 + 8 * kSROWB));
+        };
+        Frag<bf16> vfr[2][DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) vfr[0][dt] = load_v(0, 0, dt);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int step = 0; step < 2 * NT; ++step) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                mma32(o_acc[dt], vfr[step & 1][dt], pf[step >> 1][step & 1]);
+                if (step + 1 < 2 * NT) {
+                    vfr[(step + 1) & 1][dt] = load_v((step + 1) >> 1, (step + 1) & 1, dt);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+        stage ^= 1;
+        const int delta = stage == 0 ? -kSSTAGE : kSSTAGE;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) v_addr[dt] += delta;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) k_addr[ks] += delta;
+    }
+    float sum = l_run;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) sum += o_acc[dt][j];
+    out[(int64_t)blockIdx.x * blockDim.x + tid] = sum;
+}
+
+template <bool EXP>
+__global__ __launch_bounds__(512, 6) void softmax_loop_probe_thin_kernel(const bf16* data, float* out, int tiles) {
+    constexpr int KS = kSD / 32, DB = kSD / 16;
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, li = lane & 15, g = lane >> 4;
+    for (int i = tid; i < 2 * kSSTAGE / 16; i += 512) reinterpret_cast<u32x4*>(smem)[i] = reinterpret_cast<const u32x4*>(data)[i];
+    Frag<bf16> qf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = global_frag<bf16>(data + (tid & 127) * kSD + 32 * ks + 8 * g);
+    __syncthreads();
+    const uint32_t smem_base = lds_address(smem);
+    uint32_t k_addr[KS], v_addr[kSD / 32];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) k_addr[ks] = smem_base + li * kSROWB + (((4 * ks + g) ^ (li & 7)) << 4);
+    {
+        const int row = 4 * g + (li >> 2);
+#pragma unroll
+        for (int dp = 0; dp < kSD / 32; ++dp) v_addr[dp] = smem_base + kSKB + row * kSROWB + ((dp ^ (row & 1)) * 64) + (4 * (li & 3)) * 2;
+    }
+    const uint32_t v_half = (g & 1) * 32;
+    f32x4v o_acc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o_acc[db][j] = 0.f;
+    float l_run = 0.f;
+    const float m2 = 3.0f + 0.01f * lane;
+    int stage = 0;
+    for (int it = 0; it < tiles; ++it) {
+        __syncthreads();  // (where the real loop hands a stage over)
+        f32x4v s_acc[4];
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) s_acc[blk][j] = 0.f;
+        constexpr int NFR = 4 * KS;
+        Frag<bf16> kfr[NFR];
+#pragma unroll
+        for (int i = 0; i < NFR; ++i)  // i = KS blk + ks
+            kfr[i].v = __builtin_bit_cast(typename Frag<bf16>::vec, lds_load128(k_addr[i % KS] + 16 * (i / KS) * kSROWB));
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < NFR; ++i) mma16(s_acc[i / KS], kfr[i], qf[i % KS]);
+        Frag<bf16> pf[2];
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float pv;
+                if (EXP) {
+                    pv = fast_exp2(fmaf(s_acc[blk][j], 0.18f, -m2));
+                    l_run += pv;
+                } else {
+                    pv = s_acc[blk][j] * 0.0884f;
+                }
+                pf[blk >> 1].v[4 * (blk & 1) + j] = (bf16)pv;
+            }
+        auto load_v = [&](int t, int db) {
+            const uint32_t a0 = (v_addr[db >> 1] + (((db & 1) * 32) ^ v_half)) + 32 * t * kSROWB;
+            return frag_from_tr<bf16>(lds_load_tr16(a0), lds_load_tr16(a0 + 16 * kSROWB));
+        };
+        Frag<bf16> vfr[2 * DB];
+#pragma unroll
+        for (int i = 0; i < 2 * DB; ++i) vfr[i] = load_v(i / DB, i % DB);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 2 * DB; ++i) mma16(o_acc[i % DB], vfr[i], pf[i / DB]);
+        stage ^= 1;
+        const int delta = stage == 0 ? -kSSTAGE : kSSTAGE;
+#pragma unroll
+        for (int dp = 0; dp < kSD / 32; ++dp) v_addr[dp] += delta;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) k_addr[ks] += delta;
+    }
+    float sum = l_run;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sum += o_acc[db][j];
+    out[(int64_t)blockIdx.x * blockDim.x + tid] = sum;
+}
+
 // The streaming ceiling the HBM-bound kernels are held against: a plain copy with the loads and stores the row softmax
 // uses (16 bytes per lane, non-temporal, four requests in flight per lane), workgroups striding over the buffer.
 __global__ __launch_bounds__(256) void stream_copy_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, int64_t n16) {
@@ -292,5 +470,41 @@ extern "C" int splat_bench_mfma_lds_probe(const void* data, int64_t data_bytes, 
         if (int rc = reserve_dynamic_lds(&reserved[2], (const void*)mfma_lds_probe_thin_kernel, 65536, who)) return rc;
         mfma_lds_probe_thin_kernel<<<workgroups, 512, 65536, st>>>(d, o, tiles);
     }
+    return check_launch(who);
+}
+
+extern "C" int64_t splat_bench_softmax_loop_probe_flops(int32_t workgroups, int32_t tiles) {
+    return (int64_t)workgroups * tiles * 128 * 2 * 64 * kSD * 2;
+}
+
+extern "C" int splat_bench_softmax_loop_probe(const void* data, int64_t data_bytes, void* out, int64_t out_bytes, int32_t shape,
+                                              int32_t exponentials, int32_t workgroups, int32_t tiles, void* stream) {
+    begin_launch();
+    const char* who = "splat_bench_softmax_loop_probe";
+    if (!data || !out) return fail(SPLAT_E_NULL, "%s: null pointer argument", who);
+    if (shape < 0 || shape > 1) return fail(SPLAT_E_UNSUPPORTED, "%s: shape must be 0 or 1 (got %d)", who, shape);
+    if (workgroups < 1 || workgroups > (1 << 20) || tiles < 1 || tiles > (1 << 20))
+        return fail(SPLAT_E_SHAPE, "%s: workgroups and tiles must be 1..2^20 (got %d, %d)", who, workgroups, tiles);
+    if (data_bytes < 65536) return fail(SPLAT_E_SHAPE, "%s: data must hold 65536 bytes (got %lld)", who, (long long)data_bytes);
+    const int threads = shape == 1 ? 512 : 256;
+    if (out_bytes < (int64_t)workgroups * threads * 4)
+        return fail(SPLAT_E_SHAPE, "%s: out must hold %d bytes per workgroup (got %lld for %d)", who, threads * 4, (long long)out_bytes, workgroups);
+    if ((reinterpret_cast<uintptr_t>(data) & 15) != 0 || (reinterpret_cast<uintptr_t>(out) & 3) != 0)
+        return fail(SPLAT_E_ALIGN, "%s: data must be 16-byte aligned, out 4-byte aligned", who);
+    const bf16* d = static_cast<const bf16*>(data);
+    float* o = static_cast<float*>(out);
+    hipStream_t st = (hipStream_t)stream;
+    static uint64_t reserved[4] = {0, 0, 0, 0};
+    auto go = [&](auto kern, uint64_t* res) -> int {
+        if (int rc = reserve_dynamic_lds(res, (const void*)kern, kSLDS, who)) return rc;
+        kern<<<workgroups, threads, kSLDS, st>>>(d, o, tiles);
+        return 0;
+    };
+    int rc;
+    if (shape == 0)
+        rc = exponentials ? go(softmax_loop_probe_wide_kernel<true>, &reserved[0]) : go(softmax_loop_probe_wide_kernel<false>, &reserved[1]);
+    else
+        rc = exponentials ? go(softmax_loop_probe_thin_kernel<true>, &reserved[2]) : go(softmax_loop_probe_thin_kernel<false>, &reserved[3]);
+    if (rc) return rc;
     return check_launch(who);
 }
