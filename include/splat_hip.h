@@ -323,22 +323,25 @@ int splat_attention_bwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl,
                         void* stream);
 
 /* The keys' side of that pass for a list of rows of the transposed mask (no counterpart in the reference, which is forward
- * only: r_attention.py:77-100): row r of segs_t (n_rows rows, each an arithmetic progression of queries below L) belongs
- * to key key_of_row[r] (device int32 [n_rows], values in [0, L); several rows may name one key, e.g. one per stretch of
- * its queries), and dk_rows / dv_rows (contiguous [B, H, n_rows, d], overwritten) receive that row's share of dk / dv, which
- * the caller adds up per key.  For transposed masks that keep a few keys with very long columns (a strided pattern's far
+ * only: r_attention.py:77-100).  For transposed masks that keep a few keys with very long columns (a strided pattern's far
  * field: one key in 128 with up to L queries), whose walk by 128 consecutive keys runs almost empty tiles: the caller
- * leaves such a segment out of splat_attention_bwd's segs_t, lists its live rows here (cut into stretches of queries so
- * that many workgroups share the walk) and adds the result to dk and dv.  q, k, v, dout, lse as for splat_attention_bwd;
- * delta as splat_attention_bwd wrote it for the same inputs (earlier on the same stream); plan_t is
- * splat_attention_plan(segs_t, n_seg_t, n_rows). */
+ * leaves such a segment out of splat_attention_bwd's segs_t and lists its live rows here, cut into stretches of queries so
+ * that many workgroups share the walk.  Row r of segs_t (n_rows rows, each an arithmetic progression of queries below L)
+ * belongs to key key_of_row[r] (device int32 [n_rows]; values in [0, L), or negative for an empty padding row); dk_rows /
+ * dv_rows (contiguous [B, H, n_rows, d], overwritten) receive every row's share of dk / dv.  With dk and dv given (contiguous
+ * [B, H, L, d], as splat_attention_bwd wrote them for the other segments; both or neither), a second kernel adds the shares
+ * onto them: rows k, k + rows_per_stretch, k + 2 rows_per_stretch, ... must then name the same key (one row per stretch,
+ * the keys in the same order in every stretch, n_rows a multiple of rows_per_stretch) and the keys of one stretch must be
+ * distinct; the shares are summed in fp32 together with the value already there and rounded once.  q, k, v, dout, lse as
+ * for splat_attention_bwd; delta as splat_attention_bwd wrote it for the same inputs (earlier on the same stream); plan_t
+ * is splat_attention_plan(segs_t, n_seg_t, n_rows). */
 int splat_attention_bwd_keys(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sl, const void* k, int64_t k_sb,
                              int64_t k_sh, int64_t k_sl, const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sl,
                              const void* dout, int64_t g_sb, int64_t g_sh, int64_t g_sl, const float* lse,
                              const float* delta, const int32_t* key_of_row, void* dk_rows, void* dv_rows,
                              const splat_acsr_seg* segs_t /* host */, int32_t n_seg_t, const void* plan_t,
                              int64_t plan_t_bytes, int32_t B, int32_t H, int32_t L, int32_t n_rows, int32_t d, float scale,
-                             int32_t dtype, void* stream);
+                             int32_t dtype, void* dk, void* dv, int32_t rows_per_stretch, void* stream);
 
 #ifdef __cplusplus
 }

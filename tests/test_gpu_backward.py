@@ -179,7 +179,7 @@ def _even_rows_far_field(L, local, stride):
 def test_fused_backward_with_sparse_rows_of_the_transposed_mask_listed(dev, name, make, dense, B, H, L, d, dtype):
     """Segments of the transposed mask that keep few keys with long columns (a strided pattern's far field), taken row by
     row through splat_attention_bwd_keys: against the oracle's dense gradients, and within an ulp or two of the plain walk
-    of 128 consecutive keys (the listed keys' shares pass through one more rounding)."""
+    of 128 consecutive keys (a listed key's shares, one per stretch of queries, are rounded to the 16-bit type before they are added)."""
     from r_backward import keys_side_schedule
     scale = d ** -0.5
     q, k, v = O.make_inputs(11 * L + d, B, H, L, d, dtype)
@@ -218,10 +218,12 @@ def test_keys_side_schedule_lists_every_entry_of_the_sparse_rows_once(dev):
     key_of_row = sched.key_of_row.cpu().numpy()
     seen = np.zeros_like(far_t, dtype=np.int64)
     for r in range(sched.n_rows):
+        if r % sched.per_stretch >= sched.keys.numel():
+            assert nnz[r] == 0 and key_of_row[r] == -1
+            continue
+        assert key_of_row[r] == key_of_row[r % sched.per_stretch]     # the same keys in the same order in every stretch
         cols = fcol[r] + lin[r].astype(np.int64) * np.arange(nnz[r])
         seen[key_of_row[r], cols] += 1
-        if r % sched.per_stretch >= sched.keys.numel():
-            assert nnz[r] == 0
     assert np.array_equal(seen, far_t.astype(np.int64))
     assert sorted(sched.keys.cpu().tolist()) == sorted(np.nonzero(far_t.sum(1))[0].tolist())
     # config 3's shape takes the schedule by itself; a causal window has nothing to list
@@ -267,19 +269,24 @@ def test_keys_entry_point_checks_its_arguments(dev):
     part = torch.zeros(2, B, H, R, d, device=dev, dtype=torch.float16)
     plan = sched.rows.plan(R, dev)
 
+    grads = torch.zeros(2, B, H, L, d, device=dev, dtype=torch.float16)
+
     def call(**kw):
         a = dict(q=t.data_ptr(), k=t.data_ptr(), keys=sched.key_of_row.data_ptr(), plan_bytes=plan.numel(), n_rows=R, d=d,
-                 scale=0.125, sl=d)
+                 scale=0.125, sl=d, dk=grads[0].data_ptr(), dv=grads[1].data_ptr(), rps=sched.per_stretch)
         a.update(kw)
         rows = lambda ptr: [ptr, H * L * d, L * d, a["sl"]]
         return hip.lib().splat_attention_bwd_keys(*rows(a["q"]), *rows(a["k"]), *rows(t.data_ptr()), *rows(t.data_ptr()),
                                                   stat.data_ptr(), stat.data_ptr(), a["keys"], part[0].data_ptr(), part[1].data_ptr(),
                                                   sched.rows.seg_array(R), 1, plan.data_ptr(), a["plan_bytes"], B, H, L, a["n_rows"],
-                                                  a["d"], a["scale"], hip.dtype_code(torch.float16), hip.stream_ptr(dev))
+                                                  a["d"], a["scale"], hip.dtype_code(torch.float16), a["dk"], a["dv"], a["rps"],
+                                                  hip.stream_ptr(dev))
     assert call() == 0
+    assert call(dk=None, dv=None, rps=0) == 0      # the rows' shares only
     for kw, what in [(dict(q=None), "null"), (dict(keys=None), "null"), (dict(n_rows=0), "n_rows"), (dict(d=96), "head dim"),
                      (dict(scale=0.0), "scale"), (dict(plan_bytes=plan.numel() - 16), "plan"), (dict(q=t.data_ptr() + 2), "aligned"),
-                     (dict(sl=d - 8), "row strides")]:
+                     (dict(sl=d - 8), "row strides"), (dict(dv=None), "dk and dv"), (dict(rps=R - 1), "rows_per_stretch"),
+                     (dict(rps=0), "rows_per_stretch"), (dict(dk=grads[0].data_ptr() + 2), "dk and dv")]:
         assert call(**kw) != 0, kw
         msg = hip.lib().splat_last_error().decode()
         assert what in msg, (kw, msg)

@@ -79,7 +79,8 @@ _SIGNATURES = {
     "splat_attention_bwd": (ctypes.c_int, [_vp, _i64, _i64, _i64] * 5 + [_vp] * 5 +
                             [ctypes.POINTER(AcsrSeg), _i32, _vp, _i64] * 2 + [_i32, _i32, _i32, _i32, _f32, _i32, _vp]),
     "splat_attention_bwd_keys": (ctypes.c_int, [_vp, _i64, _i64, _i64] * 4 + [_vp] * 5 +
-                                 [ctypes.POINTER(AcsrSeg), _i32, _vp, _i64] + [_i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp]),
+                                 [ctypes.POINTER(AcsrSeg), _i32, _vp, _i64] + [_i32, _i32, _i32, _i32, _i32, _f32, _i32] +
+                                 [_vp, _vp, _i32, _vp]),
 }
 EXPORTS = tuple(_SIGNATURES)
 

@@ -206,8 +206,8 @@ class KeysSideSchedule:
     column of queries: ``main`` holds the other segments (walked by 128 consecutive keys as usual), and the live rows of the
     sparse segments are listed one per (key, stretch of queries): ``rows`` is their single-segment ACSR (``n_rows`` rows;
     stretch c owns rows [c * per_stretch, (c + 1) * per_stretch), the keys in the same order in every stretch),
-    ``key_of_row`` the key each row belongs to (int32, 0 for padding rows, which are empty) and ``keys`` the
-    listed keys (int64, ``len(keys) <= per_stretch``)."""
+    ``key_of_row`` the key each row belongs to (int32, -1 for padding rows, which are empty) and ``keys`` the
+    listed keys (int64, distinct, ``len(keys) <= per_stretch``)."""
 
     def __init__(self, main: ACSRSegments, rows: ACSRSegments, key_of_row: torch.Tensor, keys: torch.Tensor,
                  n_stretches: int, per_stretch: int):
@@ -228,7 +228,7 @@ _WORTH_TILES = 40
 def keys_side_schedule(segments_t: ACSRSegments, L: int, device, batch_heads: int,
                        always: bool = False) -> KeysSideSchedule | None:
     """The ``KeysSideSchedule`` of a transposed mask, or None when no segment of it is row-sparse (or all are, or a
-    sparse one lacks its rows' first columns), or when the walk it replaces is too short for the extra launch to pay
+    sparse one lacks its rows' first columns, or two of them keep the same key), or when the walk it replaces is too short for the extra launch to pay
     (unless ``always``).  A block of 128 consecutive keys of a strided pattern's far field holds
     one live key with up to L queries: its workgroup walks up to L / 64 tiles for one row in 128, and the pass takes 5 x
     what the rest of the mask needs.  Listed row by row and cut into stretches of queries, the same entries fill a few
@@ -252,7 +252,7 @@ def keys_side_schedule(segments_t: ACSRSegments, L: int, device, batch_heads: in
             first.append(fc[live].to(torch.int64))
             step.append(torch.where(n > 1, t[2][live].to(torch.int64), torch.ones_like(n)).clamp(min=1))
             cnt.append(n)
-        if not sparse or len(sparse) == len(segments_t):
+        if not sparse or len(sparse) == len(segments_t) or torch.cat(key).unique().numel() != sum(x.numel() for x in key):
             facts = False
         else:
             first, step, cnt, key = (torch.cat(x) for x in (first, step, cnt, key))
@@ -297,7 +297,7 @@ def keys_side_schedule(segments_t: ACSRSegments, L: int, device, batch_heads: in
                         [fcol])
     main = ACSRSegments([t for i, t in enumerate(segments_t.tuples) if i not in sparse],
                         [c for i, c in enumerate(segments_t.first_cols) if i not in sparse])
-    key_of_row = padded(key[None, :].expand(n_stretches, n_keys), 0, torch.int32)
+    key_of_row = padded(key[None, :].expand(n_stretches, n_keys), -1, torch.int32)
     sched = KeysSideSchedule(main, rows, key_of_row, key.contiguous(), n_stretches, per_stretch)
     sched.main.plan(L, dev)
     sched.rows.plan(sched.n_rows, dev)
@@ -335,8 +335,7 @@ def attention_backward_fused(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor,
         raise _hip.SplatError(f"lse must be a contiguous float32 tensor of shape {(B, H, L)}")
     delta = torch.empty((B, H, L), dtype=torch.float32, device=dev)
     dq = torch.empty((B, H, L, d), dtype=dt, device=dev)
-    dkv = torch.empty((2, B, H, L, d), dtype=dt, device=dev)
-    dk, dv = dkv[0], dkv[1]
+    dk, dv = (torch.empty((B, H, L, d), dtype=dt, device=dev) for _ in range(2))
     sched = None if sparse_rows is False else keys_side_schedule(segments_t, L, dev, B * H, always=bool(sparse_rows))
     if sched is not None:  # the row-sparse segments of the transposed mask go row by row, after the others
         segments_t, plan_t = sched.main, sched.main.plan(L, dev)
@@ -361,14 +360,10 @@ def attention_backward_fused(q: torch.Tensor, kT: torch.Tensor, v: torch.Tensor,
             part = torch.empty((2, B, H, R, d), dtype=dt, device=dev)
             plan_r = sched.rows.plan(R, dev)
             args = strides3(q, k, v, grad_out)
+            # (the call's second kernel adds a key's shares, one per stretch, onto what the other segments gave it)
             args += [lse.data_ptr(), delta.data_ptr(), sched.key_of_row.data_ptr(), part[0].data_ptr(), part[1].data_ptr(),
                      sched.rows.seg_array(R), 1, plan_r.data_ptr(), plan_r.numel() * plan_r.element_size(),
-                     B, H, L, R, d, float(scale), _hip.dtype_code(dt)]
+                     B, H, L, R, d, float(scale), _hip.dtype_code(dt), dk.data_ptr(), dv.data_ptr(), sched.per_stretch]
             rc = _hip.lib().splat_attention_bwd_keys(*args, _hip.stream_ptr(dev))
             _hip.check(rc, "splat_attention_bwd_keys")
-            # a key's shares (one per stretch) added up (the reduction accumulates in fp32 and rounds once), then onto what
-            # the other segments gave it
-            n_keys = sched.keys.numel()
-            share = part.view(2, B, H, sched.n_stretches, sched.per_stretch, d)[:, :, :, :, :n_keys].sum(3)
-            dkv.index_add_(3, sched.keys, share)
     return dq, dk, dv

@@ -588,6 +588,59 @@ static int launch_bwd(BwdParams p, hipStream_t st) {
     return check_launch("splat_attention_bwd");
 }
 
+// Adds the shares of listed rows onto the gradients of their keys: row k of every stretch (rows k + rps * s of the share
+// buffers, [B*H, n_rows, D]) belongs to key key_of_row[k] (negative: padding).  One thread takes 8 features of one listed
+// key of one (b, h) and one gradient (blockIdx.y: dk, dv), eight stretches' shares requested at a time, summing in fp32
+// and rounding once.
+template <typename T, int D>
+__global__ __launch_bounds__(256) void bwd_rows_add_kernel(const T* __restrict__ dk_rows, const T* __restrict__ dv_rows, T* dk, T* dv,
+                                                           const int* __restrict__ key_of_row, int n_rows, int rps, int L, int64_t total) {
+    constexpr int CPR = D / 8;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int c = (int)(idx % CPR);
+    const int64_t r = idx / CPR;
+    const int k = (int)(r % rps);
+    const int64_t bh = r / rps;
+    const int key = key_of_row[k];
+    if (key < 0 || key >= L) return;
+    const int n_stretches = n_rows / rps;
+    const T* rows = (blockIdx.y ? dv_rows : dk_rows) + ((int64_t)bh * n_rows + k) * D + 8 * c;
+    T* out = (blockIdx.y ? dv : dk) + ((int64_t)bh * L + key) * D + 8 * c;
+    Frag<T> cur = global_frag<T>(out);
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = (float)cur.v[e];
+    for (int st = 0; st < n_stretches; st += 8) {
+        Frag<T> f[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) f[u] = global_frag<T>(rows + (int64_t)min(st + u, n_stretches - 1) * rps * D);  // (unconditional)
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const float w = st + u < n_stretches ? 1.f : 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] = fmaf(w, (float)f[u].v[e], acc[e]);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) cur.v[e] = (T)acc[e];
+    *reinterpret_cast<typename Frag<T>::vec*>(out) = cur.v;
+}
+
+template <typename T>
+static int launch_rows_add(const void* dk_rows, const void* dv_rows, void* dk, void* dv, const int* key_of_row, int B, int H, int L,
+                           int n_rows, int rps, int d, hipStream_t st) {
+    begin_launch();
+    const int64_t total = (int64_t)B * H * rps * (d / 8);
+    const int64_t blocks = (total + 255) / 256;
+    if (blocks > 0x7ffffff0) return fail(SPLAT_E_SHAPE, "splat_attention_bwd_keys: too many listed rows");
+    if (d == 64)
+        bwd_rows_add_kernel<T, 64><<<dim3((unsigned)blocks, 2), 256, 0, st>>>((const T*)dk_rows, (const T*)dv_rows, (T*)dk, (T*)dv, key_of_row, n_rows, rps, L, total);
+    else
+        bwd_rows_add_kernel<T, 128><<<dim3((unsigned)blocks, 2), 256, 0, st>>>((const T*)dk_rows, (const T*)dv_rows, (T*)dk, (T*)dv, key_of_row, n_rows, rps, L, total);
+    return check_launch("splat_attention_bwd_keys");
+}
+
 // The keys' side: dK and dV of the rows of the transposed mask that `dk` describes (dv: the same launch geometry).
 template <typename T>
 static int run_bwd_keys(const BwdParams& dk, const BwdParams& dv, int d, hipStream_t st) {
@@ -714,13 +767,20 @@ extern "C" int splat_attention_bwd_keys(const void* q, int64_t q_sb, int64_t q_s
                                         const float* delta, const int32_t* key_of_row, void* dk_rows, void* dv_rows,
                                         const splat_acsr_seg* segs_t, int32_t n_seg_t, const void* plan_t, int64_t plan_t_bytes,
                                         int32_t B, int32_t H, int32_t L, int32_t n_rows, int32_t d, float scale, int32_t dtype,
-                                        void* stream) {
+                                        void* dk, void* dv, int32_t rows_per_stretch, void* stream) {
     const char* who = "splat_attention_bwd_keys";
     if (!q || !k || !v || !dout || !lse || !delta || !key_of_row || !dk_rows || !dv_rows || !segs_t || !plan_t)
         return fail(SPLAT_E_NULL, "%s: null pointer argument", who);
     const Rows3 rq{q, q_sb, q_sh, q_sl}, rk{k, k_sb, k_sh, k_sl}, rv{v, v_sb, v_sh, v_sl}, rg{dout, g_sb, g_sh, g_sl};
     if (int rc = check_bwd_common(who, B, H, L, d, scale, dtype, {rq, rk, rv, rg}, {dk_rows, dv_rows, plan_t})) return rc;
     if (n_rows <= 0 || n_rows > (1 << 23)) return fail(SPLAT_E_SHAPE, "%s: need 0 < n_rows <= 2^23 (got %d)", who, n_rows);
+    if ((dk == nullptr) != (dv == nullptr)) return fail(SPLAT_E_NULL, "%s: dk and dv go together (both or neither)", who);
+    if (dk) {
+        if ((reinterpret_cast<uintptr_t>(dk) & 15) != 0 || (reinterpret_cast<uintptr_t>(dv) & 15) != 0)
+            return fail(SPLAT_E_ALIGN, "%s: dk and dv must be 16-byte aligned", who);
+        if (rows_per_stretch <= 0 || n_rows % rows_per_stretch != 0)
+            return fail(SPLAT_E_SHAPE, "%s: n_rows (%d) must be a multiple of rows_per_stretch (%d)", who, n_rows, rows_per_stretch);
+    }
     if ((reinterpret_cast<uintptr_t>(lse) & 3) != 0 || (reinterpret_cast<uintptr_t>(delta) & 3) != 0 ||
         (reinterpret_cast<uintptr_t>(key_of_row) & 3) != 0)
         return fail(SPLAT_E_ALIGN, "%s: lse, delta and key_of_row must be 4-byte aligned", who);
@@ -737,5 +797,8 @@ extern "C" int splat_attention_bwd_keys(const void* q, int64_t q_sb, int64_t q_s
     pv.b = nullptr;
     pv.out = dv_rows;
     hipStream_t st = (hipStream_t)stream;
-    return dtype == SPLAT_F16 ? run_bwd_keys<f16>(pk, pv, d, st) : run_bwd_keys<bf16>(pk, pv, d, st);
+    if (int rc = dtype == SPLAT_F16 ? run_bwd_keys<f16>(pk, pv, d, st) : run_bwd_keys<bf16>(pk, pv, d, st)) return rc;
+    if (!dk) return 0;
+    return dtype == SPLAT_F16 ? launch_rows_add<f16>(dk_rows, dv_rows, dk, dv, key_of_row, B, H, L, n_rows, rows_per_stretch, d, st)
+                              : launch_rows_add<bf16>(dk_rows, dv_rows, dk, dv, key_of_row, B, H, L, n_rows, rows_per_stretch, d, st);
 }
