@@ -487,3 +487,51 @@ def test_forward_and_backward_replay_from_a_captured_graph(dev, dtype, d):
         assert torch.equal(got_o, want_o) and torch.equal(got_lse, want_lse), seed
         for a, b_ in zip(got_g, want_g):
             assert torch.equal(a, b_), seed
+
+
+def test_backward_with_listed_rows_replays_from_a_captured_graph(dev):
+    """The same for a mask whose transposed far field is taken row by row (one more launch of the kernel and the kernel that
+    adds the listed keys' shares, the schedule built by an eager call beforehand): every replay equals the eager result; and
+    a capture that finds no schedule yet records the plain walk instead of building one."""
+    from r_backward import attention_backward_fused, keys_side_schedule, transposed_segments
+    B, H, L, d, dtype = 1, 2, 1100, 64, torch.bfloat16
+    scale = d ** -0.5
+    pats = A.strided_patterns(L, 48, 40)
+    attn = RegularAttention(B, L, H, d, pats, 16, 16, dev, dtype, scale=scale)
+    g = torch.Generator().manual_seed(12)
+    q, k, v, go = [torch.randn(B, H, L, d, generator=g).to(dtype).to(dev) for _ in range(4)]
+    x = [q, k.transpose(2, 3), v]
+    out, lse = attn.forward_with_stats(x)
+    attn.backward_pass(x, go, lse.clone(), out.clone(), sparse_rows=True)   # builds the transposed ACSR, the plans, the schedule
+    assert keys_side_schedule(attn._segments_t, L, dev, B * H, always=True) is not None
+    fresh_t = transposed_segments(pats, 16, dev)                             # no schedule attached to these yet
+    fresh_plan_t = fresh_t.plan(L, dev)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            o_g, lse_g = attn.forward_with_stats(x)
+            grads_g = attention_backward_fused(q, x[1], v, o_g, go, lse_g, attn.segments, attn._segments_t, attn._plan,
+                                               attn._plan_t, scale, sparse_rows=True)
+            plain_g = attention_backward_fused(q, x[1], v, o_g, go, lse_g, attn.segments, fresh_t, attn._plan,
+                                               fresh_plan_t, scale, sparse_rows=True)
+    torch.cuda.current_stream(dev).wait_stream(side)
+    assert not fresh_t.__dict__.get("_keys_side")                            # nothing was built under capture
+    for seed in (1, 2, 3):
+        gen = torch.Generator().manual_seed(seed)
+        for t in (q, k, v, go):
+            t.copy_(torch.randn(B, H, L, d, generator=gen).to(dtype))
+        graph.replay()
+        torch.cuda.synchronize()
+        got_g, got_plain = [t.clone() for t in grads_g], [t.clone() for t in plain_g]
+        want_o, want_lse = attn.forward_with_stats(x)
+        want_o, want_lse = want_o.clone(), want_lse.clone()
+        want_g = [t.clone() for t in attn.backward_pass(x, go, want_lse, want_o, sparse_rows=True)]
+        want_plain = attn.backward_pass(x, go, want_lse, want_o, sparse_rows=False)
+        torch.cuda.synchronize()
+        for a, b_ in zip(got_g, want_g):
+            assert torch.equal(a, b_), seed
+        for a, b_ in zip(got_plain, want_plain):
+            assert torch.equal(a, b_), seed
